@@ -1,0 +1,90 @@
+/*
+ * ckq_oracle.h - CPU oracle for the quantized dequant-dot matmul path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This is a plain-C restatement of the reference
+ * engine's CPU arithmetic for the Q4_K/Q5_K/Q6_K/Q8_0 x Q8_K/Q8_0 kernels and
+ * the fp32->Q8_K / fp32->Q8_0 activation quantizers.  Only the test-suite,
+ * the smoke check and the CPU-baseline leg of the benchmark may link or load
+ * it; the GPU library never does.
+ *
+ * Every function names the reference file:line it follows (paths relative to
+ * the reference checkout).
+ */
+#ifndef CKQ_ORACLE_H
+#define CKQ_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- scalar helpers ---------------------------------------------------- */
+float    orc_fp16_to_fp32(uint16_t h);          /* include/ckernel_quant.h:265-294 */
+uint16_t orc_fp32_to_fp16(float f);             /* include/ckernel_quant.h:311-336,355-357 (RNE) */
+void     orc_unpack_scales_k4(const uint8_t *s12, uint8_t *sc8, uint8_t *m8);      /* ckernel_quant.h:227-251 */
+void     orc_unpack_scales_k4_kmask(const uint8_t *s12, uint8_t *sc8, uint8_t *m8); /* gemm_kernels_q5_k.c:163-170 */
+
+/* ---- activation quantizers (bit-exact contract) ------------------------ */
+void orc_quantize_row_q8_k(const float *x, void *y, int k);                 /* quantize_row_q8_k_sse.c:22-82 */
+void orc_quantize_batch_q8_k(const float *x, void *y, int rows, int k);     /* gemm_kernels_q8_0.c:221-239 */
+void orc_quantize_row_q8_0(const float *x, void *y, int k);                 /* gemm_kernels_q8_0.c:70-146 */
+void orc_quantize_batch_q8_0(const float *x, void *y, int rows, int k);     /* gemm_kernels_q8_0.c:194-209 */
+
+/* ---- dequantizers (fp32 cross-check reference) ------------------------- */
+void orc_dequant_q4_k_row(const void *src, float *dst, size_t n);           /* dequant_kernels.c:336-385 */
+void orc_dequant_q5_k_row(const void *src, float *dst, size_t n);           /* gemm_kernels_q5_k.c:130-208 (layout) */
+void orc_dequant_q6_k_row(const void *src, float *dst, size_t n);           /* dequant_kernels.c:396-430 */
+void orc_dequant_q8_0_row(const void *src, float *dst, size_t n);           /* dequant_kernels.c:276-296 */
+void orc_dequant_q8_k_row(const void *src, float *dst, size_t n);           /* d * qs; block layout ckernel_quant.h:153-157 */
+
+/* ---- integer sub-block dots (bit-exact contract) ----------------------- *
+ * One weight row against one activation vector.  Output counts per
+ * super-block: Q4_K/Q5_K 8 (sum over 32 of q*q8), Q6_K 16 (sum over 16 of
+ * (q-32)*q8), Q8_0 1 per 32-block.                                         */
+void orc_subdots_q4_k_q8_k(const void *w_row, const void *x_q8, int K, int32_t *out);
+void orc_subdots_q5_k_q8_k(const void *w_row, const void *x_q8, int K, int32_t *out);
+void orc_subdots_q6_k_q8_k(const void *w_row, const void *x_q8, int K, int32_t *out);
+void orc_subdots_q8_0_q8_0(const void *w_row, const void *x_q8, int K, int32_t *out);
+
+/* ---- GEMV: y[M] = W[M x K] . x ----------------------------------------- */
+void orc_gemv_q4_k_q8_k(float *y, const void *W, const void *x_q8, int M, int K);      /* gemm_kernels_q4k_q8k.c:121-200 */
+void orc_gemv_q4_k_q8_k_parallel(float *y, const void *W, const void *x_q8, int M, int K, int ith, int nth); /* :212-243 */
+void orc_gemv_q5_k_q8_k(float *y, const void *W, const void *x_q8, int M, int K);      /* gemm_kernels_q5_k.c:130-208,305-329 */
+void orc_gemv_q5_k(float *y, const void *W, const float *x, int M, int K);             /* gemm_kernels_q5_k.c:369-391 (K%256==0 branch) */
+void orc_gemv_q6_k_q8_k_ref(float *y, const void *W, const void *x_q8, int M, int K);  /* gemm_kernels_q6k_q8k.c:70-120,197-214 */
+void orc_gemv_q6_k_q8_k(float *y, const void *W, const void *x_q8, int M, int K);      /* gemm_kernels_q6k_q8k.c:601-695 (integer block form, 8 float lanes) */
+void orc_gemv_q6_k_q8_k_parallel(float *y, const void *W, const void *x_q8, int M, int K, int ith, int nth); /* :1141-1197 */
+void orc_vec_dot_q6_k_q8_k(int n, float *s, const void *vx, const void *vy);           /* gemm_kernels_q6k_q8k.c:1032-1055 */
+void orc_gemv_q8_0_q8_0(float *y, const void *W, const void *x_q8, int M, int K);      /* gemm_kernels_q8_0.c:968-989,1237-1251 */
+void orc_gemv_q8_0_q8_0_lanes8(float *y, const void *W, const void *x_q8, int M, int K); /* gemm_kernels_q8_0.c:845-889,1031-1058 (AVX2 order) */
+void orc_gemv_q8_0_q8_0_parallel(float *y, const void *W, const void *x_q8, int M, int K, int ith, int nth); /* :1263-1287 */
+void orc_vec_dot_q8_0_q8_0(int n, float *s, const void *vx, const void *vy);           /* gemm_kernels_q8_0.c:968-989 */
+void orc_gemv_q8_0(float *y, const void *W, const float *x, int M, int K);             /* gemm_kernels_q8_0.c:254-277 */
+
+/* ---- GEMM ---------------------------------------------------------------
+ * gemm_*   : Y[n*M + row], M = output rows, N = tokens.
+ * gemm_nt_*: C[m*N + n],   M = tokens,      N = output rows, optional bias[N]. */
+void orc_gemm_q4_k_q8_k(float *Y, const void *W, const void *X_q8, int M, int N, int K);                        /* gemm_kernels_q4k_q8k.c:283-299 */
+void orc_gemm_nt_q4_k_q8_k(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K);  /* :301-326 */
+void orc_gemm_nt_q5_k_q8_k(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K);  /* gemm_kernels_q5_k.c:331-359 */
+void orc_gemm_nt_q5_k(const float *A, const void *B, const float *bias, float *C, int M, int N, int K);         /* gemm_kernels_q5_k.c:401-430 */
+void orc_gemm_q6_k_q8_k(float *Y, const void *W, const void *X_q8, int M, int N, int K);                        /* gemm_kernels_q6k_q8k.c:1209-1225 */
+void orc_gemm_nt_q6_k_q8_k(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K);  /* :1243-1268 */
+void orc_gemm_nt_q8_0_q8_0(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K);  /* gemm_batch_int8.c:87-120,582-610 */
+
+/* ---- exact evaluation ---------------------------------------------------
+ * Same integers, block scales combined in double: the value every fp32
+ * summation order approximates.  fmt is a ckq_format weight tag; the
+ * activation format is Q8_0 for CKQ_FMT_Q8_0 weights and Q8_K otherwise.   */
+void orc_gemv_exact_f64(int fmt, double *y, const void *W, const void *x_q8, int M, int K);
+
+/* Row-split multi-threaded GEMV used by the CPU-baseline timing: rows
+ * [ith*ceil(M/nth), ...) per thread as in gemm_kernels_q4k_q8k.c:226-231.  */
+void orc_gemv_threads(int fmt, float *y, const void *W, const void *x_q8, int M, int K, int nth);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

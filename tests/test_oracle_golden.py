@@ -1,0 +1,302 @@
+"""Pins the CPU oracle: golden vectors written from the compiled reference C
+(tests/golden/make_golden.py), hand-computed known answers, closed forms and
+brute force.  Runs on CPU."""
+import ctypes
+
+import numpy as np
+import pytest
+
+import ckq_testlib as T
+from ckq_testlib import ptr
+
+FLOAT_TOL = 2e-6  # normalised; fp32 summation order differs at the ulp level between builds
+
+
+# ---- fp16 -------------------------------------------------------------------
+
+def test_fp16_to_fp32_exhaustive():
+    O = T.oracle()
+    allh = np.arange(65536, dtype=np.uint16)
+    want = allh.view(np.float16).astype(np.float32)
+    got = np.array([O.orc_fp16_to_fp32(int(h)) for h in allh], dtype=np.float32)
+    same = (got.view(np.uint32) == want.view(np.uint32)) | (np.isnan(got) & np.isnan(want))
+    assert same.all()
+
+
+def test_fp32_to_fp16_rne():
+    O = T.oracle()
+    rng = np.random.default_rng(5)
+    xs = np.concatenate([rng.standard_normal(4000).astype(np.float32) * s
+                         for s in (1e-8, 1e-7, 1e-5, 1e-3, 1.0, 100.0, 3e4, 7e4)])
+    # exact ties between neighbouring halves, subnormal boundary, overflow edge
+    xs = np.concatenate([xs, np.array([1.0 + 2 ** -11, 1.0 + 3 * 2 ** -11, 2 ** -24, 2 ** -25, 3 * 2 ** -25,
+                                       65504.0, 65519.0, 65520.0, 6.1e-5, 0.0, -0.0], np.float32)])
+    with np.errstate(over="ignore"):
+        want = xs.astype(np.float16).view(np.uint16)
+    got = np.array([O.orc_fp32_to_fp16(float(x)) for x in xs], dtype=np.uint16)
+    assert np.array_equal(got, want)
+
+
+# ---- 6-bit scale unpack -----------------------------------------------------
+
+# the five byte patterns of the reference's unittest/test_dequant_vs_llamacpp.c:293-300
+# with scales/mins worked out by hand from the GGUF get_scale_min_k4 rule
+SCALE_KAT = [
+    ([236, 243, 254, 184, 172, 230, 235, 185, 123, 7, 255, 201],
+     [44, 51, 62, 56, 59, 55, 63, 41], [44, 38, 43, 57, 39, 48, 63, 44]),
+    ([0] * 12, [0] * 8, [0] * 8),
+    ([255] * 12, [63] * 8, [63] * 8),
+    ([0xC0] * 8 + [0] * 4, [0, 0, 0, 0, 48, 48, 48, 48], [0, 0, 0, 0, 48, 48, 48, 48]),
+    ([0x3F] * 8 + [0xFF] * 4, [63, 63, 63, 63, 15, 15, 15, 15], [63, 63, 63, 63, 15, 15, 15, 15]),
+]
+
+
+@pytest.mark.parametrize("packed,sc_want,m_want", SCALE_KAT)
+def test_scale_unpack_known_answers(packed, sc_want, m_want):
+    O = T.oracle()
+    s = np.array(packed, np.uint8)
+    for fn in (O.orc_unpack_scales_k4, O.orc_unpack_scales_k4_kmask):
+        sc = np.zeros(8, np.uint8)
+        m = np.zeros(8, np.uint8)
+        fn(ptr(s), ptr(sc), ptr(m))
+        assert sc.tolist() == sc_want and m.tolist() == m_want
+
+
+def test_scale_unpack_byte_and_word_forms_agree():
+    O = T.oracle()
+    rng = np.random.default_rng(11)
+    for _ in range(2000):
+        s = rng.integers(0, 256, 12, dtype=np.uint8)
+        a, b, c, d = (np.zeros(8, np.uint8) for _ in range(4))
+        O.orc_unpack_scales_k4(ptr(s), ptr(a), ptr(b))
+        O.orc_unpack_scales_k4_kmask(ptr(s), ptr(c), ptr(d))
+        assert np.array_equal(a, c) and np.array_equal(b, d)
+
+
+# ---- dequantizers -------------------------------------------------------------
+
+def test_q4_k_closed_form_block():
+    """d=1.0, dmin=0.5, scales 2, mins 1 (sub-blocks 0-3) / 2 (4-7), every byte
+    0x84: the block of the reference's test_dequant_vs_llamacpp.c:331-375."""
+    blk = np.zeros(144, np.uint8)
+    blk[0:2] = np.array([0x3C00], np.uint16).view(np.uint8)
+    blk[2:4] = np.array([0x3800], np.uint16).view(np.uint8)
+    blk[4:8] = 2
+    blk[8:12] = 1
+    blk[12:16] = 0x22
+    blk[16:] = 0x84
+    out = np.zeros(256, np.float32)
+    T.oracle().orc_dequant_q4_k_row(ptr(blk), ptr(out), ctypes.c_size_t(256))
+    want = np.zeros(256, np.float32)
+    for g in range(4):
+        lo, hi = (7.5, 15.5) if g < 2 else (7.0, 15.0)
+        want[64 * g:64 * g + 32] = lo
+        want[64 * g + 32:64 * g + 64] = hi
+    assert np.array_equal(out, want)
+
+
+@pytest.mark.parametrize("fmt", ["q4_k", "q6_k", "q8_0"])
+def test_dequant_matches_reference_golden(fmt):
+    G = T.golden()
+    w = G["deq_%s_w" % fmt]
+    want = G["deq_%s_out" % fmt]
+    out = np.zeros_like(want)
+    getattr(T.oracle(), "orc_dequant_%s_row" % fmt)(ptr(w), ptr(out), ctypes.c_size_t(len(want)))
+    assert np.array_equal(out.view(np.uint32), want.view(np.uint32))
+    # the NumPy decoders used by the brute-force checks read the same layout
+    assert np.allclose(T.np_dequant(fmt, w), want.astype(np.float64), rtol=1e-6, atol=1e-9)
+
+
+def test_q5_k_fifth_bit_plane():
+    """One block with a single set bit in qh: exactly one element gains 16."""
+    for g in range(4):
+        for half in range(2):
+            for l in (0, 13, 31):
+                blk = np.zeros(176, np.uint8)
+                blk[0:2] = np.array([0x3C00], np.uint16).view(np.uint8)  # d = 1
+                blk[4:8] = 1
+                blk[12:16] = 0x01  # scales 4..7 = 1, mins 0
+                blk[16 + l] = 1 << (2 * g + half)
+                out = np.zeros(256, np.float32)
+                T.oracle().orc_dequant_q5_k_row(ptr(blk), ptr(out), ctypes.c_size_t(256))
+                want = np.zeros(256, np.float32)
+                want[64 * g + 32 * half + l] = 16.0
+                assert np.array_equal(out, want), (g, half, l)
+                assert np.array_equal(T.np_dequant("q5_k", blk).astype(np.float32), want)
+
+
+# ---- activation quantizers (bit-exact) -----------------------------------------
+
+def test_quantize_q8_k_bit_exact_vs_reference():
+    G = T.golden()
+    x, want = G["q8k_in"], G["q8k_out"]
+    got = T.oracle_quantize(x, "q8_k")
+    assert np.array_equal(got, want)
+
+
+def test_quantize_q8_k_invariants():
+    x = T.normal(64 * 256, 0.0, 2.0, seed=77)
+    b = T.np_decode_q8_k(T.oracle_quantize(x, "q8_k"))
+    q = b["q"]
+    assert np.array_equal(q.reshape(-1, 16, 16).sum(axis=2), b["bsums"])
+    xb = x.reshape(-1, 256)
+    arg = np.argmax(np.abs(xb), axis=1)
+    assert np.all(q[np.arange(len(arg)), arg] == -127)
+    assert np.allclose(b["d"] * -127.0, xb[np.arange(len(arg)), arg], rtol=1e-6)
+    # round trip within half a step
+    assert np.max(np.abs(b["d"][:, None] * q - xb) / np.abs(b["d"][:, None])) <= 0.5 + 1e-3
+
+
+def test_quantize_batch_equals_row_loop():
+    x = T.normal(5 * 768, seed=9)
+    whole = T.oracle_quantize(x, "q8_k", rows=5)
+    rows = np.concatenate([T.oracle_quantize(x[r * 768:(r + 1) * 768], "q8_k") for r in range(5)])
+    assert np.array_equal(whole, rows)
+    whole = T.oracle_quantize(x, "q8_0", rows=5)
+    rows = np.concatenate([T.oracle_quantize(x[r * 768:(r + 1) * 768], "q8_0") for r in range(5)])
+    assert np.array_equal(whole, rows)
+
+
+def test_quantize_q8_0_bit_exact_vs_reference():
+    G = T.golden()
+    got = T.oracle_quantize(G["q80_in"], "q8_0")
+    assert np.array_equal(got, G["q80_out"])
+
+
+# ---- integer sub-block dots ------------------------------------------------------
+
+@pytest.mark.parametrize("fmt", ["q4_k", "q5_k", "q6_k", "q8_0"])
+@pytest.mark.parametrize("kind", ["rand", "enc"])
+def test_subdots_brute_force(fmt, kind):
+    G = T.golden()
+    M, K, _ = (int(v) for v in G["shape"])
+    W = G["w_%s_%s" % (fmt, kind)]
+    xq = G["act_q80" if fmt == "q8_0" else "act_q8k"][:T.row_bytes(T.act_fmt(fmt), K)].copy()
+    assert np.array_equal(T.oracle_subdots(fmt, W, xq, M, K), T.np_subdots(fmt, W, xq, M, K))
+
+
+# ---- GEMV / GEMM against the reference builds ------------------------------------
+
+@pytest.mark.parametrize("fmt", ["q4_k", "q5_k", "q6_k", "q8_0"])
+@pytest.mark.parametrize("kind", ["rand", "enc"])
+@pytest.mark.parametrize("build", ["avx2", "avx512"])
+def test_gemv_matches_reference(fmt, kind, build):
+    G = T.golden()
+    M, K, _ = (int(v) for v in G["shape"])
+    W = G["w_%s_%s" % (fmt, kind)]
+    xq = G["act_q80" if fmt == "q8_0" else "act_q8k"]
+    y = T.oracle_gemv(fmt, W, xq, M, K)
+    assert T.norm_err(y, G["y_%s_%s_%s" % (fmt, kind, build)]) <= FLOAT_TOL
+
+
+@pytest.mark.parametrize("fmt", ["q4_k", "q5_k", "q6_k", "q8_0"])
+@pytest.mark.parametrize("kind", ["rand", "enc"])
+def test_gemm_nt_with_bias_matches_reference(fmt, kind):
+    G = T.golden()
+    N, K, M = (int(v) for v in G["shape"])
+    W = G["w_%s_%s" % (fmt, kind)]
+    A = G["act_q80" if fmt == "q8_0" else "act_q8k"]
+    c = T.oracle_gemm_nt(fmt, A, W, G["bias"], M, N, K)
+    assert T.norm_err(c, G["c_%s_%s_avx2" % (fmt, kind)]) <= FLOAT_TOL
+    # token 0 without bias is the GEMV
+    c0 = T.oracle_gemm_nt(fmt, A, W, None, 1, N, K)
+    y = T.oracle_gemv(fmt, W, A, N, K)
+    assert T.norm_err(c0, y) <= FLOAT_TOL
+
+
+@pytest.mark.parametrize("kind", ["rand", "enc"])
+def test_variants_match_reference(kind):
+    G = T.golden()
+    M, K, TOK = (int(v) for v in G["shape"])
+    O = T.oracle()
+    xq, xf = G["act_q8k"], G["act_f32"]
+    # Q4_K scalar reference, and stored-bsums semantics (zeroed bsums)
+    W = G["w_q4_k_" + kind]
+    assert T.norm_err(T.oracle_gemv("q4_k", W, xq, M, K), G["y_q4_k_%s_ref" % kind]) <= FLOAT_TOL
+    y = T.oracle_gemv("q4_k", W, G["act_q8k_zero_bsums"], M, K)
+    assert T.norm_err(y, G["y_q4_k_%s_zero_bsums" % kind]) <= FLOAT_TOL
+    assert T.norm_err(y, G["y_q4_k_%s_avx2" % kind]) > 1e-3  # the min term really is gone
+    # row-split union equals serial
+    yp = np.zeros(M, np.float32)
+    for ith in range(5):
+        O.orc_gemv_q4_k_q8_k_parallel(ptr(yp), ptr(W), ptr(xq), M, K, ith, 5)
+    assert np.array_equal(yp, T.oracle_gemv("q4_k", W, xq, M, K))
+    assert T.norm_err(yp, G["y_q4_k_%s_parallel5" % kind]) <= FLOAT_TOL
+    # Q5_K: zero bsums, fp32 adapter
+    W = G["w_q5_k_" + kind]
+    y = T.oracle_gemv("q5_k", W, G["act_q8k_zero_bsums"], M, K)
+    assert T.norm_err(y, G["y_q5_k_%s_zero_bsums" % kind]) <= FLOAT_TOL
+    y = np.zeros(M, np.float32)
+    O.orc_gemv_q5_k(ptr(y), ptr(W), ptr(xf), M, K)
+    assert T.norm_err(y, G["y_q5_k_%s_f32act" % kind]) <= FLOAT_TOL
+    c = np.zeros(TOK * M, np.float32)
+    O.orc_gemm_nt_q5_k(ptr(xf), ptr(W), ptr(G["bias"]), ptr(c), TOK, M, K)
+    assert T.norm_err(c, G["c_q5_k_%s_f32act" % kind]) <= FLOAT_TOL
+    # Q6_K: element-wise scalar form, bsums are not read, vec_dot
+    W = G["w_q6_k_" + kind]
+    assert T.norm_err(T.oracle_gemv("q6_k", W, xq, M, K, "orc_gemv_q6_k_q8_k_ref"),
+                      G["y_q6_k_%s_ref" % kind]) <= 1e-5
+    y = T.oracle_gemv("q6_k", W, G["act_q8k_zero_bsums"], M, K)
+    assert np.array_equal(y, T.oracle_gemv("q6_k", W, xq, M, K))
+    assert T.norm_err(y, G["y_q6_k_%s_zero_bsums" % kind]) <= FLOAT_TOL
+    s = np.zeros(1, np.float32)
+    O.orc_vec_dot_q6_k_q8_k(K, ptr(s), ptr(W), ptr(xq))
+    assert T.norm_err(s, G["s_q6_k_%s_vecdot" % kind]) <= FLOAT_TOL
+    # Q8_0: fp32 activations, vec_dot, AVX2 lane order
+    W = G["w_q8_0_" + kind]
+    y = np.zeros(M, np.float32)
+    O.orc_gemv_q8_0(ptr(y), ptr(W), ptr(xf), M, K)
+    assert T.norm_err(y, G["y_q8_0_%s_f32act" % kind]) <= 1e-5
+    s = np.zeros(1, np.float32)
+    O.orc_vec_dot_q8_0_q8_0(K, ptr(s), ptr(W), ptr(G["act_q80"]))
+    assert T.norm_err(s, G["s_q8_0_%s_vecdot" % kind]) <= FLOAT_TOL
+
+
+@pytest.mark.parametrize("kind", ["rand", "enc"])
+def test_lane_order_variants_bit_identical_to_avx2_build(kind):
+    """The 8-lane restatements follow the AVX2 routines' summation order
+    exactly, so they reproduce that build's fp32 results bit for bit."""
+    G = T.golden()
+    M, K, _ = (int(v) for v in G["shape"])
+    y = T.oracle_gemv("q6_k", G["w_q6_k_" + kind], G["act_q8k"], M, K)
+    assert np.array_equal(y.view(np.uint32), G["y_q6_k_%s_avx2" % kind].view(np.uint32))
+    y = T.oracle_gemv("q8_0", G["w_q8_0_" + kind], G["act_q80"], M, K, "orc_gemv_q8_0_q8_0_lanes8")
+    assert np.array_equal(y.view(np.uint32), G["y_q8_0_%s_avx2" % kind].view(np.uint32))
+
+
+# ---- exact evaluation: dequantize-then-fp64 matmul ---------------------------------
+
+@pytest.mark.parametrize("fmt", ["q4_k", "q5_k", "q6_k", "q8_0"])
+@pytest.mark.parametrize("kind", ["rand", "enc"])
+def test_exact_equals_dequant_matmul(fmt, kind):
+    G = T.golden()
+    M, K, _ = (int(v) for v in G["shape"])
+    W = G["w_%s_%s" % (fmt, kind)]
+    af = T.act_fmt(fmt)
+    xq = G["act_q80" if fmt == "q8_0" else "act_q8k"][:T.row_bytes(af, K)].copy()
+    want = T.np_dequant(fmt, W).reshape(M, K) @ T.np_dequant(af, xq)
+    got = T.oracle_exact(fmt, W, xq, M, K)
+    assert T.norm_err(got, want) <= 1e-12
+    # and every fp32 kernel order approximates it
+    assert T.norm_err(T.oracle_gemv(fmt, W, xq, M, K), want) <= 1e-5
+
+
+def test_encoders_round_trip():
+    """The weight encoders emit format-valid blocks: dequant(quant(w)) is
+    within one quantisation step of w, and an all-zero row encodes to zeros."""
+    S = T.synth()
+    w = T.normal(16 * 256, 0.0, 0.02, seed=3)
+    for fmt, steps in (("q4_k", 15), ("q5_k", 31), ("q6_k", 63), ("q8_0", 254)):
+        out = np.zeros(T.row_bytes(fmt, len(w)), np.uint8)
+        assert S.ckq_synth_quantize(T.FMT[fmt], ptr(w), ptr(out), ctypes.c_size_t(len(w))) == 0
+        back = T.np_dequant(fmt, out)
+        span = np.ptp(w.reshape(-1, T.ELEMS[fmt] if fmt == "q8_0" else 32), axis=1).max()
+        assert np.max(np.abs(back - w)) <= 1.5 * span / steps
+        z = np.zeros(256, np.float32)
+        outz = np.zeros(T.row_bytes(fmt, 256), np.uint8)
+        S.ckq_synth_quantize(T.FMT[fmt], ptr(z), ptr(outz), ctypes.c_size_t(256))
+        assert np.all(T.np_dequant(fmt, outz) == 0.0)
+    # non-zero dmin so the bsums half of the kernels is exercised
+    out = np.zeros(T.row_bytes("q4_k", len(w)), np.uint8)
+    S.ckq_synth_quantize(T.FMT["q4_k"], ptr(w), ptr(out), ctypes.c_size_t(len(w)))
+    assert np.all(T.np_decode_q4_k(out)["dmin"] > 0)
