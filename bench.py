@@ -1,0 +1,226 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized dequant-dot hot path on one MI355X.
+
+A step is one pass of the hot path over one batch of synthetic input: one
+Q4_K x Q8_K GEMV, N=11008 output rows, K=4096, M=1 token (the shape
+BASELINE.json's metric is quoted on), device-resident inputs, launched
+back-to-back on one stream.  Consecutive steps read different copies of the
+weight matrix, enough of them to exceed the 256 MB Infinity Cache, so the
+figure is an HBM figure; the cache-resident rate is reported beside it.
+
+Prints ONE JSON line:  python bench.py [--gpus 1] [--steps K] [--warmup W]
+"""
+import argparse
+import ctypes
+import importlib
+import json
+import os
+import sys
+import threading
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+INT8_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA, published
+MALL_BYTES = 256 << 20
+
+FMT_BYTES = {"q4_k": 144, "q5_k": 176, "q6_k": 210, "q8_0": 34}
+
+
+def gemv_bytes(fmt, rows, K, M=1):
+    """Algorithmic bytes of one call: weights + activations + outputs
+    (the reference's W + x + y accounting, unittest/test_gemv_q_benchmark.py:397-400)."""
+    if fmt == "q8_0":
+        w = rows * (K // 32) * 34
+        x = M * (K // 32) * 34
+    else:
+        w = rows * (K // 256) * FMT_BYTES[fmt]
+        x = M * (K // 256) * 292
+    return w + x + 4 * M * rows
+
+
+class Harness:
+    def __init__(self):
+        import torch
+        self.torch = torch
+        self.ckq = importlib.import_module("c-kernel-engine_amd")
+        self.P = self.ckq.parity
+        self.L = self.ckq.lib()
+        assert self.L.ckq_init() == 0
+        import ckq_testlib as T
+        self.T = T
+
+    def weight_copies(self, fmt, rows, K, seed, min_total=3 * MALL_BYTES // 2):
+        """Distinct device buffers holding the same-shaped matrix (rows rolled
+        so the contents differ), enough of them to defeat the Infinity Cache."""
+        torch = self.torch
+        W = self.T.synth_weights(fmt, rows, K, seed)
+        rb = len(W) // rows
+        base = torch.from_numpy(W).cuda().view(rows, rb)
+        n = max(2, -(-min_total // len(W)))
+        copies = [base.reshape(-1)]
+        for i in range(1, n):
+            copies.append(torch.roll(base, shifts=i * 17, dims=0).contiguous().reshape(-1))
+        return W, copies
+
+    def time_gemv(self, fmt, rows, K, M, copies, xq_d, steps, warmup):
+        """Average seconds per launch over `steps` back-to-back launches,
+        measured with events on the launch stream."""
+        torch, P = self.torch, self.P
+        out = torch.empty(M * rows, dtype=torch.float32, device="cuda")
+        n = len(copies)
+        # one C call enqueues a whole rotation through the weight copies, so no
+        # Python runs between launches
+        ops = [(fmt, xq_d, c, None, out, M, rows, K) for c in copies]
+
+        def run(count):
+            full, rest = divmod(count, n)
+            if full:
+                P.dev_matmul_sequence(ops, repeat=full)
+            if rest:
+                P.dev_matmul_sequence(ops[:rest], repeat=1)
+
+        run(warmup)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        run(steps)
+        e1.record()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        return e0.elapsed_time(e1) * 1e-3 / steps, wall / steps
+
+
+def cpu_baseline(rows, K, seconds_budget=12.0):
+    """Q4_K x Q8_K GEMV on the host cores, same shape.  Uses the reference's
+    own kernels (oracle/_ref, built from the reference checkout) when that
+    library loads, else this repository's restatement."""
+    import numpy as np
+    import ckq_testlib as T
+    W = T.synth_weights("q4_k", rows, K, seed=1)
+    xq = T.oracle_quantize(T.normal(K, seed=2), "q8_k")
+    y = np.zeros(rows, np.float32)
+    kind, lib, fn_name = "port", None, None
+    ref = os.path.join(ROOT, "oracle", "_ref", "libckref_avx2.so")
+    try:
+        lib = ctypes.CDLL(ref)
+        fn_name = "gemv_q4_k_q8_k_parallel_simd"
+        kind = "reference"
+    except OSError:
+        lib = T.oracle()
+        fn_name = "orc_gemv_q4_k_q8_k_parallel"
+    fn = getattr(lib, fn_name)
+    nth = max(1, min(os.cpu_count() or 1, 16))
+    p = T.ptr
+
+    def one_call(threads):
+        if threads == 1:
+            fn(p(y), p(W), p(xq), rows, K, 0, 1)
+            return
+        ts = [threading.Thread(target=fn, args=(p(y), p(W), p(xq), rows, K, i, threads)) for i in range(threads)]
+        for t in ts:
+            t.start()
+        for t in ts:
+            t.join()
+
+    res = {}
+    for threads in (1, nth):
+        one_call(threads)
+        t0 = time.perf_counter()
+        one_call(threads)
+        per = max(time.perf_counter() - t0, 1e-6)
+        iters = int(max(3, min(200, (seconds_budget / 2) / per)))
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            one_call(threads)
+        res[threads] = ((time.perf_counter() - t0) / iters, iters)
+    bytes_ = gemv_bytes("q4_k", rows, K)
+    sec, iters = res[nth]
+    return {
+        "value": round(bytes_ / sec / 1e9, 3), "unit": "GB/s", "cores": nth, "kind": kind,
+        "sample": "%d calls of %s %dx%d M=1 row-split over %d threads (%.2f ms/call); single thread %.2f ms/call = %.3f GB/s"
+                  % (iters, fn_name, rows, K, nth, sec * 1e3, res[1][0] * 1e3, bytes_ / res[1][0] / 1e9),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extras", action="store_true", help="only the headline workload")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported (every box here has one GPU, "
+                 "see DESIGN.md for how the path would shard)" % a.gpus)
+
+    H = Harness()
+    torch, P, T = H.torch, H.P, H.T
+    rows, K, M = 11008, 4096, 1
+    xf = T.normal(K, 0.0, 1.0, seed=4242)
+    xq_d = P.dev_quantize(P.to_device(xf), "q8_k")
+    W, copies = H.weight_copies("q4_k", rows, K, seed=4243)
+
+    # parity guard on the exact buffers being timed
+    import numpy as np
+    y = P.dev_gemm_nt("q4_k", xq_d, copies[0], None, 1, rows, K).cpu().numpy().reshape(-1)
+    err = T.norm_err(y, T.oracle_gemv("q4_k", W, xq_d.cpu().numpy(), rows, K))
+    assert err <= 1e-4, "parity check failed before timing: %g" % err
+
+    sec, wall = H.time_gemv("q4_k", rows, K, M, copies, xq_d, a.steps, a.warmup)
+    bytes_ = gemv_bytes("q4_k", rows, K, M)
+    gbs = bytes_ / sec / 1e9
+    sec_hot, _ = H.time_gemv("q4_k", rows, K, M, copies[:1], xq_d, a.steps, a.warmup)
+
+    out = {
+        "metric": "Q4_K GEMV GB/s (% HBM peak) at M=1; Q4_K x Q8_K GEMM TOPS at M=512",
+        "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(sec * 1e3, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8 dot (Q4_K x Q8_K), fp32 accumulate", "data": "synthetic",
+        "config": {"workload": "Q4_K x Q8_K GEMV N=11008 K=4096 M=1", "weights": "seeded N(0,0.02) -> Q4_K",
+                   "activations": "seeded N(0,1) -> Q8_K (quantized on the GPU)",
+                   "weight_copies_rotated": len(copies), "bytes_per_step": bytes_},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+        "pct_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
+        "cache_resident_gbs": round(bytes_ / sec_hot / 1e9, 2),
+        "host_wall_ms_per_step": round(wall * 1e3, 6),
+        "parity_norm_err": err,
+    }
+
+    if not a.no_extras:
+        extras = {}
+        # prefill GEMM, M=512 x N=11008 x K=4096
+        Mg = 512
+        xg = P.dev_quantize(P.to_device(T.normal(Mg * K, seed=99)), "q8_k", rows=Mg)
+        steps_g = max(3, min(20, a.steps // 100))
+        sg, _ = H.time_gemv("q4_k", rows, K, Mg, copies[:2], xg, steps_g, 2)
+        ops = 2.0 * Mg * rows * K
+        extras["gemm_q4_k_q8_k_M512"] = {"tops": round(ops / sg / 1e12, 2), "ms": round(sg * 1e3, 4),
+                                         "frac_int8_peak": round(ops / sg / 1e12 / INT8_PEAK_TOPS, 4),
+                                         "ops_per_call": ops, "kernel": "dot4 GEMV kernel, 8-token tiles"}
+        for name, fmt, r, k in (("gemv_q4_k_4096x4096", "q4_k", 4096, 4096),
+                                ("lm_head_q6_k_32000x4096", "q6_k", 32000, 4096),
+                                ("down_q6_k_4096x11008", "q6_k", 4096, 11008),
+                                ("lm_head_q8_0_151936x896", "q8_0", 151936, 896)):
+            _, cps = H.weight_copies(fmt, r, k, seed=r + k)
+            xq = P.dev_quantize(P.to_device(T.normal(k, seed=k)), T.act_fmt(fmt))
+            s, _ = H.time_gemv(fmt, r, k, 1, cps, xq, max(50, a.steps // 4), 20)
+            b = gemv_bytes(fmt, r, k)
+            extras[name] = {"gbs": round(b / s / 1e9, 1), "us": round(s * 1e6, 2), "frac_hbm": round(b / s / 1e9 / HBM_PEAK_GBS, 4)}
+            del cps
+            torch.cuda.empty_cache()
+        out["extras"] = extras
+
+    if not a.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(rows, K)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,159 @@
+"""ctypes binding of libckernel_quant_hip.so (the C ABI declared in
+include/ckernel_quant_hip.h) and of the host-side synthetic-data helper."""
+import ctypes
+import os
+import re
+import subprocess
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+HEADER = os.path.join(ROOT, "include", "ckernel_quant_hip.h")
+
+FMT = {"q4_k": 0, "q5_k": 1, "q6_k": 2, "q8_0": 3, "q8_k": 4}
+BLOCK_BYTES = {"q4_k": 144, "q5_k": 176, "q6_k": 210, "q8_0": 34, "q8_k": 292}
+BLOCK_ELEMS = {"q4_k": 256, "q5_k": 256, "q6_k": 256, "q8_0": 32, "q8_k": 256}
+
+
+class CkqError(RuntimeError):
+    pass
+
+
+def row_bytes(fmt, k):
+    return (k // BLOCK_ELEMS[fmt]) * BLOCK_BYTES[fmt]
+
+
+def lib_path():
+    return os.path.join(CSRC, "libckernel_quant_hip.so")
+
+
+def build(targets=("synth", "hip")):
+    """Compile the host helper and the gfx950 library in-tree (hipcc
+    cross-compiles without a GPU)."""
+    subprocess.run(["make", "-C", CSRC, "-B"] + list(targets), check=True)
+
+
+_c = ctypes
+_vp, _i, _l, _f32p = _c.c_void_p, _c.c_int, _c.c_long, _c.c_void_p
+
+# name -> (restype, argtypes); pointers are passed as integers / c_void_p so
+# that host arrays and device addresses go through the same binding.
+_SIGS = {
+    "quantize_row_q8_k": (None, [_vp, _vp, _i]),
+    "quantize_batch_q8_k": (None, [_vp, _vp, _i, _i]),
+    "quantize_row_q8_0": (None, [_vp, _vp, _i]),
+    "quantize_batch_q8_0": (None, [_vp, _vp, _i, _i]),
+    "gemv_q4_k_q8_k": (None, [_vp, _vp, _vp, _i, _i]),
+    "gemv_q4_k_q8_k_ref": (None, [_vp, _vp, _vp, _i, _i]),
+    "gemv_q4_k_q8_k_parallel": (None, [_vp, _vp, _vp, _i, _i, _i, _i]),
+    "gemv_q4_k_q8_k_parallel_simd": (None, [_vp, _vp, _vp, _i, _i, _i, _i]),
+    "gemm_q4_k_q8_k": (None, [_vp, _vp, _vp, _i, _i, _i]),
+    "gemm_nt_q4_k_q8_k": (None, [_vp, _vp, _vp, _vp, _i, _i, _i]),
+    "gemv_q5_k_q8_k": (None, [_vp, _vp, _vp, _i, _i]),
+    "gemm_nt_q5_k_q8_k": (None, [_vp, _vp, _vp, _vp, _i, _i, _i]),
+    "gemv_q5_k": (None, [_vp, _vp, _vp, _i, _i]),
+    "gemm_nt_q5_k": (None, [_vp, _vp, _vp, _vp, _i, _i, _i]),
+    "vec_dot_q6_k_q8_k": (None, [_i, _vp, _vp, _vp]),
+    "gemv_q6_k_q8_k": (None, [_vp, _vp, _vp, _i, _i]),
+    "gemv_q6_k_q8_k_parallel": (None, [_vp, _vp, _vp, _i, _i, _i, _i]),
+    "gemv_q6_k_q8_k_parallel_simd": (None, [_vp, _vp, _vp, _i, _i, _i, _i]),
+    "gemm_q6_k_q8_k": (None, [_vp, _vp, _vp, _i, _i, _i]),
+    "gemm_nt_q6_k_q8_k": (None, [_vp, _vp, _vp, _vp, _i, _i, _i]),
+    "vec_dot_q8_0_q8_0": (None, [_i, _vp, _vp, _vp]),
+    "gemv_q8_0_q8_0": (None, [_vp, _vp, _vp, _i, _i]),
+    "gemv_q8_0_q8_0_parallel": (None, [_vp, _vp, _vp, _i, _i, _i, _i]),
+    "gemv_q8_0_q8_0_parallel_simd": (None, [_vp, _vp, _vp, _i, _i, _i, _i]),
+    "gemv_q8_0": (None, [_vp, _vp, _vp, _i, _i]),
+    "gemm_nt_q8_0_q8_0": (None, [_vp, _vp, _vp, _vp, _i, _i, _i]),
+    "ck_test_quantize_q8_k": (None, [_vp, _vp, _i]),
+    "ck_test_gemv_q4_k": (None, [_vp, _vp, _vp, _i]),
+    "ck_test_gemv_q6_k": (None, [_vp, _vp, _vp, _i]),
+    "ck_test_gemv_q8_0": (None, [_vp, _vp, _vp, _i, _i]),
+    "ck_test_gemv_q8_0_q8_0": (None, [_vp, _vp, _vp, _i, _i]),
+    "ck_test_vec_dot_q8_0_q8_0": (None, [_vp, _vp, _vp, _i]),
+    "ck_test_gemm_q4_k": (None, [_vp, _vp, _vp, _i, _i, _i]),
+    "ck_test_gemm_q6_k": (None, [_vp, _vp, _vp, _i, _i, _i]),
+    "ck_test_gemm_q8_0": (None, [_vp, _vp, _vp, _i, _i, _i]),
+    "ck_get_block_q4_k_size": (_i, []),
+    "ck_get_block_q6_k_size": (_i, []),
+    "ck_get_block_q8_k_size": (_i, []),
+    "ck_get_qk_k": (_i, []),
+    "ckq_quantize_q8_k_dev": (_i, [_vp, _vp, _i, _i, _vp]),
+    "ckq_quantize_q8_0_dev": (_i, [_vp, _vp, _i, _i, _vp]),
+    "ckq_gemm_nt_dev": (_i, [_i, _vp, _vp, _vp, _vp, _i, _i, _i, _l, _vp]),
+    "ckq_gemv_q4_k_q8_k_dev": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
+    "ckq_gemv_q5_k_q8_k_dev": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
+    "ckq_gemv_q6_k_q8_k_dev": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
+    "ckq_gemv_q8_0_q8_0_dev": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
+    "ckq_gemv_q8_0_dev": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
+    "ckq_gemm_nt_q4_k_q8_k_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "ckq_gemm_nt_q5_k_q8_k_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "ckq_gemm_nt_q6_k_q8_k_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "ckq_gemm_nt_q8_0_q8_0_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "ckq_matmul_sequence_dev": (_i, [_vp, _i, _i, _vp]),
+    "ckq_subblock_dots_dev": (_i, [_i, _vp, _vp, _vp, _i, _i, _vp]),
+    "ckq_copy_dev": (_i, [_vp, _vp, _c.c_size_t, _vp]),
+    "ckq_init": (_i, []),
+    "ckq_synchronize": (_i, []),
+    "ckq_weights_register": (_i, [_vp, _c.c_size_t]),
+    "ckq_weights_invalidate": (None, [_vp]),
+    "ckq_weights_clear": (None, []),
+    "ckq_weights_set_cache": (None, [_i]),
+    "ckq_set_parallel_whole": (None, [_i]),
+    "ckq_last_error": (_i, []),
+    "ckq_error_string": (_c.c_char_p, [_i]),
+}
+
+
+
+class MatmulOp(ctypes.Structure):
+    """ckq_matmul_op of include/ckernel_quant_hip.h."""
+    _fields_ = [("fmt", _i), ("M", _i), ("N", _i), ("K", _i), ("ldc", _l),
+                ("A_q8", _vp), ("B", _vp), ("bias", _vp), ("C", _vp)]
+
+
+_lib = None
+_synth = None
+
+
+def declared_symbols():
+    """Function names declared in include/ckernel_quant_hip.h."""
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"typedef\s+struct\s*\{.*?\}\s*\w+;", "", text, flags=re.S)
+    names = re.findall(r"^\s*(?:const\s+)?(?:void|int|char)\s*\*?\s*(\w+)\s*\(", text, flags=re.M)
+    return sorted(set(names))
+
+
+def lib():
+    """The gfx950 library.  Raises CkqError if it has not been built: there is
+    no fallback implementation."""
+    global _lib
+    if _lib is None:
+        path = lib_path()
+        if not os.path.exists(path):
+            raise CkqError("%s is missing: run `python -c 'import __graft_entry__ as g; g.build()'` "
+                           "(there is no CPU fallback)" % path)
+        L = ctypes.CDLL(path)
+        for name, (res, args) in _SIGS.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+def synth_lib():
+    """Host-side synthetic-data generator and weight encoders."""
+    global _synth
+    if _synth is None:
+        path = os.path.join(CSRC, "libckq_synth.so")
+        if not os.path.exists(path):
+            raise CkqError("%s is missing: build it with `make -C %s synth`" % (path, CSRC))
+        _synth = ctypes.CDLL(path)
+    return _synth
+
+
+def check(rc, what):
+    if rc != 0:
+        raise CkqError("%s failed: %s (%d)" % (what, lib().ckq_error_string(rc).decode(), rc))

@@ -1,0 +1,267 @@
+/*
+ * ckq_formats.cuh - per-format traits for the dequant-dot kernels.
+ *
+ * A weight row is cut into "positions": the unit of work of one lane.
+ *   Q4_K / Q5_K : one 64-element group of a super-block (header + 32 B of
+ *                 nibbles [+ 32 B of fifth bits]); two sub-blocks, two scales.
+ *   Q6_K        : 64 elements of a super-block: a 16-wide slice l0 of one
+ *                 128-half, i.e. elements l0+{0,32,64,96}+[0,16); 48 B of
+ *                 quants, four scales.
+ *   Q8_0        : one 32-element block (34 B).
+ * Each trait provides
+ *   Wt  / load_w   raw weight dwords of a position (nothing decoded yet, so all
+ *                  loads of a wave can be in flight together),
+ *   Act / load_act the activation slice the position multiplies with,
+ *   Dec / decode   quants unpacked to int8x4 dwords and integer scales,
+ *   dot            integer sub-block dots -> integer block-scale combination
+ *                  -> one fp32 partial,
+ *   NSUB / dump    the raw integer sub-block dots, for the bit-exactness tests.
+ *
+ * Arithmetic contracts (reference file:line):
+ *   Q4_K x Q8_K  gemm_kernels_q4k_q8k.c:121-181   d*sc*S - dmin*m*(stored bsums)
+ *   Q5_K x Q8_K  gemm_kernels_q5_k.c:130-208      same with 5-bit quants
+ *   Q6_K x Q8_K  gemm_kernels_q6k_q8k.c:601-695   d * sum_s sc_s*sum (q-32)*q8, bsums unused
+ *   Q8_0 x Q8_0  gemm_kernels_q8_0.c:968-989      sumi * (fp16 dw * fp16 dx)
+ *   Q8_0 x fp32  gemm_kernels_q8_0.c:254-277      sum d*q*x
+ */
+#pragma once
+#include "ckq_device.cuh"
+
+/* 6-bit scale/min pair of sub-blocks (2g, 2g+1) from the 12 packed bytes
+ * (layout: reference include/ckernel_quant.h:227-251).  u0,u1,u2 are the
+ * three little-endian words of scales[12].  Returns sc in the low two bytes
+ * of *sc2 (byte 0 = sub-block 2g) and likewise the mins. */
+__device__ __forceinline__ void k4_scale_pair(u32 u0, u32 u1, u32 u2, int g, u32 *sc2, u32 *mn2)
+{
+    const int sh = 16 * (g & 1);
+    const u32 a = u0 >> sh, b = u1 >> sh, c = u2 >> sh;
+    const u32 sc_lo = a & 0x3f3fu, mn_lo = b & 0x3f3fu;
+    const u32 sc_hi = (c & 0x0f0fu) | (((a >> 6) & 0x0303u) << 4);
+    const u32 mn_hi = ((c >> 4) & 0x0f0fu) | (((b >> 6) & 0x0303u) << 4);
+    *sc2 = g < 2 ? sc_lo : sc_hi;
+    *mn2 = g < 2 ? mn_lo : mn_hi;
+}
+
+/* ------------------------------------------------------------------------- */
+struct FmtQ4K {
+    static constexpr int POS_PER_BLOCK = 4, WBLOCK = 144, XBLOCK = 292, NSUB = 2;
+    struct Wt  { u32 hdr[4]; u32 qs[8]; };
+    struct Act { int q[16]; float d; int b_lo, b_hi; };
+    struct Dec { int lo[8], hi[8]; int sc_lo, sc_hi, mn_lo, mn_hi; float d, dmin; };
+
+    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, int pos)
+    {
+        const uint8_t *blk = row + (size_t)(pos >> 2) * WBLOCK;
+        ld16<4>(w.hdr, blk);
+        ld16<4>(w.qs, blk + 16 + 32 * (pos & 3));
+        ld16<4>(w.qs + 4, blk + 32 + 32 * (pos & 3));
+    }
+    static __device__ __forceinline__ void load_act(Act &a, const uint8_t *x, int pos)
+    {
+        const uint8_t *blk = x + (size_t)(pos >> 2) * XBLOCK;
+        const int g = pos & 3;
+        a.d = __builtin_bit_cast(float, ld4<4>(blk));
+        for (int i = 0; i < 4; ++i) ld16<4>(a.q + 4 * i, blk + 4 + 64 * g + 16 * i);
+        u32 bs[2];
+        ld8<4>(bs, blk + 260 + 8 * g);   /* stored bsums[4g..4g+3] */
+        a.b_lo = (int)(int16_t)(bs[0] & 0xffff) + (int)(int16_t)(bs[0] >> 16);
+        a.b_hi = (int)(int16_t)(bs[1] & 0xffff) + (int)(int16_t)(bs[1] >> 16);
+    }
+    static __device__ __forceinline__ void decode(Dec &d, const Wt &w, int pos)
+    {
+        u32 sc2, mn2;
+        k4_scale_pair(w.hdr[1], w.hdr[2], w.hdr[3], pos & 3, &sc2, &mn2);
+        d.sc_lo = sc2 & 0xff; d.sc_hi = (sc2 >> 8) & 0xff;
+        d.mn_lo = mn2 & 0xff; d.mn_hi = (mn2 >> 8) & 0xff;
+        d.d = h2f(w.hdr[0] & 0xffff);
+        d.dmin = h2f(w.hdr[0] >> 16);
+        for (int i = 0; i < 8; ++i) {
+            d.lo[i] = (int)(w.qs[i] & 0x0f0f0f0fu);
+            d.hi[i] = (int)((w.qs[i] >> 4) & 0x0f0f0f0fu);
+        }
+    }
+    static __device__ __forceinline__ float dot(const Dec &d, const Act &a, int *sub)
+    {
+        int s_lo = 0, s_hi = 0;
+        for (int i = 0; i < 8; ++i) {
+            s_lo = dot4(d.lo[i], a.q[i], s_lo);
+            s_hi = dot4(d.hi[i], a.q[8 + i], s_hi);
+        }
+        sub[0] = s_lo; sub[1] = s_hi;
+        const int i1 = mul24(d.sc_lo, s_lo) + mul24(d.sc_hi, s_hi);
+        const int i2 = mul24(d.mn_lo, a.b_lo) + mul24(d.mn_hi, a.b_hi);
+        return (d.d * a.d) * (float)i1 - (d.dmin * a.d) * (float)i2;
+    }
+    /* index of sub[i] among the 8 sub-block dots of the position's block */
+    static __device__ __forceinline__ int sub_index(int pos, int i) { return 8 * (pos >> 2) + 2 * (pos & 3) + i; }
+    static constexpr int SUBS_PER_BLOCK = 8;
+};
+
+/* ------------------------------------------------------------------------- */
+struct FmtQ5K {
+    static constexpr int POS_PER_BLOCK = 4, WBLOCK = 176, XBLOCK = 292, NSUB = 2;
+    struct Wt  { u32 hdr[4]; u32 qh[8]; u32 qs[8]; };
+    typedef FmtQ4K::Act Act;
+    typedef FmtQ4K::Dec Dec;
+
+    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, int pos)
+    {
+        const uint8_t *blk = row + (size_t)(pos >> 2) * WBLOCK;
+        ld16<4>(w.hdr, blk);
+        ld16<4>(w.qh, blk + 16);
+        ld16<4>(w.qh + 4, blk + 32);
+        ld16<4>(w.qs, blk + 48 + 32 * (pos & 3));
+        ld16<4>(w.qs + 4, blk + 64 + 32 * (pos & 3));
+    }
+    static __device__ __forceinline__ void load_act(Act &a, const uint8_t *x, int pos) { FmtQ4K::load_act(a, x, pos); }
+    static __device__ __forceinline__ void decode(Dec &d, const Wt &w, int pos)
+    {
+        const int g = pos & 3;
+        u32 sc2, mn2;
+        k4_scale_pair(w.hdr[1], w.hdr[2], w.hdr[3], g, &sc2, &mn2);
+        d.sc_lo = sc2 & 0xff; d.sc_hi = (sc2 >> 8) & 0xff;
+        d.mn_lo = mn2 & 0xff; d.mn_hi = (mn2 >> 8) & 0xff;
+        d.d = h2f(w.hdr[0] & 0xffff);
+        d.dmin = h2f(w.hdr[0] >> 16);
+        for (int i = 0; i < 8; ++i) {
+            const u32 h = w.qh[i] >> (2 * g);   /* bit 0: fifth bit of low-nibble element, bit 1: of high-nibble element */
+            d.lo[i] = (int)((w.qs[i] & 0x0f0f0f0fu) | ((h & 0x01010101u) << 4));
+            d.hi[i] = (int)(((w.qs[i] >> 4) & 0x0f0f0f0fu) | (((h >> 1) & 0x01010101u) << 4));
+        }
+    }
+    static __device__ __forceinline__ float dot(const Dec &d, const Act &a, int *sub) { return FmtQ4K::dot(d, a, sub); }
+    static __device__ __forceinline__ int sub_index(int pos, int i) { return FmtQ4K::sub_index(pos, i); }
+    static constexpr int SUBS_PER_BLOCK = 8;
+};
+
+/* ------------------------------------------------------------------------- */
+struct FmtQ6K {
+    static constexpr int POS_PER_BLOCK = 4, WBLOCK = 210, XBLOCK = 292, NSUB = 4;
+    struct Wt  { u32 ql0[4], ql1[4], qh[4]; u32 sc[2]; u32 d; };
+    struct Act { int q[16]; float d; int a32[4]; };      /* a32[r] = 32 * sum of the run's 16 quants */
+    struct Dec { int q[16]; int sc[4]; float d; };
+
+    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, int pos)
+    {
+        const uint8_t *blk = row + (size_t)(pos >> 2) * WBLOCK;
+        const int n = (pos >> 1) & 1, l0 = 16 * (pos & 1);
+        ld16<2>(w.ql0, blk + 64 * n + l0);
+        ld16<2>(w.ql1, blk + 64 * n + 32 + l0);
+        ld16<2>(w.qh, blk + 128 + 32 * n + l0);
+        ld8<2>(w.sc, blk + 192 + 8 * n);
+        w.d = ld2(blk + 208);
+    }
+    static __device__ __forceinline__ void load_act(Act &a, const uint8_t *x, int pos)
+    {
+        const uint8_t *blk = x + (size_t)(pos >> 2) * XBLOCK;
+        const int n = (pos >> 1) & 1, l0 = 16 * (pos & 1);
+        a.d = __builtin_bit_cast(float, ld4<4>(blk));
+        for (int r = 0; r < 4; ++r) {
+            ld16<4>(a.q + 4 * r, blk + 4 + 128 * n + 32 * r + l0);
+            int s = 0;
+            for (int i = 0; i < 4; ++i) s = dot4(0x01010101, a.q[4 * r + i], s);
+            a.a32[r] = 32 * s;   /* computed from the quants: the reference's x86 routine never reads bsums here */
+        }
+    }
+    static __device__ __forceinline__ void decode(Dec &d, const Wt &w, int pos)
+    {
+        const int odd = pos & 1;
+        for (int i = 0; i < 4; ++i) {
+            const u32 h = w.qh[i];
+            d.q[i]      = (int)((w.ql0[i] & 0x0f0f0f0fu)        | ((h & 0x03030303u) << 4));
+            d.q[4 + i]  = (int)((w.ql1[i] & 0x0f0f0f0fu)        | (((h >> 2) & 0x03030303u) << 4));
+            d.q[8 + i]  = (int)(((w.ql0[i] >> 4) & 0x0f0f0f0fu) | (((h >> 4) & 0x03030303u) << 4));
+            d.q[12 + i] = (int)(((w.ql1[i] >> 4) & 0x0f0f0f0fu) | (((h >> 6) & 0x03030303u) << 4));
+        }
+        /* scales[8n + odd + 2r], r = 0..3 */
+        d.sc[0] = sbyte(w.sc[0], odd);
+        d.sc[1] = sbyte(w.sc[0], odd + 2);
+        d.sc[2] = sbyte(w.sc[1], odd);
+        d.sc[3] = sbyte(w.sc[1], odd + 2);
+        d.d = h2f(w.d);
+    }
+    static __device__ __forceinline__ float dot(const Dec &d, const Act &a, int *sub)
+    {
+        int i1 = 0;
+        for (int r = 0; r < 4; ++r) {
+            int s = 0;
+            for (int i = 0; i < 4; ++i) s = dot4(d.q[4 * r + i], a.q[4 * r + i], s);
+            s -= a.a32[r];              /* sum (q-32)*q8 = sum q*q8 - 32*sum q8 */
+            sub[r] = s;
+            i1 += mul24(d.sc[r], s);
+        }
+        return (d.d * a.d) * (float)i1;
+    }
+    static __device__ __forceinline__ int sub_index(int pos, int r)
+    {
+        return 16 * (pos >> 2) + 8 * ((pos >> 1) & 1) + (pos & 1) + 2 * r;
+    }
+    static constexpr int SUBS_PER_BLOCK = 16;
+};
+
+/* ------------------------------------------------------------------------- */
+struct FmtQ80 {
+    static constexpr int POS_PER_BLOCK = 1, WBLOCK = 34, XBLOCK = 34, NSUB = 1;
+    struct Wt  { u32 q[8]; u32 d; };
+    struct Act { int q[8]; float d; };
+    struct Dec { int q[8]; float d; };
+
+    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, int pos)
+    {
+        const uint8_t *blk = row + (size_t)pos * WBLOCK;
+        w.d = ld2(blk);
+        ld16<2>(w.q, blk + 2);
+        ld16<2>(w.q + 4, blk + 18);
+    }
+    static __device__ __forceinline__ void load_act(Act &a, const uint8_t *x, int pos)
+    {
+        const uint8_t *blk = x + (size_t)pos * XBLOCK;
+        a.d = h2f(ld2(blk));
+        ld16<2>(a.q, blk + 2);
+        ld16<2>(a.q + 4, blk + 18);
+    }
+    static __device__ __forceinline__ void decode(Dec &d, const Wt &w, int)
+    {
+        for (int i = 0; i < 8; ++i) d.q[i] = (int)w.q[i];
+        d.d = h2f(w.d);
+    }
+    static __device__ __forceinline__ float dot(const Dec &d, const Act &a, int *sub)
+    {
+        int s = 0;
+        for (int i = 0; i < 8; ++i) s = dot4(d.q[i], a.q[i], s);
+        sub[0] = s;
+        return (float)s * (d.d * a.d);
+    }
+    static __device__ __forceinline__ int sub_index(int pos, int) { return pos; }
+    static constexpr int SUBS_PER_BLOCK = 1;
+};
+
+/* Q8_0 weights against fp32 activations (no activation quantization). */
+struct FmtQ80F32 {
+    static constexpr int POS_PER_BLOCK = 1, WBLOCK = 34, XBLOCK = 128, NSUB = 1;
+    typedef FmtQ80::Wt Wt;
+    typedef FmtQ80::Dec Dec;
+    struct Act { float x[32]; };
+
+    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, int pos) { FmtQ80::load_w(w, row, pos); }
+    static __device__ __forceinline__ void load_act(Act &a, const uint8_t *x, int pos)
+    {
+        const uint8_t *p = x + (size_t)pos * XBLOCK;
+        for (int i = 0; i < 8; ++i) {
+            u32 t[4];
+            ld16<4>(t, p + 16 * i);
+            for (int j = 0; j < 4; ++j) a.x[4 * i + j] = __builtin_bit_cast(float, t[j]);
+        }
+    }
+    static __device__ __forceinline__ void decode(Dec &d, const Wt &w, int pos) { FmtQ80::decode(d, w, pos); }
+    static __device__ __forceinline__ float dot(const Dec &d, const Act &a, int *sub)
+    {
+        float s = 0.0f;
+        for (int i = 0; i < 8; ++i)
+            for (int j = 0; j < 4; ++j) s += (d.d * (float)sbyte((u32)d.q[i], j)) * a.x[4 * i + j];
+        sub[0] = 0;
+        return s;
+    }
+    static __device__ __forceinline__ int sub_index(int pos, int) { return pos; }
+    static constexpr int SUBS_PER_BLOCK = 1;
+};

@@ -1,0 +1,692 @@
+/*
+ * ckq_host.c - host layer of libckernel_quant_hip.so (plain C).
+ *
+ * Implements the reference engine's kernel symbols for the quantized
+ * dequant-dot path (declared in include/ckernel_quant_hip.h, part 1) on top of
+ * the device launchers of ckq_launch.h, plus the device-resident `_dev` entry
+ * points and the library control calls.
+ *
+ * Host-pointer calls: activations are copied to the device, the kernel runs on
+ * the library's stream, results are copied back and the stream is synchronized
+ * before returning (the reference kernels are synchronous).  Weight matrices
+ * are uploaded once and stay resident, keyed by host address, size and a
+ * sampled fingerprint.  Device pointers are detected and used in place.
+ * One mutex serializes the host-pointer entry points, so they may be called
+ * from any number of threads (the reference's thread pool calls the same
+ * symbol from every worker).
+ *
+ * There is no CPU fallback: if no gfx950 device is usable every entry point
+ * reports the HIP error on stderr and aborts (set CKQ_ABORT_ON_ERROR=0 to get
+ * the code from ckq_last_error() instead).
+ */
+#include <hip/hip_runtime_api.h>
+#include <pthread.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "ckernel_quant_hip.h"
+#include "ckq_launch.h"
+
+/* ------------------------------------------------------------------------ */
+/* State                                                                     */
+/* ------------------------------------------------------------------------ */
+
+typedef struct {
+    const void *host;
+    size_t      bytes;
+    uint64_t    fp;
+    void       *dev;
+} weight_entry;
+
+typedef struct {
+    void  *dev;
+    size_t cap;
+} dev_buf;
+
+enum { BUF_X = 0, BUF_Y, BUF_BIAS, BUF_Q, BUF_COUNT };
+
+static pthread_mutex_t g_mu = PTHREAD_MUTEX_INITIALIZER;
+static int          g_inited = 0;
+static int          g_err = 0;
+static int          g_cache_on = 1;
+static int          g_parallel_whole = 0;
+static hipStream_t  g_stream = NULL;
+static dev_buf      g_buf[BUF_COUNT];
+static weight_entry *g_w = NULL;
+static size_t       g_nw = 0, g_capw = 0;
+
+/* ------------------------------------------------------------------------ */
+/* Errors                                                                    */
+/* ------------------------------------------------------------------------ */
+
+const char *ckq_error_string(int code)
+{
+    switch (code) {
+    case 0: return "success";
+    case CKQ_EINVAL: return "invalid argument (NULL pointer or non-positive dimension)";
+    case CKQ_ESHAPE: return "K is not a multiple of the quantization block size";
+    case CKQ_EFORMAT: return "unknown weight format";
+    default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
+    }
+}
+
+int ckq_last_error(void) { return g_err; }
+
+static int fail(int code, const char *what)
+{
+    if (code == 0) return 0;
+    g_err = code;
+    fprintf(stderr, "libckernel_quant_hip: %s failed: %s (%d)\n", what, ckq_error_string(code), code);
+    const char *e = getenv("CKQ_ABORT_ON_ERROR");
+    if (!e || strcmp(e, "0") != 0) {
+        fprintf(stderr, "libckernel_quant_hip: no CPU fallback exists; aborting (CKQ_ABORT_ON_ERROR=0 to continue)\n");
+        abort();
+    }
+    return code;
+}
+
+#define HIP_TRY(expr)                                   \
+    do {                                                \
+        hipError_t e_ = (expr);                         \
+        if (e_ != hipSuccess) return fail((int)e_, #expr); \
+    } while (0)
+
+/* ------------------------------------------------------------------------ */
+/* Init, buffers, pointer classification                                     */
+/* ------------------------------------------------------------------------ */
+
+static int init_locked(void)
+{
+    if (g_inited) return 0;
+    int n = 0;
+    HIP_TRY(hipGetDeviceCount(&n));
+    if (n <= 0) return fail((int)hipErrorNoDevice, "hipGetDeviceCount");
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, dev));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        fprintf(stderr, "libckernel_quant_hip: device %d is %s; this library holds gfx950 code only\n", dev,
+                prop.gcnArchName);
+        return fail((int)hipErrorInvalidDeviceFunction, "architecture check");
+    }
+    HIP_TRY(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
+    const char *c = getenv("CKQ_WEIGHT_CACHE");
+    if (c && strcmp(c, "0") == 0) g_cache_on = 0;
+    const char *p = getenv("CKQ_PARALLEL_MODE");
+    if (p && strcmp(p, "whole") == 0) g_parallel_whole = 1;
+    g_inited = 1;
+    return 0;
+}
+
+int ckq_init(void)
+{
+    pthread_mutex_lock(&g_mu);
+    const int rc = init_locked();
+    pthread_mutex_unlock(&g_mu);
+    return rc;
+}
+
+int ckq_synchronize(void)
+{
+    pthread_mutex_lock(&g_mu);
+    int rc = init_locked();
+    if (rc == 0) {
+        hipError_t e = hipStreamSynchronize(g_stream);
+        if (e != hipSuccess) rc = fail((int)e, "hipStreamSynchronize");
+    }
+    pthread_mutex_unlock(&g_mu);
+    return rc;
+}
+
+static int is_device_ptr(const void *p)
+{
+    hipPointerAttribute_t at;
+    memset(&at, 0, sizeof(at));
+    hipError_t e = hipPointerGetAttributes(&at, p);
+    if (e != hipSuccess) {
+        (void)hipGetLastError(); /* plain host memory: clear the sticky error */
+        return 0;
+    }
+    return at.type == hipMemoryTypeDevice || at.type == hipMemoryTypeManaged;
+}
+
+static int buf_reserve(int which, size_t bytes, void **out)
+{
+    dev_buf *b = &g_buf[which];
+    if (b->cap < bytes) {
+        if (b->dev) {
+            HIP_TRY(hipStreamSynchronize(g_stream));
+            HIP_TRY(hipFree(b->dev));
+            b->dev = NULL;
+            b->cap = 0;
+        }
+        size_t cap = bytes + bytes / 4 + 4096;
+        HIP_TRY(hipMalloc(&b->dev, cap));
+        b->cap = cap;
+    }
+    *out = b->dev;
+    return 0;
+}
+
+/* Device view of an input: device pointers pass through, host memory is
+ * copied into staging buffer `which`. */
+static int stage_in(int which, const void *p, size_t bytes, const void **out)
+{
+    if (is_device_ptr(p)) {
+        *out = p;
+        return 0;
+    }
+    void *d = NULL;
+    int rc = buf_reserve(which, bytes, &d);
+    if (rc) return rc;
+    HIP_TRY(hipMemcpyAsync(d, p, bytes, hipMemcpyHostToDevice, g_stream));
+    *out = d;
+    return 0;
+}
+
+/* ------------------------------------------------------------------------ */
+/* Weight residency                                                          */
+/* ------------------------------------------------------------------------ */
+
+static uint64_t fingerprint(const void *p, size_t bytes)
+{
+    /* FNV-1a over 64 samples of 64 bytes spread across the matrix. */
+    const uint8_t *b = (const uint8_t *)p;
+    uint64_t h = 0xcbf29ce484222325ull ^ bytes;
+    const size_t chunk = 64, n = 64;
+    const size_t step = bytes > chunk * n ? (bytes - chunk) / (n - 1) : chunk;
+    for (size_t i = 0; i < n; ++i) {
+        size_t off = i * step;
+        if (off >= bytes) break;
+        size_t len = bytes - off < chunk ? bytes - off : chunk;
+        for (size_t j = 0; j < len; ++j) h = (h ^ b[off + j]) * 0x100000001b3ull;
+    }
+    return h;
+}
+
+static int weights_lookup(const void *W, size_t bytes, const void **out)
+{
+    if (is_device_ptr(W)) {
+        *out = W;
+        return 0;
+    }
+    const uint64_t fp = fingerprint(W, bytes);
+    for (size_t i = 0; i < g_nw; ++i) {
+        if (g_w[i].host == W && g_w[i].bytes == bytes) {
+            if (g_w[i].fp == fp) {
+                *out = g_w[i].dev;
+                return 0;
+            }
+            /* same address, new content: refresh in place */
+            HIP_TRY(hipMemcpyAsync(g_w[i].dev, W, bytes, hipMemcpyHostToDevice, g_stream));
+            g_w[i].fp = fp;
+            *out = g_w[i].dev;
+            return 0;
+        }
+    }
+    if (g_nw == g_capw) {
+        size_t nc = g_capw ? g_capw * 2 : 64;
+        weight_entry *nw = (weight_entry *)realloc(g_w, nc * sizeof(*nw));
+        if (!nw) return fail((int)hipErrorOutOfMemory, "realloc weight table");
+        g_w = nw;
+        g_capw = nc;
+    }
+    void *d = NULL;
+    HIP_TRY(hipMalloc(&d, bytes));
+    HIP_TRY(hipMemcpyAsync(d, W, bytes, hipMemcpyHostToDevice, g_stream));
+    g_w[g_nw].host = W;
+    g_w[g_nw].bytes = bytes;
+    g_w[g_nw].fp = fp;
+    g_w[g_nw].dev = d;
+    g_nw++;
+    *out = d;
+    return 0;
+}
+
+/* Uncached weights share no staging buffer with activations: they get their
+ * own grow-only device buffer. */
+static dev_buf g_wtmp;
+static int weights_uncached(const void *W, size_t bytes, const void **out)
+{
+    if (g_wtmp.cap < bytes) {
+        if (g_wtmp.dev) {
+            HIP_TRY(hipStreamSynchronize(g_stream));
+            HIP_TRY(hipFree(g_wtmp.dev));
+            g_wtmp.dev = NULL;
+            g_wtmp.cap = 0;
+        }
+        HIP_TRY(hipMalloc(&g_wtmp.dev, bytes));
+        g_wtmp.cap = bytes;
+    }
+    HIP_TRY(hipMemcpyAsync(g_wtmp.dev, W, bytes, hipMemcpyHostToDevice, g_stream));
+    *out = g_wtmp.dev;
+    return 0;
+}
+
+static int weights_resolve(const void *W, size_t bytes, const void **out)
+{
+    if (is_device_ptr(W)) {
+        *out = W;
+        return 0;
+    }
+    if (!g_cache_on) return weights_uncached(W, bytes, out);
+    return weights_lookup(W, bytes, out);
+}
+
+int ckq_weights_register(const void *W, size_t bytes)
+{
+    if (!W || bytes == 0) return CKQ_EINVAL;
+    pthread_mutex_lock(&g_mu);
+    int rc = init_locked();
+    const void *d;
+    if (rc == 0) rc = weights_lookup(W, bytes, &d);
+    if (rc == 0) {
+        hipError_t e = hipStreamSynchronize(g_stream);
+        if (e != hipSuccess) rc = fail((int)e, "hipStreamSynchronize");
+    }
+    pthread_mutex_unlock(&g_mu);
+    return rc;
+}
+
+static void drop_entry(size_t i)
+{
+    (void)hipStreamSynchronize(g_stream);
+    (void)hipFree(g_w[i].dev);
+    g_w[i] = g_w[g_nw - 1];
+    g_nw--;
+}
+
+void ckq_weights_invalidate(const void *W)
+{
+    pthread_mutex_lock(&g_mu);
+    for (size_t i = 0; i < g_nw;) {
+        if (g_w[i].host == W) drop_entry(i);
+        else ++i;
+    }
+    pthread_mutex_unlock(&g_mu);
+}
+
+void ckq_weights_clear(void)
+{
+    pthread_mutex_lock(&g_mu);
+    while (g_nw) drop_entry(g_nw - 1);
+    pthread_mutex_unlock(&g_mu);
+}
+
+void ckq_weights_set_cache(int enabled)
+{
+    pthread_mutex_lock(&g_mu);
+    g_cache_on = enabled != 0;
+    pthread_mutex_unlock(&g_mu);
+}
+
+void ckq_set_parallel_whole(int enabled)
+{
+    pthread_mutex_lock(&g_mu);
+    g_parallel_whole = enabled != 0;
+    pthread_mutex_unlock(&g_mu);
+}
+
+/* ------------------------------------------------------------------------ */
+/* Shapes                                                                    */
+/* ------------------------------------------------------------------------ */
+
+static int fmt_block_elems(int fmt) { return (fmt == CKQ_FMT_Q8_0 || fmt == CKQ_KERNEL_Q80_F32) ? 32 : 256; }
+
+static size_t weight_row_bytes(int fmt, int K)
+{
+    return ckq_row_bytes(fmt == CKQ_KERNEL_Q80_F32 ? CKQ_FMT_Q8_0 : fmt, K);
+}
+
+static size_t act_row_bytes(int fmt, int K)
+{
+    if (fmt == CKQ_KERNEL_Q80_F32) return (size_t)K * 4;
+    if (fmt == CKQ_FMT_Q8_0) return ckq_row_bytes(CKQ_FMT_Q8_0, K);
+    return ckq_row_bytes(CKQ_FMT_Q8_K, K);
+}
+
+/* ------------------------------------------------------------------------ */
+/* Core host-pointer matmul                                                  */
+/* ------------------------------------------------------------------------ */
+
+/*
+ * C[t*ldc + n] = dot(B[n], A[t]) (+bias[n]) for n in [row0,row1), t < ntok,
+ * any mix of host and device pointers; synchronous.
+ */
+static void matmul_locked(int fmt, const void *A, const void *B, const float *bias, float *C,
+                          int ntok, int nrows, int K, long ldc, int row0, int row1)
+{
+    do {
+        if (init_locked()) break;
+        const void *dB, *dA, *dbias = NULL;
+        if (weights_resolve(B, (size_t)nrows * weight_row_bytes(fmt, K), &dB)) break;
+        if (stage_in(BUF_X, A, (size_t)ntok * act_row_bytes(fmt, K), &dA)) break;
+        if (bias && stage_in(BUF_BIAS, bias, (size_t)nrows * sizeof(float), &dbias)) break;
+        const int c_on_dev = is_device_ptr(C);
+        float *dC = C;
+        long   ld = ldc;
+        if (!c_on_dev) {
+            void *t;
+            ld = row1 - row0; /* compact staging: only the computed rows */
+            if (buf_reserve(BUF_Y, (size_t)ntok * (size_t)ld * sizeof(float), &t)) break;
+            dC = (float *)t - row0; /* kernel indexes with absolute rows */
+        }
+        int rc = ckq_launch_gemv(fmt, dC, dB, dA, (const float *)dbias, nrows, K, ntok, ld, row0, row1, NULL, g_stream);
+        if (rc) { fail(rc, "ckq_launch_gemv"); break; }
+        if (!c_on_dev) {
+            hipError_t e = hipSuccess;
+            const size_t w = (size_t)(row1 - row0) * sizeof(float);
+            if (ldc == ld || ntok == 1) {
+                for (int t = 0; t < ntok && e == hipSuccess; ++t)
+                    e = hipMemcpyAsync(C + (size_t)t * ldc + row0, (float *)g_buf[BUF_Y].dev + (size_t)t * ld, w,
+                                       hipMemcpyDeviceToHost, g_stream);
+            } else {
+                e = hipMemcpy2DAsync(C + row0, (size_t)ldc * sizeof(float), g_buf[BUF_Y].dev, (size_t)ld * sizeof(float),
+                                     w, (size_t)ntok, hipMemcpyDeviceToHost, g_stream);
+            }
+            if (e != hipSuccess) { fail((int)e, "copy result to host"); break; }
+        }
+        hipError_t e = hipStreamSynchronize(g_stream);
+        if (e != hipSuccess) fail((int)e, "hipStreamSynchronize");
+    } while (0);
+}
+
+static void host_matmul(int fmt, const void *A, const void *B, const float *bias, float *C,
+                        int ntok, int nrows, int K, long ldc, int row0, int row1)
+{
+    if (!A || !B || !C || ntok <= 0 || nrows <= 0 || K <= 0) return;
+    if (K % fmt_block_elems(fmt) != 0) return;
+    if (row0 < 0) row0 = 0;
+    if (row1 > nrows) row1 = nrows;
+    if (row0 >= row1) return;
+    pthread_mutex_lock(&g_mu);
+    matmul_locked(fmt, A, B, bias, C, ntok, nrows, K, ldc, row0, row1);
+    pthread_mutex_unlock(&g_mu);
+}
+
+/* Row range of thread ith of nth (reference: gemm_kernels_q4k_q8k.c:226-231). */
+static int split_rows(int M, int ith, int nth, int *r0, int *r1)
+{
+    if (ith < 0 || nth <= 0 || ith >= nth) return 0;
+    if (g_parallel_whole) {
+        if (ith != 0) return 0;
+        *r0 = 0;
+        *r1 = M;
+        return 1;
+    }
+    const int dr = (M + nth - 1) / nth;
+    *r0 = dr * ith;
+    *r1 = (*r0 + dr < M) ? *r0 + dr : M;
+    return *r0 < M;
+}
+
+static void host_gemv_split(int fmt, float *y, const void *W, const void *x, int M, int K, int ith, int nth)
+{
+    if (!y || !W || !x || M <= 0 || K <= 0) return;
+    int r0, r1;
+    if (!split_rows(M, ith, nth, &r0, &r1)) return;
+    host_matmul(fmt, x, W, NULL, y, 1, M, K, M, r0, r1);
+}
+
+/* fp32 [rows x k] -> quantized blocks, any pointer mix, synchronous. */
+static void host_quantize(int q8k, const float *x, void *y, int rows, int k)
+{
+    if (!x || !y || rows <= 0 || k <= 0) return;
+    const int be = q8k ? 256 : 32;
+    if (k % be) return; /* the reference asserts; a release build would write nothing sensible */
+    const size_t in_bytes = (size_t)rows * k * 4;
+    const size_t out_bytes = (size_t)rows * ckq_row_bytes(q8k ? CKQ_FMT_Q8_K : CKQ_FMT_Q8_0, k);
+    pthread_mutex_lock(&g_mu);
+    do {
+        if (init_locked()) break;
+        const void *dx;
+        if (stage_in(BUF_X, x, in_bytes, &dx)) break;
+        const int y_on_dev = is_device_ptr(y);
+        void *dy = y;
+        if (!y_on_dev && buf_reserve(BUF_Y, out_bytes, &dy)) break;
+        int rc = q8k ? ckq_launch_quantize_q8_k((const float *)dx, dy, rows, k, g_stream)
+                     : ckq_launch_quantize_q8_0((const float *)dx, dy, rows, k, g_stream);
+        if (rc) { fail(rc, "quantize launch"); break; }
+        if (!y_on_dev) {
+            hipError_t e = hipMemcpyAsync(y, dy, out_bytes, hipMemcpyDeviceToHost, g_stream);
+            if (e != hipSuccess) { fail((int)e, "copy result to host"); break; }
+        }
+        hipError_t e = hipStreamSynchronize(g_stream);
+        if (e != hipSuccess) fail((int)e, "hipStreamSynchronize");
+    } while (0);
+    pthread_mutex_unlock(&g_mu);
+}
+
+/* fp32 activations: quantize on the device, then the quantized kernel. */
+static void host_matmul_f32act(int fmt, const float *A, const void *B, const float *bias, float *C,
+                               int ntok, int nrows, int K, long ldc)
+{
+    if (!A || !B || !C || ntok <= 0 || nrows <= 0 || K <= 0) return;
+    const int q8k = fmt != CKQ_FMT_Q8_0;
+    if (K % (q8k ? 256 : 32)) return;
+    pthread_mutex_lock(&g_mu);
+    void *dq = NULL;
+    do {
+        if (init_locked()) break;
+        const void *dA;
+        if (stage_in(BUF_X, A, (size_t)ntok * K * 4, &dA)) break;
+        if (buf_reserve(BUF_Q, (size_t)ntok * act_row_bytes(fmt, K), &dq)) break;
+        int rc = q8k ? ckq_launch_quantize_q8_k((const float *)dA, dq, ntok, K, g_stream)
+                     : ckq_launch_quantize_q8_0((const float *)dA, dq, ntok, K, g_stream);
+        if (rc) { fail(rc, "quantize launch"); break; }
+        /* dq is a device pointer, so the second stage uses it in place; work
+         * on one stream runs in order. */
+        matmul_locked(fmt, dq, B, bias, C, ntok, nrows, K, ldc, 0, nrows);
+    } while (0);
+    pthread_mutex_unlock(&g_mu);
+}
+
+/* ------------------------------------------------------------------------ */
+/* Part 1: drop-in symbols                                                   */
+/* ------------------------------------------------------------------------ */
+
+void quantize_row_q8_k(const float *x, void *y, int k) { host_quantize(1, x, y, 1, k); }
+void quantize_batch_q8_k(const float *x, void *y, int num_rows, int k) { host_quantize(1, x, y, num_rows, k); }
+void quantize_row_q8_0(const float *x, void *y, int k) { host_quantize(0, x, y, 1, k); }
+void quantize_batch_q8_0(const float *x, void *y, int num_rows, int k) { host_quantize(0, x, y, num_rows, k); }
+
+#define DEFINE_GEMV_FAMILY(NAME, FMT)                                                                         \
+    void gemv_##NAME(float *y, const void *W, const void *x_q8, int M, int K)                                \
+    {                                                                                                         \
+        host_matmul(FMT, x_q8, W, NULL, y, 1, M, K, M, 0, M);                                                \
+    }                                                                                                         \
+    void gemv_##NAME##_parallel(float *y, const void *W, const void *x_q8, int M, int K, int ith, int nth)    \
+    {                                                                                                         \
+        host_gemv_split(FMT, y, W, x_q8, M, K, ith, nth);                                                    \
+    }                                                                                                         \
+    void gemv_##NAME##_parallel_simd(float *y, const void *W, const void *x_q8, int M, int K, int ith, int nth) \
+    {                                                                                                         \
+        host_gemv_split(FMT, y, W, x_q8, M, K, ith, nth);                                                    \
+    }
+
+DEFINE_GEMV_FAMILY(q4_k_q8_k, CKQ_FMT_Q4_K)
+DEFINE_GEMV_FAMILY(q6_k_q8_k, CKQ_FMT_Q6_K)
+DEFINE_GEMV_FAMILY(q8_0_q8_0, CKQ_FMT_Q8_0)
+
+void gemv_q4_k_q8_k_ref(float *y, const void *W, const void *x_q8, int M, int K)
+{
+    host_matmul(CKQ_FMT_Q4_K, x_q8, W, NULL, y, 1, M, K, M, 0, M);
+}
+
+void gemm_q4_k_q8_k(float *Y, const void *W, const void *X_q8, int M, int N, int K)
+{
+    host_matmul(CKQ_FMT_Q4_K, X_q8, W, NULL, Y, N, M, K, M, 0, M);
+}
+
+void gemm_nt_q4_k_q8_k(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K)
+{
+    host_matmul(CKQ_FMT_Q4_K, A_q8, B, bias, C, M, N, K, N, 0, N);
+}
+
+void gemv_q5_k_q8_k(float *y, const void *W, const void *x_q8, int M, int K)
+{
+    host_matmul(CKQ_FMT_Q5_K, x_q8, W, NULL, y, 1, M, K, M, 0, M);
+}
+
+void gemm_nt_q5_k_q8_k(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K)
+{
+    host_matmul(CKQ_FMT_Q5_K, A_q8, B, bias, C, M, N, K, N, 0, N);
+}
+
+void gemv_q5_k(float *y, const void *W, const float *x, int M, int K)
+{
+    host_matmul_f32act(CKQ_FMT_Q5_K, x, W, NULL, y, 1, M, K, M);
+}
+
+void gemm_nt_q5_k(const float *A, const void *B, const float *bias, float *C, int M, int N, int K)
+{
+    host_matmul_f32act(CKQ_FMT_Q5_K, A, B, bias, C, M, N, K, N);
+}
+
+void vec_dot_q6_k_q8_k(int n, float *s, const void *vx, const void *vy)
+{
+    if (!s || !vx || !vy || n <= 0) return;
+    host_matmul(CKQ_FMT_Q6_K, vy, vx, NULL, s, 1, 1, n, 1, 0, 1);
+}
+
+void gemm_q6_k_q8_k(float *Y, const void *W, const void *X_q8, int M, int N, int K)
+{
+    host_matmul(CKQ_FMT_Q6_K, X_q8, W, NULL, Y, N, M, K, M, 0, M);
+}
+
+void gemm_nt_q6_k_q8_k(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K)
+{
+    host_matmul(CKQ_FMT_Q6_K, A_q8, B, bias, C, M, N, K, N, 0, N);
+}
+
+void vec_dot_q8_0_q8_0(int n, float *s, const void *vx, const void *vy)
+{
+    if (!s || !vx || !vy || n <= 0) return;
+    host_matmul(CKQ_FMT_Q8_0, vy, vx, NULL, s, 1, 1, n, 1, 0, 1);
+}
+
+void gemv_q8_0(float *y, const void *W, const float *x, int M, int K)
+{
+    host_matmul(CKQ_KERNEL_Q80_F32, x, W, NULL, y, 1, M, K, M, 0, M);
+}
+
+void gemm_nt_q8_0_q8_0(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K)
+{
+    host_matmul(CKQ_FMT_Q8_0, A_q8, B, bias, C, M, N, K, N, 0, N);
+}
+
+/* Parity-test wrappers (reference: src/ck_parity_api.c). */
+void ck_test_quantize_q8_k(const float *src, void *dst, int n) { quantize_row_q8_k(src, dst, n); }
+
+void ck_test_gemv_q4_k(const void *w, const float *in, float *out, int cols)
+{
+    host_matmul_f32act(CKQ_FMT_Q4_K, in, w, NULL, out, 1, 1, cols, 1);
+}
+
+void ck_test_gemv_q6_k(const void *w, const float *in, float *out, int cols)
+{
+    host_matmul_f32act(CKQ_FMT_Q6_K, in, w, NULL, out, 1, 1, cols, 1);
+}
+
+void ck_test_gemv_q8_0(const void *w, const float *in, float *out, int rows, int cols)
+{
+    host_matmul_f32act(CKQ_FMT_Q8_0, in, w, NULL, out, 1, rows, cols, rows);
+}
+
+void ck_test_gemv_q8_0_q8_0(const void *w, const float *in, float *out, int rows, int cols)
+{
+    host_matmul_f32act(CKQ_FMT_Q8_0, in, w, NULL, out, 1, rows, cols, rows);
+}
+
+void ck_test_vec_dot_q8_0_q8_0(const void *w, const void *in_q8, float *out, int cols)
+{
+    vec_dot_q8_0_q8_0(cols, out, w, in_q8);
+}
+
+void ck_test_gemm_q4_k(const void *w, const float *in, float *out, int rows, int cols, int n_tokens)
+{
+    host_matmul_f32act(CKQ_FMT_Q4_K, in, w, NULL, out, n_tokens, rows, cols, rows);
+}
+
+void ck_test_gemm_q6_k(const void *w, const float *in, float *out, int rows, int cols, int n_tokens)
+{
+    host_matmul_f32act(CKQ_FMT_Q6_K, in, w, NULL, out, n_tokens, rows, cols, rows);
+}
+
+void ck_test_gemm_q8_0(const void *w, const float *in, float *out, int rows, int cols, int n_tokens)
+{
+    host_matmul_f32act(CKQ_FMT_Q8_0, in, w, NULL, out, n_tokens, rows, cols, rows);
+}
+
+int ck_get_block_q4_k_size(void) { return CKQ_BLOCK_Q4_K_SIZE; }
+int ck_get_block_q6_k_size(void) { return CKQ_BLOCK_Q6_K_SIZE; }
+int ck_get_block_q8_k_size(void) { return CKQ_BLOCK_Q8_K_SIZE; }
+int ck_get_qk_k(void) { return CKQ_QK_K; }
+
+/* ------------------------------------------------------------------------ */
+/* Part 2: device-resident entry points                                      */
+/* ------------------------------------------------------------------------ */
+
+int ckq_quantize_q8_k_dev(const float *x, void *y, int num_rows, int k, void *stream)
+{
+    return ckq_launch_quantize_q8_k(x, y, num_rows, k, stream);
+}
+
+int ckq_quantize_q8_0_dev(const float *x, void *y, int num_rows, int k, void *stream)
+{
+    return ckq_launch_quantize_q8_0(x, y, num_rows, k, stream);
+}
+
+int ckq_gemm_nt_dev(int fmt, const void *A_q8, const void *B, const float *bias, float *C,
+                    int M, int N, int K, long ldc, void *stream)
+{
+    if (fmt != CKQ_FMT_Q4_K && fmt != CKQ_FMT_Q5_K && fmt != CKQ_FMT_Q6_K && fmt != CKQ_FMT_Q8_0) return CKQ_EFORMAT;
+    return ckq_launch_gemv(fmt, C, B, A_q8, bias, N, K, M, ldc, 0, N, NULL, stream);
+}
+
+#define DEFINE_DEV(NAME, FMT)                                                                                   \
+    int ckq_gemv_##NAME##_dev(float *y, const void *W, const void *x_q8, int M, int K, void *stream)            \
+    {                                                                                                           \
+        return ckq_launch_gemv(FMT, y, W, x_q8, NULL, M, K, 1, M, 0, M, NULL, stream);                          \
+    }                                                                                                           \
+    int ckq_gemm_nt_##NAME##_dev(const void *A_q8, const void *B, const float *bias, float *C, int M, int N,    \
+                                 int K, void *stream)                                                           \
+    {                                                                                                           \
+        return ckq_launch_gemv(FMT, C, B, A_q8, bias, N, K, M, N, 0, N, NULL, stream);                          \
+    }
+
+DEFINE_DEV(q4_k_q8_k, CKQ_FMT_Q4_K)
+DEFINE_DEV(q5_k_q8_k, CKQ_FMT_Q5_K)
+DEFINE_DEV(q6_k_q8_k, CKQ_FMT_Q6_K)
+DEFINE_DEV(q8_0_q8_0, CKQ_FMT_Q8_0)
+
+int ckq_gemv_q8_0_dev(float *y, const void *W, const float *x, int M, int K, void *stream)
+{
+    return ckq_launch_gemv(CKQ_KERNEL_Q80_F32, y, W, x, NULL, M, K, 1, M, 0, M, NULL, stream);
+}
+
+int ckq_matmul_sequence_dev(const ckq_matmul_op *ops, int nops, int repeat, void *stream)
+{
+    if (!ops || nops <= 0 || repeat <= 0) return CKQ_EINVAL;
+    for (int r = 0; r < repeat; ++r)
+        for (int i = 0; i < nops; ++i) {
+            const ckq_matmul_op *o = &ops[i];
+            const int rc = ckq_gemm_nt_dev(o->fmt, o->A_q8, o->B, o->bias, o->C, o->M, o->N, o->K, o->ldc, stream);
+            if (rc) return rc;
+        }
+    return 0;
+}
+
+int ckq_subblock_dots_dev(int fmt, int32_t *out, const void *W, const void *x_q8, int M, int K, void *stream)
+{
+    if (!out) return CKQ_EINVAL;
+    if (fmt != CKQ_FMT_Q4_K && fmt != CKQ_FMT_Q5_K && fmt != CKQ_FMT_Q6_K && fmt != CKQ_FMT_Q8_0) return CKQ_EFORMAT;
+    return ckq_launch_gemv(fmt, NULL, W, x_q8, NULL, M, K, 1, M, 0, M, out, stream);
+}
+
+int ckq_copy_dev(void *dst, const void *src, size_t bytes, void *stream)
+{
+    return ckq_launch_copy(dst, src, bytes, stream);
+}

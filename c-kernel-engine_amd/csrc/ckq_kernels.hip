@@ -1,0 +1,322 @@
+/*
+ * ckq_kernels.hip - gfx950 kernels of the quantized dequant-dot path and their
+ * C launchers.
+ *
+ *   gemv_kernel<F,...>      weight rows x up to 8 activation rows (decode and
+ *                           small-batch prefill); weights are streamed once
+ *                           with 128-bit loads, unpacked in registers, dotted
+ *                           with v_dot4_i32_i8, reduced with DPP.
+ *   quantize_q8_k_kernel    fp32 -> Q8_K, bit-exact with the reference
+ *   quantize_q8_0_kernel    fp32 -> Q8_0, bit-exact with the reference
+ *   copy_kernel             plain streaming copy (counter calibration)
+ *
+ * wave64 only; every kernel is launched with 256-thread blocks.
+ */
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "ckq_blocks.h"
+#include "ckq_formats.cuh"
+#include "ckq_launch.h"
+
+/* ========================================================================= */
+/* GEMV                                                                       */
+/* ========================================================================= */
+
+struct GemvArgs {
+    float         *y;
+    const uint8_t *W;
+    const uint8_t *X;
+    const float   *bias;
+    int32_t       *sub;
+    int  nrows, npos, ntok, row0, row1, nsub_row;
+    long wrow, xrow, ldy;
+};
+
+/*
+ * One wave handles (64/LPR)*RPI weight rows: LPR lanes share a row, lane l of
+ * the group owns positions l, l+LPR, ... (PPL of them per pass).  All weight
+ * and activation loads of a pass are issued before anything is decoded, so a
+ * wave keeps RPI*PPL*(48..80) bytes per lane in flight; there is no loop over
+ * rows, the grid supplies the parallelism.  The fp32 partials are summed over
+ * the LPR lanes with a fixed DPP tree and the last lane of the group stores.
+ */
+template <class F, int LPR, int PPL, int MT, int RPI, bool DUMP>
+__global__ void __launch_bounds__(256) gemv_kernel(GemvArgs a)
+{
+    constexpr int SLOTS = 64 / LPR;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int slot = lane / LPR, l = lane % LPR;
+    const int wave_row = a.row0 + (blockIdx.x * 4 + wave) * (SLOTS * RPI);
+    if (wave_row >= a.row1) return;
+    const int rbase = wave_row + slot * RPI;
+    const int t0 = blockIdx.y * MT;
+
+    float acc[RPI][MT];
+#pragma unroll
+    for (int r = 0; r < RPI; ++r)
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc[r][t] = 0.0f;
+
+    for (int p0 = 0; p0 < a.npos; p0 += LPR * PPL) {
+        typename F::Wt  w[RPI][PPL];
+        typename F::Act act[MT][PPL];
+#pragma unroll
+        for (int p = 0; p < PPL; ++p) {
+            const int pos = min(p0 + p * LPR + l, a.npos - 1);
+#pragma unroll
+            for (int r = 0; r < RPI; ++r) {
+                const int row = min(rbase + r, a.row1 - 1);
+                F::load_w(w[r][p], a.W + (size_t)row * a.wrow, pos);
+            }
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                const int tok = min(t0 + t, a.ntok - 1);
+                F::load_act(act[t][p], a.X + (size_t)tok * a.xrow, pos);
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < PPL; ++p) {
+            const int  upos  = p0 + p * LPR + l;
+            const bool valid = upos < a.npos;
+            const int  pos   = min(upos, a.npos - 1);
+#pragma unroll
+            for (int r = 0; r < RPI; ++r) {
+                typename F::Dec dec;
+                F::decode(dec, w[r][p], pos);
+#pragma unroll
+                for (int t = 0; t < MT; ++t) {
+                    int sub[F::NSUB];
+                    const float v = F::dot(dec, act[t][p], sub);
+                    acc[r][t] += valid ? v : 0.0f;
+                    if (DUMP && t == 0 && valid && rbase + r < a.row1) {
+#pragma unroll
+                        for (int i = 0; i < F::NSUB; ++i)
+                            a.sub[(size_t)(rbase + r) * a.nsub_row + F::sub_index(pos, i)] = sub[i];
+                    }
+                }
+            }
+        }
+    }
+
+#pragma unroll
+    for (int r = 0; r < RPI; ++r)
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            const float s = group_sum<LPR>(acc[r][t]);
+            const int row = rbase + r, tok = t0 + t;
+            if (!DUMP && l == LPR - 1 && row < a.row1 && tok < a.ntok)
+                a.y[(size_t)tok * a.ldy + row] = a.bias ? s + a.bias[row] : s;
+        }
+}
+
+template <class F, int LPR, int PPL, int MT, int RPI, bool DUMP>
+static int launch_one(const GemvArgs &a, hipStream_t s)
+{
+    constexpr int rows_per_block = 4 * (64 / LPR) * RPI;
+    const int nr = a.row1 - a.row0;
+    dim3 grid((nr + rows_per_block - 1) / rows_per_block, (a.ntok + MT - 1) / MT);
+    hipLaunchKernelGGL((gemv_kernel<F, LPR, PPL, MT, RPI, DUMP>), grid, dim3(256), 0, s, a);
+    return (int)hipGetLastError();
+}
+
+/* Rows per wave-slot for each token tile: more rows in flight for the
+ * bandwidth-bound single-token case, fewer as the activation tile grows. */
+template <int MT> struct RowsPer { static constexpr int v = MT == 1 ? 4 : (MT <= 4 ? 2 : 1); };
+
+template <class F, int LPR, int PPL>
+static int launch_mt(const GemvArgs &a, bool dump, int max_mt, hipStream_t s)
+{
+    if (dump) return launch_one<F, LPR, PPL, 1, 1, true>(a, s);
+    if (a.ntok == 1 || max_mt == 1) return launch_one<F, LPR, PPL, 1, RowsPer<1>::v, false>(a, s);
+    if (a.ntok == 2) return launch_one<F, LPR, PPL, 2, RowsPer<2>::v, false>(a, s);
+    if (a.ntok <= 4) return launch_one<F, LPR, PPL, 4, RowsPer<4>::v, false>(a, s);
+    return launch_one<F, LPR, PPL, 8, RowsPer<8>::v, false>(a, s);
+}
+
+template <class F>
+static int launch_fmt(const GemvArgs &a, bool dump, int max_mt, hipStream_t s)
+{
+    const int np = a.npos;
+    if (np <= 8)  return launch_mt<F, 8, 1>(a, dump, max_mt, s);
+    if (np <= 16) return launch_mt<F, 16, 1>(a, dump, max_mt, s);
+    if (np <= 32) return launch_mt<F, 32, 1>(a, dump, max_mt, s);
+    if (np <= 64) return launch_mt<F, 64, 1>(a, dump, max_mt, s);
+    if (np <= 128) return launch_mt<F, 64, 2>(a, dump, max_mt, s);
+    if (np <= 192) return launch_mt<F, 64, 3>(a, dump, max_mt, s);
+    return launch_mt<F, 64, 4>(a, dump, max_mt, s);   /* longer rows loop in passes of 256 positions */
+}
+
+extern "C" int ckq_launch_gemv(int fmt, float *y, const void *W, const void *X, const float *bias,
+                               int nrows, int K, int ntok, long ldy, int row0, int row1,
+                               int32_t *subdots, void *stream)
+{
+    if ((!y && !subdots) || !W || !X || nrows <= 0 || K <= 0 || ntok <= 0) return CKQ_EINVAL;
+    if (row0 < 0) row0 = 0;
+    if (row1 > nrows) row1 = nrows;
+    if (row0 >= row1) return 0;
+    if (subdots && ntok != 1) return CKQ_EINVAL;
+    GemvArgs a;
+    a.y = y; a.W = (const uint8_t *)W; a.X = (const uint8_t *)X; a.bias = bias; a.sub = subdots;
+    a.nrows = nrows; a.ntok = ntok; a.row0 = row0; a.row1 = row1; a.ldy = ldy;
+    hipStream_t s = (hipStream_t)stream;
+    const bool dump = subdots != nullptr;
+    switch (fmt) {
+    case CKQ_FMT_Q4_K:
+        if (K % 256) return CKQ_ESHAPE;
+        a.npos = K / 64; a.wrow = (long)(K / 256) * 144; a.xrow = (long)(K / 256) * 292; a.nsub_row = K / 32;
+        return launch_fmt<FmtQ4K>(a, dump, 8, s);
+    case CKQ_FMT_Q5_K:
+        if (K % 256) return CKQ_ESHAPE;
+        a.npos = K / 64; a.wrow = (long)(K / 256) * 176; a.xrow = (long)(K / 256) * 292; a.nsub_row = K / 32;
+        return launch_fmt<FmtQ5K>(a, dump, 8, s);
+    case CKQ_FMT_Q6_K:
+        if (K % 256) return CKQ_ESHAPE;
+        a.npos = K / 64; a.wrow = (long)(K / 256) * 210; a.xrow = (long)(K / 256) * 292; a.nsub_row = K / 16;
+        return launch_fmt<FmtQ6K>(a, dump, 8, s);
+    case CKQ_FMT_Q8_0:
+        if (K % 32) return CKQ_ESHAPE;
+        a.npos = K / 32; a.wrow = (long)(K / 32) * 34; a.xrow = (long)(K / 32) * 34; a.nsub_row = K / 32;
+        return launch_fmt<FmtQ80>(a, dump, 8, s);
+    case CKQ_KERNEL_Q80_F32:
+        if (K % 32) return CKQ_ESHAPE;
+        if (dump) return CKQ_EINVAL;
+        a.npos = K / 32; a.wrow = (long)(K / 32) * 34; a.xrow = (long)K * 4; a.nsub_row = K / 32;
+        return launch_fmt<FmtQ80F32>(a, false, 1, s);
+    default:
+        return CKQ_EFORMAT;
+    }
+}
+
+/* ========================================================================= */
+/* Activation quantizers                                                      */
+/* ========================================================================= */
+
+/* x86 cvtps2dq + saturating packs: round to nearest even, NaN -> -128. */
+__device__ __forceinline__ int rne_sat_i8(float p)
+{
+    if (p != p) return -128;
+    const float r = __builtin_rintf(p);
+    return (int)fminf(fmaxf(r, -128.0f), 127.0f);
+}
+
+/*
+ * fp32 -> Q8_K, one wave per 256-element block, lane l owns elements
+ * 4l..4l+3 (reference: quantize_row_q8_k_sse.c:22-82).  The scale comes from
+ * the FIRST element with the largest magnitude, sign kept; iscale = -127/max
+ * with IEEE division; each product is rounded to fp32 and then to the nearest
+ * even integer; d = 1/iscale.
+ */
+__global__ void __launch_bounds__(256) quantize_q8_k_kernel(const float *__restrict__ x, uint8_t *__restrict__ y,
+                                                            long nblocks)
+{
+    const int lane = threadIdx.x & 63;
+    const long blk = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (blk >= nblocks) return;
+    const float4 v = reinterpret_cast<const float4 *>(x + blk * 256)[lane];
+    const float e[4] = {v.x, v.y, v.z, v.w};
+
+    /* first-largest |x| inside the lane, then across lanes (lower index wins ties) */
+    float amax = 0.0f, smax = 0.0f;
+    int idx = 4 * lane;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float ax = fabsf(e[i]);
+        if (ax > amax) { amax = ax; smax = e[i]; idx = 4 * lane + i; }
+    }
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const float oa = __shfl_xor(amax, off), os = __shfl_xor(smax, off);
+        const int   oi = __shfl_xor(idx, off);
+        if (oa > amax || (oa == amax && oi < idx)) { amax = oa; smax = os; idx = oi; }
+    }
+
+    uint8_t *out = y + blk * 292;
+    if (amax == 0.0f) {
+        /* 292 bytes of zeros: d, qs, bsums */
+        reinterpret_cast<u32 *>(out)[lane] = 0;
+        if (lane < 9) reinterpret_cast<u32 *>(out)[64 + lane] = 0;
+        return;
+    }
+    const float iscale = -127.0f / smax;
+    int q[4], s = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        q[i] = rne_sat_i8(__fmul_rn(e[i], iscale));
+        s += q[i];
+    }
+    const u32 packed = (u32)(q[0] & 0xff) | ((u32)(q[1] & 0xff) << 8) | ((u32)(q[2] & 0xff) << 16) | ((u32)(q[3] & 0xff) << 24);
+    reinterpret_cast<u32 *>(out + 4)[lane] = packed;
+    s = group_sum<4>(s);                       /* 16 consecutive elements = 4 lanes */
+    if ((lane & 3) == 3) reinterpret_cast<int16_t *>(out + 260)[lane >> 2] = (int16_t)s;
+    if (lane == 0) *reinterpret_cast<float *>(out) = 1.0f / iscale;
+}
+
+/*
+ * fp32 -> Q8_0, eight lanes per 32-element block (reference:
+ * gemm_kernels_q8_0.c:70-146).  d = amax/127 stored as fp16 (RNE);
+ * id = amax ? 127/amax : 0; q = RNE(x*id) saturated.
+ */
+__global__ void __launch_bounds__(256) quantize_q8_0_kernel(const float *__restrict__ x, uint8_t *__restrict__ y,
+                                                            long nblocks)
+{
+    const long t = (long)blockIdx.x * 256 + threadIdx.x;
+    const long blk = t >> 3;
+    const int  j = (int)(t & 7);
+    const bool live = blk < nblocks;
+    const long b = live ? blk : nblocks - 1;
+    const float4 v = reinterpret_cast<const float4 *>(x + b * 32)[j];
+    const float e[4] = {v.x, v.y, v.z, v.w};
+    float amax = fmaxf(fmaxf(fabsf(e[0]), fabsf(e[1])), fmaxf(fabsf(e[2]), fabsf(e[3])));
+#pragma unroll
+    for (int off = 1; off < 8; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
+    const float d  = amax / 127.0f;
+    const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
+    int q[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) q[i] = rne_sat_i8(__fmul_rn(e[i], id));
+    if (!live) return;
+    uint8_t *out = y + b * 34;
+    uint16_t *o16 = reinterpret_cast<uint16_t *>(out + 2 + 4 * j);   /* 2-byte aligned */
+    o16[0] = (uint16_t)((q[0] & 0xff) | ((q[1] & 0xff) << 8));
+    o16[1] = (uint16_t)((q[2] & 0xff) | ((q[3] & 0xff) << 8));
+    if (j == 0) *reinterpret_cast<uint16_t *>(out) = __builtin_bit_cast(uint16_t, (_Float16)d);
+}
+
+extern "C" int ckq_launch_quantize_q8_k(const float *x, void *y, int rows, int k, void *stream)
+{
+    if (!x || !y || rows <= 0 || k <= 0) return CKQ_EINVAL;
+    if (k % 256) return CKQ_ESHAPE;
+    const long nblocks = (long)rows * (k / 256);
+    hipLaunchKernelGGL(quantize_q8_k_kernel, dim3((unsigned)((nblocks + 3) / 4)), dim3(256), 0, (hipStream_t)stream,
+                       x, (uint8_t *)y, nblocks);
+    return (int)hipGetLastError();
+}
+
+extern "C" int ckq_launch_quantize_q8_0(const float *x, void *y, int rows, int k, void *stream)
+{
+    if (!x || !y || rows <= 0 || k <= 0) return CKQ_EINVAL;
+    if (k % 32) return CKQ_ESHAPE;
+    const long nblocks = (long)rows * (k / 32);
+    hipLaunchKernelGGL(quantize_q8_0_kernel, dim3((unsigned)((nblocks * 8 + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, x, (uint8_t *)y, nblocks);
+    return (int)hipGetLastError();
+}
+
+/* ========================================================================= */
+/* Streaming copy                                                             */
+/* ========================================================================= */
+__global__ void __launch_bounds__(256) copy_kernel(uint4 *__restrict__ dst, const uint4 *__restrict__ src, size_t n16)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n16) dst[i] = src[i];
+}
+
+extern "C" int ckq_launch_copy(void *dst, const void *src, size_t bytes, void *stream)
+{
+    if (!dst || !src || bytes == 0 || (bytes & 15)) return CKQ_EINVAL;
+    const size_t n16 = bytes / 16;
+    hipLaunchKernelGGL(copy_kernel, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (uint4 *)dst, (const uint4 *)src, n16);
+    return (int)hipGetLastError();
+}

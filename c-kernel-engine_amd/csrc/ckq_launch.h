@@ -1,0 +1,48 @@
+/*
+ * ckq_launch.h - C interface between the host layer (plain C) and the HIP
+ * translation unit.  Every function takes DEVICE pointers and enqueues work on
+ * `stream` (a hipStream_t passed as void*; NULL = the null stream); none of
+ * them synchronizes.  Return value: 0 on success, a negative CKQ_E* code for a
+ * rejected argument, or a positive hipError_t.
+ */
+#ifndef CKQ_LAUNCH_H
+#define CKQ_LAUNCH_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CKQ_EINVAL  (-1)  /* NULL pointer / non-positive dimension */
+#define CKQ_ESHAPE  (-2)  /* K not a multiple of the block size */
+#define CKQ_EFORMAT (-3)  /* unknown format tag */
+
+/* Weight-format tags as in ckq_blocks.h, plus the fp32-activation variant. */
+#define CKQ_KERNEL_Q80_F32 16
+
+/*
+ * y[t*ldy + row] = dot(W[row], X[t]) (+ bias[row]) for row < nrows, t < ntok.
+ * W: nrows rows of K elements in `fmt` blocks; X: ntok activation rows
+ * (Q8_K, or Q8_0 / fp32 for the Q8_0 weight kernels).
+ * `row0`/`row1` restrict the computed rows to [row0,row1) (thread-split entry
+ * points); outputs outside the range are not touched.
+ * `subdots`, when non-NULL (ntok must be 1), receives the raw integer
+ * sub-block dots: nrows x (K/blk x per-block count) int32.
+ */
+int ckq_launch_gemv(int fmt, float *y, const void *W, const void *X, const float *bias,
+                    int nrows, int K, int ntok, long ldy, int row0, int row1,
+                    int32_t *subdots, void *stream);
+
+/* fp32 [rows x k] -> Q8_K / Q8_0 blocks, row-major. */
+int ckq_launch_quantize_q8_k(const float *x, void *y, int rows, int k, void *stream);
+int ckq_launch_quantize_q8_0(const float *x, void *y, int rows, int k, void *stream);
+
+/* Plain device copy kernel (calibration of the memory counters / roofline). */
+int ckq_launch_copy(void *dst, const void *src, size_t bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,123 @@
+"""NumPy / torch front-ends over the C ABI, shaped like the calls the
+reference's parity scripts make (ctypes into ck_test_* and the kernel symbols,
+e.g. unittest/test_q4_k_q8_k_matvec.py:93-132, unittest/test_parallel_gemv.py:112-170).
+
+Host functions take NumPy arrays and go through the drop-in (host-pointer)
+symbols; `dev_*` functions take torch CUDA tensors and go through the
+device-resident entry points on torch's current stream."""
+import ctypes
+
+import numpy as np
+
+from .api import BLOCK_ELEMS, FMT, MatmulOp, check, lib, row_bytes
+
+_vp = ctypes.c_void_p
+
+
+def _p(a):
+    if a is None:
+        return None
+    assert a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(_vp)
+
+
+def act_format(wfmt):
+    return "q8_0" if wfmt == "q8_0" else "q8_k"
+
+
+# ---- host-pointer (drop-in) path ------------------------------------------------
+
+def quantize(x, fmt="q8_k", rows=1):
+    """fp32 [rows*k] -> Q8_K / Q8_0 bytes via quantize_batch_*."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    k = x.size // rows
+    out = np.zeros(rows * row_bytes(fmt, k), dtype=np.uint8)
+    fn = lib().quantize_batch_q8_k if fmt == "q8_k" else lib().quantize_batch_q8_0
+    fn(_p(x), _p(out), rows, k)
+    return out
+
+
+_GEMV = {"q4_k": "gemv_q4_k_q8_k", "q5_k": "gemv_q5_k_q8_k", "q6_k": "gemv_q6_k_q8_k", "q8_0": "gemv_q8_0_q8_0"}
+_GEMM_NT = {"q4_k": "gemm_nt_q4_k_q8_k", "q5_k": "gemm_nt_q5_k_q8_k", "q6_k": "gemm_nt_q6_k_q8_k",
+            "q8_0": "gemm_nt_q8_0_q8_0"}
+
+
+def gemv(fmt, W, x_q8, M, K, name=None):
+    y = np.zeros(M, dtype=np.float32)
+    getattr(lib(), name or _GEMV[fmt])(_p(y), _p(W), _p(x_q8), M, K)
+    return y
+
+
+def gemv_parallel(fmt, W, x_q8, M, K, nth, simd=True, y=None):
+    """Union over ith of the thread-split entry point."""
+    y = np.zeros(M, dtype=np.float32) if y is None else y
+    fn = getattr(lib(), _GEMV[fmt] + ("_parallel_simd" if simd else "_parallel"))
+    for ith in range(nth):
+        fn(_p(y), _p(W), _p(x_q8), M, K, ith, nth)
+    return y
+
+
+def gemm_nt(fmt, A_q8, B, bias, M, N, K):
+    c = np.zeros(M * N, dtype=np.float32)
+    getattr(lib(), _GEMM_NT[fmt])(_p(A_q8), _p(B), _p(bias), _p(c), M, N, K)
+    return c.reshape(M, N)
+
+
+# ---- device-resident path ---------------------------------------------------------
+
+def _stream():
+    import torch
+    return _vp(torch.cuda.current_stream().cuda_stream)
+
+
+def _dp(t):
+    return None if t is None else _vp(t.data_ptr())
+
+
+def to_device(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def dev_quantize(x_t, fmt="q8_k", rows=1):
+    import torch
+    k = x_t.numel() // rows
+    out = torch.empty(rows * row_bytes(fmt, k), dtype=torch.uint8, device=x_t.device)
+    fn = lib().ckq_quantize_q8_k_dev if fmt == "q8_k" else lib().ckq_quantize_q8_0_dev
+    check(fn(_dp(x_t), _dp(out), rows, k, _stream()), "quantize_dev")
+    return out
+
+
+def dev_gemm_nt(fmt, A_t, B_t, bias_t, M, N, K, out=None):
+    """C[M,N] on the device; M = 1 is the GEMV."""
+    import torch
+    c = out if out is not None else torch.empty(M * N, dtype=torch.float32, device=B_t.device)
+    check(lib().ckq_gemm_nt_dev(FMT[fmt], _dp(A_t), _dp(B_t), _dp(bias_t), _dp(c), M, N, K, N, _stream()),
+          "ckq_gemm_nt_dev")
+    return c.view(M, N)
+
+
+def dev_gemv_q8_0_f32(W_t, x_t, M, K):
+    import torch
+    y = torch.empty(M, dtype=torch.float32, device=W_t.device)
+    check(lib().ckq_gemv_q8_0_dev(_dp(y), _dp(W_t), _dp(x_t), M, K, _stream()), "ckq_gemv_q8_0_dev")
+    return y
+
+
+def dev_subblock_dots(fmt, W_t, x_t, M, K):
+    import torch
+    per = (K // 16) if fmt == "q6_k" else (K // 32)
+    out = torch.zeros(M * per, dtype=torch.int32, device=W_t.device)
+    check(lib().ckq_subblock_dots_dev(FMT[fmt], _dp(out), _dp(W_t), _dp(x_t), M, K, _stream()),
+          "ckq_subblock_dots_dev")
+    return out.view(M, per)
+
+
+def dev_matmul_sequence(ops, repeat=1):
+    """ops: list of (fmt, A_t, B_t, bias_t, C_t, M, N, K); enqueued back-to-back
+    `repeat` times by one C call (no Python between launches)."""
+    arr = (MatmulOp * len(ops))()
+    for i, (fmt, A_t, B_t, bias_t, C_t, M, N, K) in enumerate(ops):
+        arr[i] = MatmulOp(FMT[fmt], M, N, K, N, A_t.data_ptr(), B_t.data_ptr(),
+                          bias_t.data_ptr() if bias_t is not None else None, C_t.data_ptr())
+    check(lib().ckq_matmul_sequence_dev(ctypes.cast(arr, _vp), len(ops), repeat, _stream()), "ckq_matmul_sequence_dev")

@@ -1,0 +1,185 @@
+/*
+ * ckernel_quant_hip.h - C ABI of libckernel_quant_hip.so, the MI355X (gfx950)
+ * implementation of the C-Kernel-Engine quantized dequant-dot matmul path.
+ *
+ * Part 1 re-exports, with identical names, signatures, argument meaning and
+ * error behaviour, the reference's kernel symbols for this path, so a
+ * generated libmodel.so (or libck_parity.so users) can link against this
+ * library instead of the CPU kernels.  Pointers may be HOST pointers (as the
+ * reference passes them) or DEVICE pointers; host buffers are staged, weight
+ * matrices are uploaded once and kept resident (see ckq_weights_*).
+ * Like the reference: void return, NULL pointer or non-positive dimension
+ * returns without touching the output.
+ *
+ * Part 2 (`ckq_*_dev`) is the same arithmetic on device-resident buffers with
+ * an explicit stream and an int status; nothing is copied or synchronized.
+ *
+ * Naming trap kept from the reference: in gemv_* M = output rows, K = input
+ * width; in gemm_nt_* M = tokens, N = output rows; in gemm_*_q8_k(Y,W,X,M,N,K)
+ * M = output rows, N = tokens and Y[n*M + row].
+ */
+#ifndef CKERNEL_QUANT_HIP_H
+#define CKERNEL_QUANT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+#include "ckq_blocks.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ======================================================================== */
+/* Part 1: drop-in symbols (reference declarations: include/ckernel_engine.h */
+/* :192-363 and include/ckernel_quant.h:398-410)                             */
+/* ======================================================================== */
+
+/* fp32 -> Q8_K, k % 256 == 0.  Replaces src/kernels/gemm_kernels_q4k_q8k.c:109-119
+ * (dispatch) -> quantize_row_q8_k_sse.c:22-82.  Bit-exact. */
+void quantize_row_q8_k(const float *x, void *y, int k);
+/* Row loop, output stride (k/256)*292.  Replaces gemm_kernels_q8_0.c:221-239. */
+void quantize_batch_q8_k(const float *x, void *y, int num_rows, int k);
+/* fp32 -> Q8_0, k % 32 == 0.  Replaces gemm_kernels_q8_0.c:70-175.  Bit-exact. */
+void quantize_row_q8_0(const float *x, void *y, int k);
+/* Replaces gemm_kernels_q8_0.c:194-209. */
+void quantize_batch_q8_0(const float *x, void *y, int num_rows, int k);
+
+/* Q4_K x Q8_K.  Replace gemm_kernels_q4k_q8k.c:245-263 (dispatch), :183-200 (_ref). */
+void gemv_q4_k_q8_k(float *y, const void *W, const void *x_q8, int M, int K);
+void gemv_q4_k_q8_k_ref(float *y, const void *W, const void *x_q8, int M, int K);
+/* Thread-split variants: rows [ith*ceil(M/nth), ...) only.  Replace
+ * gemm_kernels_q4k_q8k.c:212-243 and gemm_kernels_q4k_avx.c:136-245. */
+void gemv_q4_k_q8_k_parallel(float *y, const void *W, const void *x_q8, int M, int K, int ith, int nth);
+void gemv_q4_k_q8_k_parallel_simd(float *y, const void *W, const void *x_q8, int M, int K, int ith, int nth);
+/* Y[n*M + row].  Replaces gemm_kernels_q4k_q8k.c:283-299. */
+void gemm_q4_k_q8_k(float *Y, const void *W, const void *X_q8, int M, int N, int K);
+/* C[m*N + n] (+bias[n]).  Replaces gemm_kernels_q4k_q8k.c:301-326. */
+void gemm_nt_q4_k_q8_k(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K);
+
+/* Q5_K.  Replace gemm_kernels_q5_k.c:436-456 (gemv_q5_k_q8_k), :458-479
+ * (gemm_nt_q5_k_q8_k), :481-498 (gemv_q5_k) and :500-521 (gemm_nt_q5_k).  The
+ * fp32 adapters quantize the activations to Q8_K first; K % 256 != 0 returns
+ * without writing (the reference's non-GGUF fp32 fallback is not provided). */
+void gemv_q5_k_q8_k(float *y, const void *W, const void *x_q8, int M, int K);
+void gemm_nt_q5_k_q8_k(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K);
+void gemv_q5_k(float *y, const void *W, const float *x, int M, int K);
+void gemm_nt_q5_k(const float *A, const void *B, const float *bias, float *C, int M, int N, int K);
+
+/* Q6_K x Q8_K.  Replace gemm_kernels_q6k_q8k.c:1032-1055 (vec_dot), :1060-1088
+ * (gemv), :1105-1197 (_parallel, _parallel_simd), :1209-1225 (gemm), :1243-1268
+ * (gemm_nt). */
+void vec_dot_q6_k_q8_k(int n, float *s, const void *vx, const void *vy);
+void gemv_q6_k_q8_k(float *y, const void *W, const void *x_q8, int M, int K);
+void gemv_q6_k_q8_k_parallel(float *y, const void *W, const void *x_q8, int M, int K, int ith, int nth);
+void gemv_q6_k_q8_k_parallel_simd(float *y, const void *W, const void *x_q8, int M, int K, int ith, int nth);
+void gemm_q6_k_q8_k(float *Y, const void *W, const void *X_q8, int M, int N, int K);
+void gemm_nt_q6_k_q8_k(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K);
+
+/* Q8_0.  Replace gemm_kernels_q8_0.c:1204-1219 (vec_dot), :1237-1251 (gemv
+ * q8_0 x q8_0), :1263-1343 (_parallel, _parallel_simd), :632-649 (gemv_q8_0,
+ * fp32 activations) and gemm_batch_int8.c:582-610 (gemm_nt_q8_0_q8_0). */
+void vec_dot_q8_0_q8_0(int n, float *s, const void *vx, const void *vy);
+void gemv_q8_0_q8_0(float *y, const void *W, const void *x_q8, int M, int K);
+void gemv_q8_0_q8_0_parallel(float *y, const void *W, const void *x_q8, int M, int K, int ith, int nth);
+void gemv_q8_0_q8_0_parallel_simd(float *y, const void *W, const void *x_q8, int M, int K, int ith, int nth);
+void gemv_q8_0(float *y, const void *W, const float *x, int M, int K);
+void gemm_nt_q8_0_q8_0(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K);
+
+/* Parity-test wrappers: fp32 input is quantized, then the kernel runs.
+ * Replace src/ck_parity_api.c:207-210 (quantize), :217-258 (gemv q4_k/q6_k),
+ * :288-360 (gemv q8_0), :397-400 (vec_dot), :411-503 (gemm) and the size
+ * getters of include/ck_parity_api.h:614-629. */
+void ck_test_quantize_q8_k(const float *src, void *dst, int n);
+void ck_test_gemv_q4_k(const void *weight_q4k, const float *input_f32, float *output, int cols);
+void ck_test_gemv_q6_k(const void *weight_q6k, const float *input_f32, float *output, int cols);
+void ck_test_gemv_q8_0(const void *weight_q8_0, const float *input_f32, float *output, int rows, int cols);
+void ck_test_gemv_q8_0_q8_0(const void *weight_q8_0, const float *input_f32, float *output, int rows, int cols);
+void ck_test_vec_dot_q8_0_q8_0(const void *weight_q8_0, const void *input_q8_0, float *output, int cols);
+void ck_test_gemm_q4_k(const void *weight_q4k, const float *input_f32, float *output, int rows, int cols, int n_tokens);
+void ck_test_gemm_q6_k(const void *weight_q6k, const float *input_f32, float *output, int rows, int cols, int n_tokens);
+void ck_test_gemm_q8_0(const void *weight_q8_0, const float *input_f32, float *output, int rows, int cols, int n_tokens);
+int  ck_get_block_q4_k_size(void);
+int  ck_get_block_q6_k_size(void);
+int  ck_get_block_q8_k_size(void);
+int  ck_get_qk_k(void);
+
+/* ======================================================================== */
+/* Part 2: device-resident entry points                                      */
+/* ======================================================================== */
+/* All pointers are device pointers; `stream` is a hipStream_t (NULL = null
+ * stream); work is enqueued, never synchronized.  Outputs must not overlap
+ * inputs.  Return 0, or a negative CKQ_E* / positive hipError_t code.
+ * Alignment: Q4_K/Q5_K weights and Q8_K activations 4 bytes, Q6_K/Q8_0 2
+ * bytes, fp32 inputs of the quantizers 16 bytes, other fp32 4 bytes. */
+
+int ckq_quantize_q8_k_dev(const float *x, void *y, int num_rows, int k, void *stream);
+int ckq_quantize_q8_0_dev(const float *x, void *y, int num_rows, int k, void *stream);
+
+/* Generic form: fmt is a ckq_format weight tag (activations Q8_0 for
+ * CKQ_FMT_Q8_0, Q8_K otherwise).  C[m*ldc + n] = dot(B[n], A[m]) (+bias[n]),
+ * m < M tokens, n < N rows.  M = 1 with ldc = N is the GEMV. */
+int ckq_gemm_nt_dev(int fmt, const void *A_q8, const void *B, const float *bias, float *C,
+                    int M, int N, int K, long ldc, void *stream);
+
+/* Named forms mirroring Part 1. */
+int ckq_gemv_q4_k_q8_k_dev(float *y, const void *W, const void *x_q8, int M, int K, void *stream);
+int ckq_gemv_q5_k_q8_k_dev(float *y, const void *W, const void *x_q8, int M, int K, void *stream);
+int ckq_gemv_q6_k_q8_k_dev(float *y, const void *W, const void *x_q8, int M, int K, void *stream);
+int ckq_gemv_q8_0_q8_0_dev(float *y, const void *W, const void *x_q8, int M, int K, void *stream);
+int ckq_gemv_q8_0_dev(float *y, const void *W, const float *x, int M, int K, void *stream);
+int ckq_gemm_nt_q4_k_q8_k_dev(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K, void *stream);
+int ckq_gemm_nt_q5_k_q8_k_dev(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K, void *stream);
+int ckq_gemm_nt_q6_k_q8_k_dev(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K, void *stream);
+int ckq_gemm_nt_q8_0_q8_0_dev(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K, void *stream);
+
+/* A list of matmuls enqueued back-to-back, the whole list `repeat` times: the
+ * per-token projection set of a decoder layer (Q/K/V/O, gate/up, down) is one
+ * such list.  Entry i computes C[m*ldc + n] as ckq_gemm_nt_dev does. */
+typedef struct {
+    int          fmt;    /* ckq_format weight tag */
+    int          M;      /* tokens */
+    int          N;      /* output rows */
+    int          K;      /* input width */
+    long         ldc;    /* output row stride (elements) */
+    const void  *A_q8;   /* activations, M rows */
+    const void  *B;      /* weights, N rows */
+    const float *bias;   /* N, or NULL */
+    float       *C;      /* M x ldc */
+} ckq_matmul_op;
+int ckq_matmul_sequence_dev(const ckq_matmul_op *ops, int nops, int repeat, void *stream);
+
+/* Raw integer sub-block dots of W (M rows) against one activation row, as the
+ * GEMV kernel computes them: out[row*(K/sub) + i], sub = 32 (Q4_K, Q5_K, Q8_0)
+ * or 16 (Q6_K, sum of (q-32)*q8).  For the bit-exactness tests. */
+int ckq_subblock_dots_dev(int fmt, int32_t *out, const void *W, const void *x_q8, int M, int K, void *stream);
+
+/* Streaming device copy of `bytes` (multiple of 16): calibration kernel for
+ * memory counters. */
+int ckq_copy_dev(void *dst, const void *src, size_t bytes, void *stream);
+
+/* ======================================================================== */
+/* Library control                                                           */
+/* ======================================================================== */
+/* Explicit initialisation (optional; every entry point initialises lazily).
+ * Returns 0 or a hipError_t; fails when no gfx950 device is usable. */
+int ckq_init(void);
+/* Wait for all work the host-pointer entry points enqueued. */
+int ckq_synchronize(void);
+/* Weight residency: host weight matrices are uploaded on first use and cached
+ * by (address, bytes, fingerprint).  register = upload now; invalidate = drop
+ * one; clear = drop all; set_cache(0) = upload on every call. */
+int  ckq_weights_register(const void *W, size_t bytes);
+void ckq_weights_invalidate(const void *W);
+void ckq_weights_clear(void);
+void ckq_weights_set_cache(int enabled);
+/* Thread-split entry points: 0 (default) = every call computes its own row
+ * range; 1 = the ith==0 call computes all rows and the others return. */
+void ckq_set_parallel_whole(int enabled);
+/* Last error of the calling process (0 = none) and its text. */
+int         ckq_last_error(void);
+const char *ckq_error_string(int code);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CKERNEL_QUANT_HIP_H */

@@ -1,0 +1,104 @@
+"""CPU checks of the C-ABI library: it loads, exports every declared symbol,
+and the host logic that needs no device (argument screening) behaves like the
+reference.  No kernel is launched here."""
+import ctypes
+import importlib
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+ckq = importlib.import_module("c-kernel-engine_amd")
+
+
+@pytest.fixture(scope="module")
+def L():
+    if not os.path.exists(ckq.lib_path()):
+        ckq.build()
+    return ckq.lib()
+
+
+def test_every_declared_symbol_is_exported(L):
+    names = ckq.declared_symbols()
+    assert len(names) >= 60
+    missing = [n for n in names if not hasattr(L, n)]
+    assert not missing, missing
+    # and the binding table covers the header
+    from importlib import import_module
+    api = import_module("c-kernel-engine_amd.api")
+    assert sorted(api._SIGS) == names
+
+
+def test_reference_symbol_names_present(L):
+    # the symbols a generated libmodel.so resolves for this path
+    # (reference include/ckernel_engine.h:192-363)
+    for n in ["quantize_row_q8_k", "quantize_batch_q8_k", "quantize_row_q8_0", "gemv_q4_k_q8_k",
+              "gemv_q4_k_q8_k_parallel_simd", "gemm_nt_q4_k_q8_k", "gemv_q5_k", "gemm_nt_q5_k",
+              "gemv_q6_k_q8_k", "gemv_q6_k_q8_k_parallel_simd", "gemm_nt_q6_k_q8_k", "gemv_q8_0_q8_0",
+              "gemv_q8_0", "gemm_nt_q8_0_q8_0", "vec_dot_q6_k_q8_k", "vec_dot_q8_0_q8_0"]:
+        assert hasattr(L, n)
+
+
+def test_block_size_getters(L):
+    assert L.ck_get_block_q4_k_size() == 144
+    assert L.ck_get_block_q6_k_size() == 210
+    assert L.ck_get_block_q8_k_size() == 292
+    assert L.ck_get_qk_k() == 256
+
+
+def test_bad_arguments_return_without_touching_output(L):
+    """NULL pointer or non-positive dimension: silent return
+    (reference gemm_kernels_q4k_q8k.c:188-190, :221-223, :307-312)."""
+    y = np.full(8, 7.0, np.float32)
+    w = np.zeros(8 * 144, np.uint8)
+    x = np.zeros(292, np.uint8)
+    p = lambda a: a.ctypes.data_as(ctypes.c_void_p)
+    L.gemv_q4_k_q8_k(p(y), None, p(x), 8, 256)
+    L.gemv_q4_k_q8_k(p(y), p(w), None, 8, 256)
+    L.gemv_q4_k_q8_k(p(y), p(w), p(x), 0, 256)
+    L.gemv_q4_k_q8_k(p(y), p(w), p(x), 8, -256)
+    L.gemv_q4_k_q8_k_parallel(p(y), p(w), p(x), 8, 256, 3, 3)   # ith >= nth
+    L.gemv_q4_k_q8_k_parallel(p(y), p(w), p(x), 8, 256, -1, 3)
+    L.gemv_q4_k_q8_k_parallel_simd(p(y), p(w), p(x), 8, 256, 0, 0)
+    L.gemv_q6_k_q8_k_parallel(p(y), p(w), p(x), 8, 256, 5, 2)
+    L.gemv_q8_0_q8_0_parallel_simd(p(y), p(w), p(x), 8, 256, 2, 2)
+    L.gemm_nt_q4_k_q8_k(None, p(w), None, p(y), 1, 8, 256)
+    L.gemm_nt_q6_k_q8_k(p(x), p(w), None, p(y), 1, 0, 256)
+    L.gemv_q5_k_q8_k(p(y), p(w), p(x), 8, 200)                   # K % 256 != 0 (gemm_kernels_q5_k.c:313-315)
+    L.vec_dot_q6_k_q8_k(0, p(y), p(w), p(x))
+    L.quantize_row_q8_k(None, p(x), 256)
+    L.quantize_row_q8_k(p(y), p(x), 0)
+    assert np.all(y == 7.0)
+    assert L.ckq_last_error() == 0
+
+
+def test_dev_entry_points_reject_bad_shapes(L):
+    # status codes come back before anything touches a device
+    one = ctypes.c_void_p(16)
+    assert L.ckq_gemv_q4_k_q8_k_dev(one, one, one, 4, 100, None) == -2
+    assert L.ckq_gemv_q4_k_q8_k_dev(None, one, one, 4, 256, None) == -1
+    assert L.ckq_gemm_nt_dev(9, one, one, None, one, 1, 4, 256, 4, None) == -3
+    assert L.ckq_quantize_q8_k_dev(one, one, 1, 100, None) == -2
+    assert L.ckq_quantize_q8_0_dev(one, one, 0, 32, None) == -1
+    assert b"multiple" in L.ckq_error_string(-2)
+
+
+def test_no_device_fails_loudly():
+    """Without a GPU a compute call must not succeed silently: the library
+    reports the HIP error and aborts the process."""
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    code = (
+        "import importlib, numpy as np, ctypes\n"
+        "ckq = importlib.import_module('c-kernel-engine_amd')\n"
+        "x = np.ones(256, np.float32); y = np.zeros(292, np.uint8)\n"
+        "ckq.lib().quantize_row_q8_k(x.ctypes.data_as(ctypes.c_void_p), y.ctypes.data_as(ctypes.c_void_p), 256)\n"
+        "print('survived')\n"
+    )
+    r = subprocess.run(["python", "-c", code], capture_output=True, text=True,
+                       cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    assert r.returncode != 0
+    assert "survived" not in r.stdout
+    assert "no CPU fallback" in r.stderr
