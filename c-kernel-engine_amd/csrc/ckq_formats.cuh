@@ -9,6 +9,8 @@
  *                 quants, four scales.
  *   Q8_0        : one 32-element block (34 B).
  * Each trait provides
+ *   Off / w_off    byte offsets of the position inside a weight row, computed
+ *                  once per lane (loads are then uniform row base + 32-bit offset),
  *   Wt  / load_w   raw weight dwords of a position (nothing decoded yet, so all
  *                  loads of a wave can be in flight together),
  *   Act / load_act the activation slice the position multiplies with,
@@ -49,16 +51,24 @@ struct FmtQ4K {
     struct Act { int q[16]; float d; int b_lo, b_hi; };
     struct Dec { int lo[8], hi[8]; int sc_lo, sc_hi, mn_lo, mn_hi; float d, dmin; };
 
-    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, int pos)
+    struct Off { u32 hdr, qs; };   /* byte offsets inside a weight row */
+    static __device__ __forceinline__ Off w_off(int pos)
     {
-        const uint8_t *blk = row + (size_t)(pos >> 2) * WBLOCK;
-        ld16<4>(w.hdr, blk);
-        ld16<4>(w.qs, blk + 16 + 32 * (pos & 3));
-        ld16<4>(w.qs + 4, blk + 32 + 32 * (pos & 3));
+        Off o;
+        o.hdr = (u32)(pos >> 2) * WBLOCK;
+        o.qs  = o.hdr + 16 + 32 * (pos & 3);
+        return o;
+    }
+    static __device__ __forceinline__ void off_shift(Off &o, u32 s) { o.hdr += s; o.qs += s; }
+    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, const Off &o)
+    {
+        ld16<4>(w.hdr, row + o.hdr);
+        ld16<4>(w.qs, row + o.qs);
+        ld16<4>(w.qs + 4, row + o.qs + 16);
     }
     static __device__ __forceinline__ void load_act(Act &a, const uint8_t *x, int pos)
     {
-        const uint8_t *blk = x + (size_t)(pos >> 2) * XBLOCK;
+        const uint8_t *blk = x + (u32)(pos >> 2) * XBLOCK;
         const int g = pos & 3;
         a.d = __builtin_bit_cast(float, ld4<4>(blk));
         for (int i = 0; i < 4; ++i) ld16<4>(a.q + 4 * i, blk + 4 + 64 * g + 16 * i);
@@ -104,14 +114,22 @@ struct FmtQ5K {
     typedef FmtQ4K::Act Act;
     typedef FmtQ4K::Dec Dec;
 
-    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, int pos)
+    typedef FmtQ4K::Off Off;
+    static __device__ __forceinline__ Off w_off(int pos)
     {
-        const uint8_t *blk = row + (size_t)(pos >> 2) * WBLOCK;
-        ld16<4>(w.hdr, blk);
-        ld16<4>(w.qh, blk + 16);
-        ld16<4>(w.qh + 4, blk + 32);
-        ld16<4>(w.qs, blk + 48 + 32 * (pos & 3));
-        ld16<4>(w.qs + 4, blk + 64 + 32 * (pos & 3));
+        Off o;
+        o.hdr = (u32)(pos >> 2) * WBLOCK;
+        o.qs  = o.hdr + 48 + 32 * (pos & 3);
+        return o;
+    }
+    static __device__ __forceinline__ void off_shift(Off &o, u32 s) { o.hdr += s; o.qs += s; }
+    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, const Off &o)
+    {
+        ld16<4>(w.hdr, row + o.hdr);
+        ld16<4>(w.qh, row + o.hdr + 16);
+        ld16<4>(w.qh + 4, row + o.hdr + 32);
+        ld16<4>(w.qs, row + o.qs);
+        ld16<4>(w.qs + 4, row + o.qs + 16);
     }
     static __device__ __forceinline__ void load_act(Act &a, const uint8_t *x, int pos) { FmtQ4K::load_act(a, x, pos); }
     static __device__ __forceinline__ void decode(Dec &d, const Wt &w, int pos)
@@ -141,19 +159,30 @@ struct FmtQ6K {
     struct Act { int q[16]; float d; int a32[4]; };      /* a32[r] = 32 * sum of the run's 16 quants */
     struct Dec { int q[16]; int sc[4]; float d; };
 
-    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, int pos)
+    struct Off { u32 ql, qh, sc, d; };
+    static __device__ __forceinline__ Off w_off(int pos)
     {
-        const uint8_t *blk = row + (size_t)(pos >> 2) * WBLOCK;
+        const u32 blk = (u32)(pos >> 2) * WBLOCK;
         const int n = (pos >> 1) & 1, l0 = 16 * (pos & 1);
-        ld16<2>(w.ql0, blk + 64 * n + l0);
-        ld16<2>(w.ql1, blk + 64 * n + 32 + l0);
-        ld16<2>(w.qh, blk + 128 + 32 * n + l0);
-        ld8<2>(w.sc, blk + 192 + 8 * n);
-        w.d = ld2(blk + 208);
+        Off o;
+        o.ql = blk + 64 * n + l0;
+        o.qh = blk + 128 + 32 * n + l0;
+        o.sc = blk + 192 + 8 * n;
+        o.d  = blk + 208;
+        return o;
+    }
+    static __device__ __forceinline__ void off_shift(Off &o, u32 s) { o.ql += s; o.qh += s; o.sc += s; o.d += s; }
+    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, const Off &o)
+    {
+        ld16<2>(w.ql0, row + o.ql);
+        ld16<2>(w.ql1, row + o.ql + 32);
+        ld16<2>(w.qh, row + o.qh);
+        ld8<2>(w.sc, row + o.sc);
+        w.d = ld2(row + o.d);
     }
     static __device__ __forceinline__ void load_act(Act &a, const uint8_t *x, int pos)
     {
-        const uint8_t *blk = x + (size_t)(pos >> 2) * XBLOCK;
+        const uint8_t *blk = x + (u32)(pos >> 2) * XBLOCK;
         const int n = (pos >> 1) & 1, l0 = 16 * (pos & 1);
         a.d = __builtin_bit_cast(float, ld4<4>(blk));
         for (int r = 0; r < 4; ++r) {
@@ -206,16 +235,23 @@ struct FmtQ80 {
     struct Act { int q[8]; float d; };
     struct Dec { int q[8]; float d; };
 
-    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, int pos)
+    struct Off { u32 blk; };
+    static __device__ __forceinline__ Off w_off(int pos)
     {
-        const uint8_t *blk = row + (size_t)pos * WBLOCK;
-        w.d = ld2(blk);
-        ld16<2>(w.q, blk + 2);
-        ld16<2>(w.q + 4, blk + 18);
+        Off o;
+        o.blk = (u32)pos * WBLOCK;
+        return o;
+    }
+    static __device__ __forceinline__ void off_shift(Off &o, u32 s) { o.blk += s; }
+    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, const Off &o)
+    {
+        w.d = ld2(row + o.blk);
+        ld16<2>(w.q, row + o.blk + 2);
+        ld16<2>(w.q + 4, row + o.blk + 18);
     }
     static __device__ __forceinline__ void load_act(Act &a, const uint8_t *x, int pos)
     {
-        const uint8_t *blk = x + (size_t)pos * XBLOCK;
+        const uint8_t *blk = x + (u32)pos * XBLOCK;
         a.d = h2f(ld2(blk));
         ld16<2>(a.q, blk + 2);
         ld16<2>(a.q + 4, blk + 18);
@@ -243,10 +279,13 @@ struct FmtQ80F32 {
     typedef FmtQ80::Dec Dec;
     struct Act { float x[32]; };
 
-    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, int pos) { FmtQ80::load_w(w, row, pos); }
+    typedef FmtQ80::Off Off;
+    static __device__ __forceinline__ Off w_off(int pos) { return FmtQ80::w_off(pos); }
+    static __device__ __forceinline__ void off_shift(Off &o, u32 s) { FmtQ80::off_shift(o, s); }
+    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, const Off &o) { FmtQ80::load_w(w, row, o); }
     static __device__ __forceinline__ void load_act(Act &a, const uint8_t *x, int pos)
     {
-        const uint8_t *p = x + (size_t)pos * XBLOCK;
+        const uint8_t *p = x + (u32)pos * XBLOCK;
         for (int i = 0; i < 8; ++i) {
             u32 t[4];
             ld16<4>(t, p + 16 * i);

@@ -33,24 +33,49 @@ struct GemvArgs {
     long wrow, xrow, ldy;
 };
 
+/* Wave index as a scalar: lets the compiler keep row indices, row base
+ * addresses and loop control in SGPRs (uniform branches, scalar address math). */
+__device__ __forceinline__ int wave_in_block() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
+
 /*
- * One wave handles (64/LPR)*RPI weight rows: LPR lanes share a row, lane l of
- * the group owns positions l, l+LPR, ... (PPL of them per pass).  All weight
- * and activation loads of a pass are issued before anything is decoded, so a
- * wave keeps RPI*PPL*(48..80) bytes per lane in flight; there is no loop over
- * rows, the grid supplies the parallelism.  The fp32 partials are summed over
- * the LPR lanes with a fixed DPP tree and the last lane of the group stores.
+ * Tiled kernel (token tiles MT >= 1, and the sub-block-dot dump).  One wave
+ * handles (64/LPR)*RPI weight rows: LPR lanes share a row, lane l of the group
+ * owns positions l, l+LPR, ... (PPL of them per pass).  All weight and
+ * activation loads of a pass are issued before anything is decoded.  There is
+ * no loop over rows: the grid supplies the parallelism.  The fp32 partials are
+ * summed over the LPR lanes with a fixed DPP tree; the last lane of the group
+ * stores.
  */
-template <class F, int LPR, int PPL, int MT, int RPI, bool DUMP>
-__global__ void __launch_bounds__(256) gemv_kernel(GemvArgs a)
+template <class F, int LPR, int PPL, int MT, int RPI, bool DUMP, int WPB, bool LDSX>
+__global__ void __launch_bounds__(64 * WPB) gemv_kernel(GemvArgs a)
 {
     constexpr int SLOTS = 64 / LPR;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    extern __shared__ __attribute__((aligned(16))) uint8_t xs[];   /* LDSX: the MT activation rows */
+    const int lane = threadIdx.x & 63, wave = wave_in_block();
     const int slot = lane / LPR, l = lane % LPR;
-    const int wave_row = a.row0 + (blockIdx.x * 4 + wave) * (SLOTS * RPI);
-    if (wave_row >= a.row1) return;
+    const int wave_row = a.row0 + (blockIdx.x * WPB + wave) * (SLOTS * RPI);   /* uniform */
+    const bool live = wave_row < a.row1;
+    if (!LDSX && !live) return;
+    const int wrow_c = min(wave_row, a.row1 - 1);
     const int rbase = wave_row + slot * RPI;
     const int t0 = blockIdx.y * MT;
+    const uint8_t *wbase = a.W + (size_t)wrow_c * a.wrow;                      /* uniform */
+
+    if (LDSX) {
+        /* every wave of the block reads the same activation rows: stage them
+         * once in LDS instead of once per wave through the vector cache */
+        const int ntok = min(MT, a.ntok - t0);
+        const uint8_t *src = a.X + (size_t)t0 * a.xrow;
+        if (F::XBLOCK % 4 == 0) {
+            const int n = (int)((long)ntok * a.xrow / 4);
+            for (int i = threadIdx.x; i < n; i += 64 * WPB)
+                reinterpret_cast<u32 *>(xs)[i] = reinterpret_cast<const u32 *>(src)[i];
+        } else {
+            const int n = (int)((long)ntok * a.xrow / 2);
+            for (int i = threadIdx.x; i < n; i += 64 * WPB)
+                reinterpret_cast<uint16_t *>(xs)[i] = reinterpret_cast<const uint16_t *>(src)[i];
+        }
+    }
 
     float acc[RPI][MT];
 #pragma unroll
@@ -58,21 +83,37 @@ __global__ void __launch_bounds__(256) gemv_kernel(GemvArgs a)
 #pragma unroll
         for (int t = 0; t < MT; ++t) acc[r][t] = 0.0f;
 
+    u32 rowoff[RPI];   /* byte offset of the lane's r-th row from wbase, clamped to the last row */
+#pragma unroll
+    for (int r = 0; r < RPI; ++r) rowoff[r] = (u32)(min(rbase + r, a.row1 - 1) - wrow_c) * (u32)a.wrow;
+
     for (int p0 = 0; p0 < a.npos; p0 += LPR * PPL) {
         typename F::Wt  w[RPI][PPL];
         typename F::Act act[MT][PPL];
 #pragma unroll
         for (int p = 0; p < PPL; ++p) {
             const int pos = min(p0 + p * LPR + l, a.npos - 1);
+            const typename F::Off o = F::w_off(pos);
 #pragma unroll
             for (int r = 0; r < RPI; ++r) {
-                const int row = min(rbase + r, a.row1 - 1);
-                F::load_w(w[r][p], a.W + (size_t)row * a.wrow, pos);
+                typename F::Off orow = o;
+                F::off_shift(orow, rowoff[r]);
+                F::load_w(w[r][p], wbase, orow);
             }
+        }
+        if (LDSX && p0 == 0) __syncthreads();
+#pragma unroll
+        for (int p = 0; p < PPL; ++p) {
+            const int pos = min(p0 + p * LPR + l, a.npos - 1);
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
-                const int tok = min(t0 + t, a.ntok - 1);
-                F::load_act(act[t][p], a.X + (size_t)tok * a.xrow, pos);
+                if (LDSX) {
+                    const int tl = min(t, a.ntok - t0 - 1);                    /* uniform */
+                    F::load_act(act[t][p], xs + (u32)tl * (u32)a.xrow, pos);
+                } else {
+                    const int tok = min(t0 + t, a.ntok - 1);                   /* uniform */
+                    F::load_act(act[t][p], a.X + (size_t)tok * a.xrow, pos);
+                }
             }
         }
 #pragma unroll
@@ -110,28 +151,36 @@ __global__ void __launch_bounds__(256) gemv_kernel(GemvArgs a)
         }
 }
 
-template <class F, int LPR, int PPL, int MT, int RPI, bool DUMP>
+template <class F, int LPR, int PPL, int MT, int RPI, bool DUMP, int WPB, bool LDSX>
 static int launch_one(const GemvArgs &a, hipStream_t s)
 {
-    constexpr int rows_per_block = 4 * (64 / LPR) * RPI;
+    constexpr int rows_per_block = WPB * (64 / LPR) * RPI;
     const int nr = a.row1 - a.row0;
     dim3 grid((nr + rows_per_block - 1) / rows_per_block, (a.ntok + MT - 1) / MT);
-    hipLaunchKernelGGL((gemv_kernel<F, LPR, PPL, MT, RPI, DUMP>), grid, dim3(256), 0, s, a);
+    const size_t lds = LDSX ? (size_t)MT * (size_t)a.xrow : 0;
+    hipLaunchKernelGGL((gemv_kernel<F, LPR, PPL, MT, RPI, DUMP, WPB, LDSX>), grid, dim3(64 * WPB), lds, s, a);
     return (int)hipGetLastError();
 }
 
-/* Rows per wave-slot for each token tile: more rows in flight for the
- * bandwidth-bound single-token case, fewer as the activation tile grows. */
-template <int MT> struct RowsPer { static constexpr int v = MT == 1 ? 4 : (MT <= 4 ? 2 : 1); };
+/* Activation rows are staged in LDS when the token tile fits in 64 KB. */
+template <class F, int LPR, int PPL, int MT, int RPI, int WPB>
+static int launch_tile(const GemvArgs &a, hipStream_t s)
+{
+    if ((size_t)MT * (size_t)a.xrow <= 65536) return launch_one<F, LPR, PPL, MT, RPI, false, WPB, true>(a, s);
+    return launch_one<F, LPR, PPL, MT, RPI, false, WPB, false>(a, s);
+}
 
+/* Rows per wave-slot and waves per block for each token tile: one row per
+ * slot and many waves for the bandwidth-bound single-token case (every load of
+ * the matrix in flight at once), fewer rows in flight as the tile grows. */
 template <class F, int LPR, int PPL>
 static int launch_mt(const GemvArgs &a, bool dump, int max_mt, hipStream_t s)
 {
-    if (dump) return launch_one<F, LPR, PPL, 1, 1, true>(a, s);
-    if (a.ntok == 1 || max_mt == 1) return launch_one<F, LPR, PPL, 1, RowsPer<1>::v, false>(a, s);
-    if (a.ntok == 2) return launch_one<F, LPR, PPL, 2, RowsPer<2>::v, false>(a, s);
-    if (a.ntok <= 4) return launch_one<F, LPR, PPL, 4, RowsPer<4>::v, false>(a, s);
-    return launch_one<F, LPR, PPL, 8, RowsPer<8>::v, false>(a, s);
+    if (dump) return launch_one<F, LPR, PPL, 1, 1, true, 4, false>(a, s);
+    if (a.ntok == 1 || max_mt == 1) return launch_tile<F, LPR, PPL, 1, 1, 8>(a, s);
+    if (a.ntok == 2) return launch_tile<F, LPR, PPL, 2, 2, 4>(a, s);
+    if (a.ntok <= 4) return launch_tile<F, LPR, PPL, 4, 2, 4>(a, s);
+    return launch_tile<F, LPR, PPL, 8, 1, 4>(a, s);
 }
 
 template <class F>
