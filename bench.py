@@ -203,7 +203,7 @@ def main():
         ops = 2.0 * Mg * rows * K
         extras["gemm_q4_k_q8_k_M512"] = {"tops": round(ops / sg / 1e12, 2), "ms": round(sg * 1e3, 4),
                                          "frac_int8_peak": round(ops / sg / 1e12 / INT8_PEAK_TOPS, 4),
-                                         "ops_per_call": ops, "kernel": "dot4 GEMV kernel, 8-token tiles"}
+                                         "ops_per_call": ops, "kernel": "two-plane int8 MFMA (v_mfma_i32_32x32x32_i8) + bf16 MFMA min term"}
         for name, fmt, r, k in (("gemv_q4_k_4096x4096", "q4_k", 4096, 4096),
                                 ("lm_head_q6_k_32000x4096", "q6_k", 32000, 4096),
                                 ("down_q6_k_4096x11008", "q6_k", 4096, 11008),

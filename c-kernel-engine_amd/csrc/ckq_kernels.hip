@@ -19,9 +19,16 @@
 #include "ckq_formats.cuh"
 #include "ckq_launch.h"
 
+__device__ __forceinline__ int wave_in_block();
+
 /* ========================================================================= */
 /* GEMV                                                                       */
 /* ========================================================================= */
+
+/* Token counts above this use the MFMA GEMM (Q4_K); at or below it the
+ * weight-streaming dot4 kernel with 8-token tiles reads the weights once or
+ * twice and is faster. */
+#define CKQ_GEMM_MIN_TOKENS 16
 
 struct GemvArgs {
     float         *y;
@@ -36,6 +43,8 @@ struct GemvArgs {
 /* Wave index as a scalar: lets the compiler keep row indices, row base
  * addresses and loop control in SGPRs (uniform branches, scalar address math). */
 __device__ __forceinline__ int wave_in_block() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
+
+#include "ckq_gemm_mfma.cuh"
 
 /*
  * Tiled kernel (token tiles MT >= 1, and the sub-block-dot dump).  One wave
@@ -213,6 +222,9 @@ extern "C" int ckq_launch_gemv(int fmt, float *y, const void *W, const void *X, 
     switch (fmt) {
     case CKQ_FMT_Q4_K:
         if (K % 256) return CKQ_ESHAPE;
+        /* prefill-sized token counts go to the matrix cores */
+        if (!dump && ntok > CKQ_GEMM_MIN_TOKENS && row0 == 0 && row1 == nrows)
+            return launch_gemm_q4k_mfma(X, W, bias, y, ntok, nrows, K, ldy, s);
         a.npos = K / 64; a.wrow = (long)(K / 256) * 144; a.xrow = (long)(K / 256) * 292; a.nsub_row = K / 32;
         return launch_fmt<FmtQ4K>(a, dump, 8, s);
     case CKQ_FMT_Q5_K:

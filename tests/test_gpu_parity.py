@@ -320,3 +320,81 @@ def test_batched_decode_small_model_shapes(M):
         say("batched decode", fmt, rows, K, "M", M)
         c = P.dev_gemm_nt(fmt, P.to_device(xq), P.to_device(W), None, M, rows, K).cpu().numpy()
         assert T.norm_err(c, T.oracle_gemm_nt(fmt, xq, W, None, M, rows, K)) <= TOL
+
+
+# ---- prefill GEMM on the matrix cores (Q4_K, token counts above 16) -------------------------
+
+@pytest.mark.parametrize("M,N,K", [(17, 128, 256), (33, 200, 1024), (64, 96, 512), (100, 333, 2048),
+                                   (128, 1, 256), (65, 129, 4096)])
+def test_gemm_mfma_q4_k_vs_oracle(M, N, K):
+    bias = T.normal(N, 0.0, 0.5, seed=N)
+    for kind in ("rand", "enc"):
+        W, _, xq = make_case("q4_k", N, K, kind, 700 + M + N, tokens=M)
+        say("gemm mfma q4_k", kind, "M", M, "N", N, "K", K)
+        ref = T.oracle_gemm_nt("q4_k", xq, W, bias, M, N, K)
+        c = P.dev_gemm_nt("q4_k", P.to_device(xq), P.to_device(W), P.to_device(bias), M, N, K).cpu().numpy()
+        assert T.norm_err(c, ref) <= TOL, (M, N, K, kind)
+        # the matrix-core path and the dot4 path agree token by token
+        ab = T.row_bytes("q8_k", K)
+        y = P.gemv("q4_k", W, xq[(M - 1) * ab:M * ab].copy(), N, K)
+        assert T.norm_err(c[M - 1] - bias, y) <= 2e-6
+        ch = P.gemm_nt("q4_k", xq, W, bias, M, N, K)      # host-pointer entry point, same kernel
+        assert np.array_equal(ch, c)
+
+
+def test_gemm_mfma_stored_bsums_and_extremes():
+    """Stored bsums are consumed (zeroed bsums drop the min term), and the
+    extreme quant values (nibble 15, scale 63, q8 = -128/127) stay exact."""
+    M, N, K = 64, 64, 512
+    W, _, xq = make_case("q4_k", N, K, "rand", 911, tokens=M)
+    xz = xq.copy().reshape(-1, 292)
+    xz[:, 260:292] = 0
+    xz = xz.reshape(-1)
+    ref = T.oracle_gemm_nt("q4_k", xz, W, None, M, N, K)
+    c = P.dev_gemm_nt("q4_k", P.to_device(xz), P.to_device(W), None, M, N, K).cpu().numpy()
+    assert T.norm_err(c, ref) <= TOL
+    # extremes: all nibbles 15, all scales/mins 63, activations alternating -128 / 127
+    Wb = W.copy().reshape(-1, 144)
+    Wb[:, 4:16] = 0xFF
+    Wb[:, 16:] = 0xFF
+    Wb = Wb.reshape(-1)
+    xb = xq.copy().reshape(-1, 292)
+    q = np.where(np.arange(256) % 2 == 0, -128, 127).astype(np.int8)
+    xb[:, 4:260] = q.view(np.uint8)
+    xb[:, 260:292] = np.tile(np.array([-8] * 16, np.int16).view(np.uint8), 1)
+    xb = xb.reshape(-1)
+    ref = T.oracle_gemm_nt("q4_k", xb, Wb, None, M, N, K)
+    c = P.dev_gemm_nt("q4_k", P.to_device(xb), P.to_device(Wb), None, M, N, K).cpu().numpy()
+    assert T.norm_err(c, ref) <= TOL
+    # largest positive dot: activations all 127
+    xb = xb.reshape(-1, 292)
+    xb[:, 4:260] = 127
+    xb[:, 260:292] = np.array([127 * 16] * 16, np.int16).view(np.uint8)
+    xb = xb.reshape(-1)
+    ref = T.oracle_gemm_nt("q4_k", xb, Wb, None, M, N, K)
+    c = P.dev_gemm_nt("q4_k", P.to_device(xb), P.to_device(Wb), None, M, N, K).cpu().numpy()
+    assert T.norm_err(c, ref) <= TOL
+
+
+def test_gemm_mfma_full_prefill_shape():
+    """M=512, N=11008, K=4096.  The oracle is evaluated on a sample of weight
+    rows (the whole product would take minutes on the CPU); every token is
+    checked for those rows, and the GEMM is checked against the GEMV kernel on
+    whole rows of C for a few tokens."""
+    M, N, K = 512, 11008, 4096
+    W = T.synth_weights("q4_k", N, K, seed=5150)
+    xf = T.normal(M * K, 0.0, 1.0, seed=5151)
+    say("gemm mfma full prefill shape")
+    xq_d = P.dev_quantize(P.to_device(xf), "q8_k", rows=M)
+    xq = xq_d.cpu().numpy()
+    Wd = P.to_device(W)
+    c = P.dev_gemm_nt("q4_k", xq_d, Wd, None, M, N, K).cpu().numpy()
+    rb = T.row_bytes("q4_k", K)
+    rows = np.array([0, 1, 31, 32, 127, 128, 5000, 5503, 5504, 11006, 11007])
+    Wsub = np.ascontiguousarray(W.reshape(N, rb)[rows]).reshape(-1)
+    ref = T.oracle_gemm_nt("q4_k", xq, Wsub, None, M, len(rows), K)
+    assert T.norm_err(c[:, rows], ref) <= TOL
+    ab = T.row_bytes("q8_k", K)
+    for t in (0, 63, 64, 300, 511):
+        y = P.dev_gemm_nt("q4_k", P.to_device(xq[t * ab:(t + 1) * ab].copy()), Wd, None, 1, N, K).cpu().numpy().reshape(-1)
+        assert T.norm_err(c[t], y) <= 2e-6, t
