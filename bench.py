@@ -24,6 +24,10 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+# HBM bytes per headline launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by the
+# same counters on the plain copy kernel (2.000 and 1.000); measurement recorded in
+# profiles/gemv_q4_k_11008x4096_hbm_traffic_pmc.txt
+TRAFFIC_BYTES_PER_LAUNCH = 25492992
 INT8_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA, published
 MALL_BYTES = 256 << 20
 
@@ -154,6 +158,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="only the headline workload")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch the plain copy kernel on a 256 MiB buffer (known traffic), for scaling "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported (every box here has one GPU, "
@@ -165,6 +172,16 @@ def main():
     xf = T.normal(K, 0.0, 1.0, seed=4242)
     xq_d = P.dev_quantize(P.to_device(xf), "q8_k")
     W, copies = H.weight_copies("q4_k", rows, K, seed=4243)
+
+    if a.calibrate_copy:
+        n = 256 << 20
+        src = torch.empty(n, dtype=torch.uint8, device="cuda").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(8):
+            H.ckq.api.check(H.L.ckq_copy_dev(ctypes.c_void_p(dst.data_ptr()), ctypes.c_void_p(src.data_ptr()), n,
+                                             ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)), "ckq_copy_dev")
+        torch.cuda.synchronize()
+        del src, dst
 
     # parity guard on the exact buffers being timed
     import numpy as np
@@ -186,7 +203,7 @@ def main():
                    "activations": "seeded N(0,1) -> Q8_K (quantized on the GPU)",
                    "weight_copies_rotated": len(copies), "bytes_per_step": bytes_},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH},
         "pct_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
         "cache_resident_gbs": round(bytes_ / sec_hot / 1e9, 2),
         "host_wall_ms_per_step": round(wall * 1e3, 6),

@@ -20,4 +20,4 @@ from .api import (  # noqa: F401
     row_bytes,
     synth_lib,
 )
-from . import parity  # noqa: F401
+from . import api, parity  # noqa: F401

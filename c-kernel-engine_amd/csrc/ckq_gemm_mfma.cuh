@@ -54,6 +54,10 @@ struct GemmArgs {
     int  ntt, nnt;        /* token tiles, weight-row tiles */
 };
 
+#ifndef CKQ_GEMM_WPE
+#define CKQ_GEMM_WPE 2          /* waves per SIMD the register budget is sized for */
+#endif
+
 constexpr int GEMM_XROW = 272;            /* padded LDS row: 256 quants + 16 */
 
 /* packed u8x4 times a small scalar, byte-wise (every product < 256) */
@@ -66,13 +70,115 @@ __device__ __forceinline__ int mul_bytes(u32 v, u32 s16x2)
 /* small non-negative / signed integer (|v| < 2^8 significant bits) -> bf16 bits */
 __device__ __forceinline__ u32 bf16_bits(float f) { return __builtin_bit_cast(u32, f) >> 16; }
 
+/* Staged activation block of BM tokens in LDS. */
+template <int BM>
+struct GemmTile {
+    uint8_t  q[2][BM * GEMM_XROW];   /* int8 quants, 272-byte rows */
+    float    d[2][BM];               /* block scale of each token */
+    uint16_t b[2][BM * 16];          /* bf16: lo_0..7, 64*hi_0..7 of the stored bsums */
+};
+
+/* Weights of one 256-block for one lane: header + the 16-byte nibble runs of
+ * its half of each 64-element group. */
+struct GemmW {
+    u32 hdr[4];
+    u32 q[16];
+};
+
+__device__ __forceinline__ void gemm_load_w(GemmW &w, const uint8_t *wrow, int b, int half)
+{
+    const uint8_t *blk = wrow + (u32)b * 144u;
+    ld16<4>(w.hdr, blk);
+#pragma unroll
+    for (int g = 0; g < 4; ++g) ld16<4>(w.q + 4 * g, blk + 16 + 32 * g + 16 * half);
+}
+
+/* One 256-block: expand the lane's weights to the two planes, run the MFMAs
+ * against the staged activations of buffer `cur`, fold into the fp32 tile. */
 template <int TS>
-__global__ void __launch_bounds__(256) gemm_q4k_mfma_kernel(GemmArgs a)
+__device__ __forceinline__ void gemm_block(const GemmW &w, const GemmTile<32 * TS> &tile, int cur, int col, int half,
+                                           ckq_v16f (&acc)[TS])
+{
+    /* 6-bit scales and mins of the 8 sub-blocks (word form of the unpack) */
+    const u32 sc03 = w.hdr[1] & 0x3f3f3f3fu;
+    const u32 sc47 = (w.hdr[3] & 0x0f0f0f0fu) | (((w.hdr[1] >> 6) & 0x03030303u) << 4);
+    const u32 mn03 = w.hdr[2] & 0x3f3f3f3fu;
+    const u32 mn47 = ((w.hdr[3] >> 4) & 0x0f0f0f0fu) | (((w.hdr[2] >> 6) & 0x03030303u) << 4);
+    const float dw = h2f(w.hdr[0] & 0xffff), dmin = h2f(w.hdr[0] >> 16);
+
+    ckq_v16i accH[TS], accL[TS];
+#pragma unroll
+    for (int ts = 0; ts < TS; ++ts)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { accH[ts][r] = 0; accL[ts][r] = 0; }
+
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+#pragma unroll
+        for (int hi = 0; hi < 2; ++hi) {
+            const int j = 2 * g + hi;
+            const u32 scw = j < 4 ? sc03 : sc47;
+            const u32 sc = (scw >> (8 * (j & 3))) & 0xff;
+            const u32 mh = (sc >> 3) * 0x00010001u, ml = (sc & 7) * 0x00010001u;
+            ckq_v4i bH, bL;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const u32 nib = hi ? ((w.q[4 * g + i] >> 4) & 0x0f0f0f0fu) : (w.q[4 * g + i] & 0x0f0f0f0fu);
+                bH[i] = mul_bytes(nib, mh);
+                bL[i] = mul_bytes(nib, ml);
+            }
+#pragma unroll
+            for (int ts = 0; ts < TS; ++ts) {
+                const ckq_v4i av = *reinterpret_cast<const ckq_v4i *>(
+                    &tile.q[cur][(32 * ts + col) * GEMM_XROW + 32 * j + 16 * half]);
+                accH[ts] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bH, accH[ts], 0, 0, 0);
+                accL[ts] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bL, accL[ts], 0, 0, 0);
+            }
+        }
+    }
+
+    /* min term: B operand = the row's 8 mins as bf16, in both k halves */
+    ckq_v8bf bm;
+    {
+        u32 m[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const u32 src = i < 2 ? mn03 : mn47;
+            const u32 m0 = (src >> (16 * (i & 1))) & 0xff, m1 = (src >> (16 * (i & 1) + 8)) & 0xff;
+            m[i] = bf16_bits((float)m0) | (bf16_bits((float)m1) << 16);
+        }
+        const ckq_v4i t = {(int)m[0], (int)m[1], (int)m[2], (int)m[3]};
+        bm = __builtin_bit_cast(ckq_v8bf, t);
+    }
+
+#pragma unroll
+    for (int ts = 0; ts < TS; ++ts) {
+        const ckq_v4i ab = *reinterpret_cast<const ckq_v4i *>(&tile.b[cur][(32 * ts + col) * 16 + 8 * half]);
+        ckq_v16f zero;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) zero[r] = 0.0f;
+        const ckq_v16f i2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(ckq_v8bf, ab), bm, zero, 0, 0, 0);
+        /* fp32 combine; D layout: register r, lane l -> token row 8*(r/4) + 4*(l/32) + r%4 */
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+            const float4 dx = *reinterpret_cast<const float4 *>(&tile.d[cur][32 * ts + 8 * r4 + 4 * half]);
+            const float dxs[4] = {dx.x, dx.y, dx.z, dx.w};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int r = 4 * r4 + k;
+                const float f = (float)((accH[ts][r] << 3) + accL[ts][r]);
+                const float u = dw * f - dmin * i2[r];
+                acc[ts][r] += u * dxs[k];
+            }
+        }
+    }
+}
+
+template <int TS, int WPE>
+__global__ void __launch_bounds__(256, WPE) gemm_q4k_mfma_kernel(GemmArgs a)
 {
     constexpr int BM = 32 * TS;
-    __shared__ __attribute__((aligned(16))) uint8_t  xs_q[2][BM * GEMM_XROW];
-    __shared__ __attribute__((aligned(16))) float    xs_d[2][BM];
-    __shared__ __attribute__((aligned(16))) uint16_t xs_b[2][BM * 16];   /* bf16: lo_0..7, 64*hi_0..7 */
+    __shared__ __attribute__((aligned(16))) GemmTile<BM> tile;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = wave_in_block();
     const int col = lane & 31, half = lane >> 5;
@@ -87,17 +193,18 @@ __global__ void __launch_bounds__(256) gemm_q4k_mfma_kernel(GemmArgs a)
     const int n_lane = min(nt * 128 + wave * 32 + col, a.N - 1);            /* this lane's weight row */
     const uint8_t *wrow = a.B + (size_t)n_lane * a.nb * 144;
     const long xstride = (long)a.nb * 292;
+    const int last = a.nb - 1;
 
     /* staging roles: thread -> (token row, 64-byte quarter) of the 256 quants */
     const int st_tok = tid >> 2, st_q = tid & 3;                            /* BM <= 64 rows x 4 quarters */
     const bool st_live = st_tok < BM;
     const uint8_t *st_src = a.A + (size_t)min(t0 + st_tok, a.M - 1) * xstride;
 
-    u32 nq[16];      /* next block's 64 quant bytes of this thread's quarter */
-    u32 nbs[2];      /* next block's 4 stored bsums (this quarter's sub-blocks 2q, 2q+1) */
+    u32 nq[16];      /* a block's 64 quant bytes of this thread's quarter */
+    u32 nbs[2];      /* its 4 stored bsums (sub-blocks 2q, 2q+1) */
     float nd = 0.f;
     auto stage_load = [&](int b) {
-        const uint8_t *blk = st_src + (size_t)b * 292;
+        const uint8_t *blk = st_src + (u32)b * 292u;
 #pragma unroll
         for (int i = 0; i < 4; ++i) ld16<4>(nq + 4 * i, blk + 4 + 64 * st_q + 16 * i);
         ld8<4>(nbs, blk + 260 + 8 * st_q);
@@ -105,26 +212,17 @@ __global__ void __launch_bounds__(256) gemm_q4k_mfma_kernel(GemmArgs a)
     };
     auto stage_store = [&](int buf) {
         if (!st_live) return;
-        u32 *dst = reinterpret_cast<u32 *>(&xs_q[buf][st_tok * GEMM_XROW + 64 * st_q]);
+        u32 *dst = reinterpret_cast<u32 *>(&tile.q[buf][st_tok * GEMM_XROW + 64 * st_q]);
 #pragma unroll
-        for (int i = 0; i < 16; ++i) dst[i] = nq[i];
-        if (st_q == 0) xs_d[buf][st_tok] = nd;
-        /* sub-blocks j = 2q, 2q+1: B32 = bsums[2j] + bsums[2j+1] */
+        for (int i = 0; i < 4; ++i)
+            *reinterpret_cast<ckq_v4i *>(dst + 4 * i) = ckq_v4i{(int)nq[4 * i], (int)nq[4 * i + 1], (int)nq[4 * i + 2], (int)nq[4 * i + 3]};
+        if (st_q == 0) tile.d[buf][st_tok] = nd;
+        /* sub-blocks j = 2q, 2q+1: B32 = bsums[2j] + bsums[2j+1] = lo + 64*hi */
         const int b0 = (int)(int16_t)(nbs[0] & 0xffff) + (int)(int16_t)(nbs[0] >> 16);
         const int b1 = (int)(int16_t)(nbs[1] & 0xffff) + (int)(int16_t)(nbs[1] >> 16);
-        const int lo0 = b0 & 63, hi0 = b0 >> 6, lo1 = b1 & 63, hi1 = b1 >> 6;
-        u32 *bd = reinterpret_cast<u32 *>(&xs_b[buf][st_tok * 16]);
-        bd[st_q]     = bf16_bits((float)lo0) | (bf16_bits((float)lo1) << 16);
-        bd[4 + st_q] = bf16_bits((float)(64 * hi0)) | (bf16_bits((float)(64 * hi1)) << 16);
-    };
-
-    /* weights of one block for this lane: header + the 16-byte runs of its half */
-    u32 whdr[4], wq[16];
-    auto weights_load = [&](int b) {
-        const uint8_t *blk = wrow + (size_t)b * 144;
-        ld16<4>(whdr, blk);
-#pragma unroll
-        for (int g = 0; g < 4; ++g) ld16<4>(wq + 4 * g, blk + 16 + 32 * g + 16 * half);
+        u32 *bd = reinterpret_cast<u32 *>(&tile.b[buf][st_tok * 16]);
+        bd[st_q]     = bf16_bits((float)(b0 & 63)) | (bf16_bits((float)(b1 & 63)) << 16);
+        bd[4 + st_q] = bf16_bits((float)(64 * (b0 >> 6))) | (bf16_bits((float)(64 * (b1 >> 6))) << 16);
     };
 
     ckq_v16f acc[TS];
@@ -133,99 +231,32 @@ __global__ void __launch_bounds__(256) gemm_q4k_mfma_kernel(GemmArgs a)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[ts][r] = 0.0f;
 
+    /* Two weight register sets alternate; every prefetch is unconditional
+     * (block index clamped) so no set is ever a conditional copy. */
+    GemmW w0, w1;
     stage_load(0);
-    weights_load(0);
+    gemm_load_w(w0, wrow, 0, half);
     stage_store(0);
     __syncthreads();
 
-    for (int b = 0; b < a.nb; ++b) {
-        const int cur = b & 1;
-        /* current weights -> local copies, then prefetch the next block */
-        u32 hdr[4], q[16];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) hdr[i] = whdr[i];
-#pragma unroll
-        for (int i = 0; i < 16; ++i) q[i] = wq[i];
-        if (b + 1 < a.nb) {
-            stage_load(b + 1);
-            weights_load(b + 1);
-        }
+    for (int b = 0; b < a.nb; b += 2) {
+        /* issue the next block's global loads BEFORE the MFMA work of this
+         * one; the scheduling barrier keeps the compiler from sinking them
+         * down to their first use */
+        stage_load(min(b + 1, last));
+        gemm_load_w(w1, wrow, min(b + 1, last), half);
+        __builtin_amdgcn_sched_barrier(0);
+        gemm_block<TS>(w0, tile, 0, col, half, acc);
+        __builtin_amdgcn_sched_barrier(0);
+        stage_store(1);
+        __syncthreads();
 
-        /* 6-bit scales and mins of the 8 sub-blocks (word form of the unpack) */
-        const u32 sc03 = hdr[1] & 0x3f3f3f3fu;
-        const u32 sc47 = (hdr[3] & 0x0f0f0f0fu) | (((hdr[1] >> 6) & 0x03030303u) << 4);
-        const u32 mn03 = hdr[2] & 0x3f3f3f3fu;
-        const u32 mn47 = ((hdr[3] >> 4) & 0x0f0f0f0fu) | (((hdr[2] >> 6) & 0x03030303u) << 4);
-        const float dw = h2f(hdr[0] & 0xffff), dmin = h2f(hdr[0] >> 16);
-
-        ckq_v16i accH[TS], accL[TS];
-#pragma unroll
-        for (int ts = 0; ts < TS; ++ts)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) { accH[ts][r] = 0; accL[ts][r] = 0; }
-
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-#pragma unroll
-            for (int hi = 0; hi < 2; ++hi) {
-                const int j = 2 * g + hi;
-                const u32 scw = j < 4 ? sc03 : sc47;
-                const u32 sc = (scw >> (8 * (j & 3))) & 0xff;
-                const u32 mh = (sc >> 3) * 0x00010001u, ml = (sc & 7) * 0x00010001u;
-                ckq_v4i bH, bL;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const u32 nib = hi ? ((q[4 * g + i] >> 4) & 0x0f0f0f0fu) : (q[4 * g + i] & 0x0f0f0f0fu);
-                    bH[i] = mul_bytes(nib, mh);
-                    bL[i] = mul_bytes(nib, ml);
-                }
-#pragma unroll
-                for (int ts = 0; ts < TS; ++ts) {
-                    const ckq_v4i av = *reinterpret_cast<const ckq_v4i *>(
-                        &xs_q[cur][(32 * ts + col) * GEMM_XROW + 32 * j + 16 * half]);
-                    accH[ts] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bH, accH[ts], 0, 0, 0);
-                    accL[ts] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bL, accL[ts], 0, 0, 0);
-                }
-            }
-        }
-
-        /* min term: B operand = the row's 8 mins as bf16, in both k halves */
-        ckq_v8bf bm;
-        {
-            u32 w[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const u32 src = i < 2 ? mn03 : mn47;
-                const u32 m0 = (src >> (16 * (i & 1))) & 0xff, m1 = (src >> (16 * (i & 1) + 8)) & 0xff;
-                w[i] = bf16_bits((float)m0) | (bf16_bits((float)m1) << 16);
-            }
-            ckq_v4i t = {(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
-            bm = __builtin_bit_cast(ckq_v8bf, t);
-        }
-
-#pragma unroll
-        for (int ts = 0; ts < TS; ++ts) {
-            const ckq_v4i ab = *reinterpret_cast<const ckq_v4i *>(&xs_b[cur][(32 * ts + col) * 16 + 8 * half]);
-            ckq_v16f zero;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) zero[r] = 0.0f;
-            const ckq_v16f i2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(ckq_v8bf, ab), bm, zero, 0, 0, 0);
-            /* fp32 combine; D layout: register r, lane l -> token row 8*(r/4) + 4*(l/32) + r%4 */
-#pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-                const float4 dx = *reinterpret_cast<const float4 *>(&xs_d[cur][32 * ts + 8 * r4 + 4 * half]);
-                const float dxs[4] = {dx.x, dx.y, dx.z, dx.w};
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const int r = 4 * r4 + k;
-                    const float f = (float)((accH[ts][r] << 3) + accL[ts][r]);
-                    const float u = dw * f - dmin * i2[r];
-                    acc[ts][r] += u * dxs[k];
-                }
-            }
-        }
-
-        if (b + 1 < a.nb) stage_store(cur ^ 1);
+        stage_load(min(b + 2, last));
+        gemm_load_w(w0, wrow, min(b + 2, last), half);
+        __builtin_amdgcn_sched_barrier(0);
+        if (b + 1 < a.nb) gemm_block<TS>(w1, tile, 1, col, half, acc);
+        __builtin_amdgcn_sched_barrier(0);
+        stage_store(0);
         __syncthreads();
     }
 
@@ -253,6 +284,6 @@ static int launch_gemm_q4k_mfma(const void *A, const void *B, const float *bias,
     g.ntt = (M + 32 * TS - 1) / (32 * TS);
     g.nnt = (N + 127) / 128;
     const int nnt8 = (g.nnt + 7) / 8 * 8;
-    hipLaunchKernelGGL((gemm_q4k_mfma_kernel<TS>), dim3(g.ntt * nnt8), dim3(256), 0, s, g);
+    hipLaunchKernelGGL((gemm_q4k_mfma_kernel<TS, CKQ_GEMM_WPE>), dim3(g.ntt * nnt8), dim3(256), 0, s, g);
     return (int)hipGetLastError();
 }
