@@ -195,27 +195,36 @@ __global__ void __launch_bounds__(256, WPE) gemm_q4k_mfma_kernel(GemmArgs a)
     const long xstride = (long)a.nb * 292;
     const int last = a.nb - 1;
 
-    /* staging roles: thread -> (token row, 64-byte quarter) of the 256 quants */
+    /* Staging roles.  Quants: 16 consecutive lanes cover the 256 contiguous
+     * bytes of one token (coalesced), a wave covers 4 tokens per load, the
+     * block 16; BM/16 loads per thread.  Side data (block scale and the 16
+     * stored bsums): 4 lanes per token, 8 bytes of bsums each. */
+    constexpr int NQ = BM / 16;
+    const int sq_tok = tid >> 4, sq_c = tid & 15;
+    const uint8_t *sq_src[NQ];
+#pragma unroll
+    for (int i = 0; i < NQ; ++i)
+        sq_src[i] = a.A + (size_t)min(t0 + sq_tok + 16 * i, a.M - 1) * xstride + 4 + 16 * sq_c;
     const int st_tok = tid >> 2, st_q = tid & 3;                            /* BM <= 64 rows x 4 quarters */
     const bool st_live = st_tok < BM;
     const uint8_t *st_src = a.A + (size_t)min(t0 + st_tok, a.M - 1) * xstride;
 
-    u32 nq[16];      /* a block's 64 quant bytes of this thread's quarter */
-    u32 nbs[2];      /* its 4 stored bsums (sub-blocks 2q, 2q+1) */
+    u32 nq[NQ][4];   /* a block's quant bytes staged by this thread */
+    u32 nbs[2];      /* 4 stored bsums (sub-blocks 2q, 2q+1) of token st_tok */
     float nd = 0.f;
     auto stage_load = [&](int b) {
-        const uint8_t *blk = st_src + (u32)b * 292u;
+        const u32 boff = (u32)b * 292u;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) ld16<4>(nq + 4 * i, blk + 4 + 64 * st_q + 16 * i);
-        ld8<4>(nbs, blk + 260 + 8 * st_q);
-        nd = __builtin_bit_cast(float, ld4<4>(blk));
+        for (int i = 0; i < NQ; ++i) ld16<4>(nq[i], sq_src[i] + boff);
+        ld8<4>(nbs, st_src + boff + 260 + 8 * st_q);
+        nd = __builtin_bit_cast(float, ld4<4>(st_src + boff));
     };
     auto stage_store = [&](int buf) {
-        if (!st_live) return;
-        u32 *dst = reinterpret_cast<u32 *>(&tile.q[buf][st_tok * GEMM_XROW + 64 * st_q]);
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            *reinterpret_cast<ckq_v4i *>(dst + 4 * i) = ckq_v4i{(int)nq[4 * i], (int)nq[4 * i + 1], (int)nq[4 * i + 2], (int)nq[4 * i + 3]};
+        for (int i = 0; i < NQ; ++i)
+            *reinterpret_cast<ckq_v4i *>(&tile.q[buf][(sq_tok + 16 * i) * GEMM_XROW + 16 * sq_c]) =
+                ckq_v4i{(int)nq[i][0], (int)nq[i][1], (int)nq[i][2], (int)nq[i][3]};
+        if (!st_live) return;
         if (st_q == 0) tile.d[buf][st_tok] = nd;
         /* sub-blocks j = 2q, 2q+1: B32 = bsums[2j] + bsums[2j+1] = lo + 64*hi */
         const int b0 = (int)(int16_t)(nbs[0] & 0xffff) + (int)(int16_t)(nbs[0] >> 16);
