@@ -19,19 +19,21 @@
  *   TWO int8 planes, H = (sc>>3)*q4 and L = (sc&7)*q4 (both <= 105), each
  *   accumulated over all eight sub-blocks of a block; I1 = 8*H + L exactly.
  *   Nibble unpack and the two multiplies (v_pk_mul_lo_u16 on byte pairs) are
- *   done once per weight and reused for every token sub-tile of the wave.
+ *   done once per weight and reused for both 32-token halves of the tile.
  * - The min term contracts 8 (min, bsum) pairs per block.  Stored bsums need
  *   13 bits; split as lo + 64*hi (lo in [0,63], hi in [-64,63]) both parts and
  *   the 6-bit mins are exact in bf16, so ONE v_mfma_f32_32x32x16_bf16 per
  *   32x32 tile per block yields I2 exactly in fp32 (|I2| < 2^24).
- * - Weights never touch LDS: each wave loads the 16-byte nibble runs of its 32
- *   rows straight into the lanes that need them as B operands (Q4_K stores
- *   sub-blocks 2g and 2g+1 as the low and high nibbles of the same bytes, so
- *   one 128-bit load feeds two K-steps).  Activations are staged per block
- *   through LDS with 272-byte rows so that ds_read_b128 of 32 token rows is
- *   bank-conflict free, double-buffered against the MFMA work.
+ * - Every operand reaches the matrix cores through LDS, filled by 16-byte
+ *   global->LDS loads (no VGPR staging): the raw Q4_K blocks of the tile's
+ *   128 rows (9 consecutive lanes read one 144-byte block contiguously) and
+ *   the int8 quants of its 64 tokens (16 lanes per token), double-buffered
+ *   against the MFMA work.  A lane reads its own row's header and nibble
+ *   runs back with ds_read_b128 (144-byte stride: conflict-free); the quants
+ *   are stored with their 16-byte chunks XOR-swizzled by the token number so
+ *   that 32 token rows at a 256-byte stride read conflict-free too.
  *
- * Block = 4 waves = (32*TS tokens) x (128 weight rows); wave w owns rows
+ * Block = 4 waves = 64 tokens x 128 weight rows; wave w owns rows
  * 32w..32w+31.  Grid: token tiles fastest inside an XCD so the eight XCD L2s
  * each see a weight tile once.
  */
@@ -43,6 +45,8 @@ typedef int   ckq_v16i __attribute__((ext_vector_type(16)));
 typedef float ckq_v16f __attribute__((ext_vector_type(16)));
 typedef __bf16 ckq_v8bf __attribute__((ext_vector_type(8)));
 typedef unsigned short ckq_v2u16 __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) void ckq_lds_void;
+typedef const __attribute__((address_space(1))) void ckq_glb_void;
 
 struct GemmArgs {
     const uint8_t *A;     /* Q8_K activations, M rows of nb blocks */
@@ -58,8 +62,6 @@ struct GemmArgs {
 #define CKQ_GEMM_WPE 2          /* waves per SIMD the register budget is sized for */
 #endif
 
-constexpr int GEMM_XROW = 272;            /* padded LDS row: 256 quants + 16 */
-
 /* packed u8x4 times a small scalar, byte-wise (every product < 256) */
 __device__ __forceinline__ int mul_bytes(u32 v, u32 s16x2)
 {
@@ -70,211 +72,239 @@ __device__ __forceinline__ int mul_bytes(u32 v, u32 s16x2)
 /* small non-negative / signed integer (|v| < 2^8 significant bits) -> bf16 bits */
 __device__ __forceinline__ u32 bf16_bits(float f) { return __builtin_bit_cast(u32, f) >> 16; }
 
-/* Staged activation block of BM tokens in LDS. */
-template <int BM>
-struct GemmTile {
-    uint8_t  q[2][BM * GEMM_XROW];   /* int8 quants, 272-byte rows */
-    float    d[2][BM];               /* block scale of each token */
-    uint16_t b[2][BM * 16];          /* bf16: lo_0..7, 64*hi_0..7 of the stored bsums */
+constexpr int GEMM_BM = 64;     /* tokens per tile */
+constexpr int GEMM_BN = 128;    /* weight rows per tile */
+
+/* LDS image of one 256-block for a tile of 128 weight rows x 64 tokens. */
+struct GemmStage {
+    uint8_t  w[GEMM_BN * 144];    /* raw Q4_K blocks, row r at byte 144 r */
+    uint8_t  q[GEMM_BM * 256];    /* int8 quants: 16-byte chunk c of token t in slot c ^ (t & 15) of its 256 bytes */
+    float    d[GEMM_BM];          /* block scale of each token */
+    uint16_t b[GEMM_BM * 16];     /* bf16: lo_0..7, 64*hi_0..7 of the stored bsums */
 };
 
-/* Weights of one 256-block for one lane: header + the 16-byte nibble runs of
- * its half of each 64-element group. */
-struct GemmW {
-    u32 hdr[4];
-    u32 q[16];
-};
-
-__device__ __forceinline__ void gemm_load_w(GemmW &w, const uint8_t *wrow, int b, int half)
+/* One 256-block of a 64-token tile, software-pipelined by hand.  The 32 int8
+ * MFMAs run in four passes of eight - (tokens 0-31 | 32-63) x (sub-blocks 0-3 |
+ * 4-7) - so that VALU work always has matrix work to hide under: the planes
+ * of sub-blocks 0-3 are expanded during pass 1, those of 4-7 during pass 2,
+ * and the fp32 combine of tokens 0-31 runs under pass 4.  Activation operands
+ * are read from LDS two steps ahead.  Scheduling barriers pin that order. */
+template <class CopyFn>
+__device__ __forceinline__ void gemm_block_pipe(const GemmStage &st, u32 wofs, const u32 (&aofs)[8], int col, int half,
+                                                ckq_v16f (&acc)[2], CopyFn copy_one)
 {
-    const uint8_t *blk = wrow + (u32)b * 144u;
-    ld16<4>(w.hdr, blk);
-#pragma unroll
-    for (int g = 0; g < 4; ++g) ld16<4>(w.q + 4 * g, blk + 16 + 32 * g + 16 * half);
-}
+#define CKQ_PIN() __builtin_amdgcn_sched_barrier(0)
+    auto lds16 = [&](const uint8_t *p) { return *reinterpret_cast<const ckq_v4i *>(p); };
+    /* step s = 0..15: pass order (ts, j) = (0,0..3) (1,0..3) (0,4..7) (1,4..7) */
+    auto step_ts = [](int s) { return (s >> 2) & 1; };
+    auto step_j  = [](int s) { return (s & 3) | ((s >> 3) << 2); };
+    auto a_read = [&](int s) { return lds16(&st.q[aofs[step_j(s)] + 32 * 256 * step_ts(s)]); };
 
-/* One 256-block: expand the lane's weights to the two planes, run the MFMAs
- * against the staged activations of buffer `cur`, fold into the fp32 tile. */
-template <int TS>
-__device__ __forceinline__ void gemm_block(const GemmW &w, const GemmTile<32 * TS> &tile, int cur, int col, int half,
-                                           ckq_v16f (&acc)[TS])
-{
-    /* 6-bit scales and mins of the 8 sub-blocks (word form of the unpack) */
-    const u32 sc03 = w.hdr[1] & 0x3f3f3f3fu;
-    const u32 sc47 = (w.hdr[3] & 0x0f0f0f0fu) | (((w.hdr[1] >> 6) & 0x03030303u) << 4);
-    const u32 mn03 = w.hdr[2] & 0x3f3f3f3fu;
-    const u32 mn47 = ((w.hdr[3] >> 4) & 0x0f0f0f0fu) | (((w.hdr[2] >> 6) & 0x03030303u) << 4);
-    const float dw = h2f(w.hdr[0] & 0xffff), dmin = h2f(w.hdr[0] >> 16);
+    const ckq_v4i hv = lds16(&st.w[wofs]);
+    ckq_v4i qv[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) qv[g] = lds16(&st.w[wofs + 16 + 32 * g + 16 * half]);
+    ckq_v4i av[3];
+    av[0] = a_read(0);
+    av[1] = a_read(1);
 
-    ckq_v16i accH[TS], accL[TS];
-#pragma unroll
-    for (int ts = 0; ts < TS; ++ts)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) { accH[ts][r] = 0; accL[ts][r] = 0; }
+    const u32 h0 = (u32)hv[0], h1 = (u32)hv[1], h2 = (u32)hv[2], h3 = (u32)hv[3];
+    const u32 sc03 = h1 & 0x3f3f3f3fu;
+    const u32 sc47 = (h3 & 0x0f0f0f0fu) | (((h1 >> 6) & 0x03030303u) << 4);
+    const float dw = h2f(h0 & 0xffff), dmin = h2f(h0 >> 16);
 
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-#pragma unroll
-        for (int hi = 0; hi < 2; ++hi) {
-            const int j = 2 * g + hi;
-            const u32 scw = j < 4 ? sc03 : sc47;
-            const u32 sc = (scw >> (8 * (j & 3))) & 0xff;
-            const u32 mh = (sc >> 3) * 0x00010001u, ml = (sc & 7) * 0x00010001u;
-            ckq_v4i bH, bL;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const u32 nib = hi ? ((w.q[4 * g + i] >> 4) & 0x0f0f0f0fu) : (w.q[4 * g + i] & 0x0f0f0f0fu);
-                bH[i] = mul_bytes(nib, mh);
-                bL[i] = mul_bytes(nib, ml);
-            }
-#pragma unroll
-            for (int ts = 0; ts < TS; ++ts) {
-                const ckq_v4i av = *reinterpret_cast<const ckq_v4i *>(
-                    &tile.q[cur][(32 * ts + col) * GEMM_XROW + 32 * j + 16 * half]);
-                accH[ts] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bH, accH[ts], 0, 0, 0);
-                accL[ts] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bL, accL[ts], 0, 0, 0);
-            }
-        }
-    }
-
-    /* min term: B operand = the row's 8 mins as bf16, in both k halves */
-    ckq_v8bf bm;
-    {
-        u32 m[4];
+    ckq_v4i bH[8], bL[8];
+    auto decode = [&](int j) {
+        const int g = j >> 1, hi = j & 1;
+        const u32 scw = j < 4 ? sc03 : sc47;
+        const u32 sc = (scw >> (8 * (j & 3))) & 0xff;
+        const u32 mh = (sc >> 3) * 0x00010001u, ml = (sc & 7) * 0x00010001u;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const u32 src = i < 2 ? mn03 : mn47;
-            const u32 m0 = (src >> (16 * (i & 1))) & 0xff, m1 = (src >> (16 * (i & 1) + 8)) & 0xff;
-            m[i] = bf16_bits((float)m0) | (bf16_bits((float)m1) << 16);
+            const u32 v = (u32)qv[g][i];
+            const u32 nib = hi ? ((v >> 4) & 0x0f0f0f0fu) : (v & 0x0f0f0f0fu);
+            bH[j][i] = mul_bytes(nib, mh);
+            bL[j][i] = mul_bytes(nib, ml);
         }
-        const ckq_v4i t = {(int)m[0], (int)m[1], (int)m[2], (int)m[3]};
-        bm = __builtin_bit_cast(ckq_v8bf, t);
-    }
+    };
+    decode(0);
 
+    ckq_v16i aH[2], aL[2];
+    const ckq_v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+
+    ckq_v8bf bm;
+    ckq_v4i ab[2];
+    float4 dx[4];
+    ckq_v16f i2;
+    auto combine = [&](int ts, int r) {
+        const float4 d4 = dx[r >> 2];
+        const float dxr = (r & 3) == 0 ? d4.x : (r & 3) == 1 ? d4.y : (r & 3) == 2 ? d4.z : d4.w;
+        const float f = (float)((aH[ts][r] << 3) + aL[ts][r]);
+        const float u = dw * f - dmin * i2[r];
+        acc[ts][r] += u * dxr;
+    };
+    auto load_dx = [&](int ts) {
 #pragma unroll
-    for (int ts = 0; ts < TS; ++ts) {
-        const ckq_v4i ab = *reinterpret_cast<const ckq_v4i *>(&tile.b[cur][(32 * ts + col) * 16 + 8 * half]);
+        for (int r4 = 0; r4 < 4; ++r4) dx[r4] = *reinterpret_cast<const float4 *>(&st.d[32 * ts + 8 * r4 + 4 * half]);
+    };
+    auto min_mfma = [&](int ts) {
         ckq_v16f zero;
 #pragma unroll
         for (int r = 0; r < 16; ++r) zero[r] = 0.0f;
-        const ckq_v16f i2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(ckq_v8bf, ab), bm, zero, 0, 0, 0);
-        /* fp32 combine; D layout: register r, lane l -> token row 8*(r/4) + 4*(l/32) + r%4 */
+        i2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(ckq_v8bf, ab[ts]), bm, zero, 0, 0, 0);
+    };
+
+    CKQ_PIN();
 #pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4) {
-            const float4 dx = *reinterpret_cast<const float4 *>(&tile.d[cur][32 * ts + 8 * r4 + 4 * half]);
-            const float dxs[4] = {dx.x, dx.y, dx.z, dx.w};
+    for (int s = 0; s < 16; ++s) {
+        const int ts = step_ts(s), j = step_j(s);
+        if (s + 2 < 16) av[(s + 2) % 3] = a_read(s + 2);
+        /* the first step of each token half starts from a literal zero accumulator */
+        aH[ts] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[s % 3], bH[j], (s == 0 || s == 4) ? zero16 : aH[ts], 0, 0, 0);
+        /* VALU work placed under this step's two MFMAs */
+        if (s < 3) decode(s + 1);                    /* pass 1: planes 1..3 */
+        else if (s >= 4 && s < 8) decode(s);         /* pass 2: planes 4..7 */
+        else if (s == 8) {                           /* pass 3: min operands, scales of tokens 0-31 */
+            const u32 mn03 = h2 & 0x3f3f3f3fu;
+            const u32 mn47 = ((h3 >> 4) & 0x0f0f0f0fu) | (((h2 >> 6) & 0x03030303u) << 4);
+            u32 m[4];
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const int r = 4 * r4 + k;
-                const float f = (float)((accH[ts][r] << 3) + accL[ts][r]);
-                const float u = dw * f - dmin * i2[r];
-                acc[ts][r] += u * dxs[k];
+            for (int i = 0; i < 4; ++i) {
+                const u32 src = i < 2 ? mn03 : mn47;
+                const u32 m0 = (src >> (16 * (i & 1))) & 0xff, m1 = (src >> (16 * (i & 1) + 8)) & 0xff;
+                m[i] = bf16_bits((float)m0) | (bf16_bits((float)m1) << 16);
             }
-        }
+            const ckq_v4i t = {(int)m[0], (int)m[1], (int)m[2], (int)m[3]};
+            bm = __builtin_bit_cast(ckq_v8bf, t);
+            ab[0] = lds16(reinterpret_cast<const uint8_t *>(&st.b[(col) * 16 + 8 * half]));
+            ab[1] = lds16(reinterpret_cast<const uint8_t *>(&st.b[(32 + col) * 16 + 8 * half]));
+        } else if (s == 10) load_dx(0);
+        else if (s >= 12) { combine(0, 4 * (s - 12)); combine(0, 4 * (s - 12) + 1); }
+        CKQ_PIN();
+        aL[ts] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[s % 3], bL[j], (s == 0 || s == 4) ? zero16 : aL[ts], 0, 0, 0);
+        if (s < 9) copy_one(s);                      /* one global->LDS copy of the next block per step */
+        if (s == 11) min_mfma(0);                    /* tokens 0-31 are complete after this step */
+        if (s >= 12) { combine(0, 4 * (s - 12) + 2); combine(0, 4 * (s - 12) + 3); }
+        if (s == 15) asm volatile("" : "+v"(acc[0]));   /* the combine of tokens 0-31 stays under pass 4 */
+        CKQ_PIN();
     }
+    min_mfma(1);
+    load_dx(1);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) combine(1, r);
+    asm volatile("" : "+v"(acc[1]));
+#undef CKQ_PIN
 }
 
-template <int TS, int WPE>
+template <int WPE>
 __global__ void __launch_bounds__(256, WPE) gemm_q4k_mfma_kernel(GemmArgs a)
 {
-    constexpr int BM = 32 * TS;
-    __shared__ __attribute__((aligned(16))) GemmTile<BM> tile;
+    constexpr int BM = GEMM_BM;
+    __shared__ __attribute__((aligned(16))) GemmStage stage[2];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = wave_in_block();
     const int col = lane & 31, half = lane >> 5;
 
-    /* block id -> (token tile, row tile); the token tiles of one row tile run
-     * on the same XCD (blocks are dealt round-robin to the 8 XCDs) */
     const int id = blockIdx.x, xcd = id & 7, seq = id >> 3;
     const int tt = seq % a.ntt;
     const int nt = (seq / a.ntt) * 8 + xcd;
     if (nt >= a.nnt) return;
-    const int t0 = tt * BM;
-    const int n_lane = min(nt * 128 + wave * 32 + col, a.N - 1);            /* this lane's weight row */
-    const uint8_t *wrow = a.B + (size_t)n_lane * a.nb * 144;
-    const long xstride = (long)a.nb * 292;
+    const int t0 = tt * BM, n0 = nt * GEMM_BN;
+    const u32 wstride = (u32)a.nb * 144u, xstride = (u32)a.nb * 292u;
     const int last = a.nb - 1;
+    const uint8_t *wbase = a.B + (size_t)n0 * wstride;       /* uniform */
+    const uint8_t *xbase = a.A + (size_t)t0 * xstride;       /* uniform */
 
-    /* Staging roles.  Quants: 16 consecutive lanes cover the 256 contiguous
-     * bytes of one token (coalesced), a wave covers 4 tokens per load, the
-     * block 16; BM/16 loads per thread.  Side data (block scale and the 16
-     * stored bsums): 4 lanes per token, 8 bytes of bsums each. */
-    constexpr int NQ = BM / 16;
-    const int sq_tok = tid >> 4, sq_c = tid & 15;
-    const uint8_t *sq_src[NQ];
+    /* Copy roles.  One wave instruction moves 64 x 16 bytes into 1 KiB of
+     * LDS (lane l lands at byte 16 l).  Weights: the tile's 128 blocks of 144
+     * bytes are 1152 chunks = 18 instructions, lane -> (row, ninth of the
+     * block), so 9 consecutive lanes read one block contiguously.  Quants: 4
+     * tokens per instruction, 16 lanes per token, the chunk order within a
+     * token XOR-swizzled by the token number. */
+    constexpr int NWI = 5, NQI = BM / 16;      /* per wave: 5 weight + 4 quant copies */
+    u32 wofs_g[NWI], qofs_g[NQI];
 #pragma unroll
-    for (int i = 0; i < NQ; ++i)
-        sq_src[i] = a.A + (size_t)min(t0 + sq_tok + 16 * i, a.M - 1) * xstride + 4 + 16 * sq_c;
-    const int st_tok = tid >> 2, st_q = tid & 3;                            /* BM <= 64 rows x 4 quarters */
+    for (int i = 0; i < NWI; ++i) {
+        const int chunk = min(wave + 4 * i, 17) * 64 + lane, row = min(chunk / 9, a.N - 1 - n0), part = chunk % 9;
+        wofs_g[i] = (u32)row * wstride + 16u * part;
+    }
+#pragma unroll
+    for (int i = 0; i < NQI; ++i) {
+        const int tl = 4 * (wave + 4 * i) + (lane >> 4), c = (lane & 15) ^ (tl & 15);
+        qofs_g[i] = (u32)min(tl, a.M - 1 - t0) * xstride + 4u + 16u * c;
+    }
+    const int st_tok = tid >> 2, st_q = tid & 3;
     const bool st_live = st_tok < BM;
-    const uint8_t *st_src = a.A + (size_t)min(t0 + st_tok, a.M - 1) * xstride;
-
-    u32 nq[NQ][4];   /* a block's quant bytes staged by this thread */
-    u32 nbs[2];      /* 4 stored bsums (sub-blocks 2q, 2q+1) of token st_tok */
+    const uint8_t *st_src = xbase + (size_t)min(st_tok, a.M - 1 - t0) * xstride;
+    u32 nbs[2];
     float nd = 0.f;
-    auto stage_load = [&](int b) {
-        const u32 boff = (u32)b * 292u;
-#pragma unroll
-        for (int i = 0; i < NQ; ++i) ld16<4>(nq[i], sq_src[i] + boff);
-        ld8<4>(nbs, st_src + boff + 260 + 8 * st_q);
-        nd = __builtin_bit_cast(float, ld4<4>(st_src + boff));
+
+    /* copies of block b into stage buf: the side loads (into registers) first,
+     * then nine global->LDS instructions that copy_one(i) issues one at a
+     * time so they can be spread over the MFMA steps */
+    const uint8_t *cp_w = wbase, *cp_x = xbase;
+    int cp_buf = 0;
+    auto copy_begin = [&](int b, int buf) {
+        ld8<4>(nbs, st_src + (u32)b * 292u + 260 + 8 * st_q);
+        nd = __builtin_bit_cast(float, ld4<4>(st_src + (u32)b * 292u));
+        cp_w = wbase + (u32)b * 144u;
+        cp_x = xbase + (u32)b * 292u;
+        cp_buf = buf;
     };
-    auto stage_store = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < NQ; ++i)
-            *reinterpret_cast<ckq_v4i *>(&tile.q[buf][(sq_tok + 16 * i) * GEMM_XROW + 16 * sq_c]) =
-                ckq_v4i{(int)nq[i][0], (int)nq[i][1], (int)nq[i][2], (int)nq[i][3]};
+    auto copy_one = [&](int i) {
+        if (i < NWI)      /* weight slots past 17 repeat slot 17: same bytes, no branch */
+            __builtin_amdgcn_global_load_lds((ckq_glb_void *)(cp_w + wofs_g[i]),
+                                             (ckq_lds_void *)(stage[cp_buf].w + 1024 * min(wave + 4 * i, 17)), 16, 0, 0);
+        else
+            __builtin_amdgcn_global_load_lds((ckq_glb_void *)(cp_x + qofs_g[i - NWI]),
+                                             (ckq_lds_void *)(stage[cp_buf].q + 1024 * (wave + 4 * (i - NWI))), 16, 0, 0);
+    };
+    static_assert(NWI + NQI == 9, "the pipelined block issues nine copies");
+    auto side_store = [&](int buf) {
         if (!st_live) return;
-        if (st_q == 0) tile.d[buf][st_tok] = nd;
-        /* sub-blocks j = 2q, 2q+1: B32 = bsums[2j] + bsums[2j+1] = lo + 64*hi */
+        if (st_q == 0) stage[buf].d[st_tok] = nd;
         const int b0 = (int)(int16_t)(nbs[0] & 0xffff) + (int)(int16_t)(nbs[0] >> 16);
         const int b1 = (int)(int16_t)(nbs[1] & 0xffff) + (int)(int16_t)(nbs[1] >> 16);
-        u32 *bd = reinterpret_cast<u32 *>(&tile.b[buf][st_tok * 16]);
+        u32 *bd = reinterpret_cast<u32 *>(&stage[buf].b[st_tok * 16]);
         bd[st_q]     = bf16_bits((float)(b0 & 63)) | (bf16_bits((float)(b1 & 63)) << 16);
         bd[4 + st_q] = bf16_bits((float)(64 * (b0 >> 6))) | (bf16_bits((float)(64 * (b1 >> 6))) << 16);
     };
 
-    ckq_v16f acc[TS];
+    /* read-side offsets of this lane */
+    const u32 wofs_l = (u32)(32 * wave + col) * 144u;   /* wave w owns rows 32w..32w+31 */
+    u32 aofs[8];
 #pragma unroll
-    for (int ts = 0; ts < TS; ++ts)
+    for (int j = 0; j < 8; ++j) aofs[j] = (u32)col * 256u + 16u * (u32)((2 * j + half) ^ (col & 15));
+
+    ckq_v16f acc[2];
+#pragma unroll
+    for (int ts = 0; ts < 2; ++ts)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[ts][r] = 0.0f;
 
-    /* Two weight register sets alternate; every prefetch is unconditional
-     * (block index clamped) so no set is ever a conditional copy. */
-    GemmW w0, w1;
-    stage_load(0);
-    gemm_load_w(w0, wrow, 0, half);
-    stage_store(0);
+    copy_begin(0, 0);
+#pragma unroll
+    for (int i = 0; i < NWI + NQI; ++i) copy_one(i);
+    side_store(0);
+    __builtin_amdgcn_s_waitcnt(0x0070);   /* vmcnt(0): this wave's copies have landed */
     __syncthreads();
 
-    for (int b = 0; b < a.nb; b += 2) {
-        /* issue the next block's global loads BEFORE the MFMA work of this
-         * one; the scheduling barrier keeps the compiler from sinking them
-         * down to their first use */
-        stage_load(min(b + 1, last));
-        gemm_load_w(w1, wrow, min(b + 1, last), half);
+    for (int b = 0; b < a.nb; ++b) {
+        const int cur = b & 1;
+        copy_begin(min(b + 1, last), cur ^ 1);
         __builtin_amdgcn_sched_barrier(0);
-        gemm_block<TS>(w0, tile, 0, col, half, acc);
+        gemm_block_pipe(stage[cur], wofs_l, aofs, col, half, acc, copy_one);
         __builtin_amdgcn_sched_barrier(0);
-        stage_store(1);
-        __syncthreads();
-
-        stage_load(min(b + 2, last));
-        gemm_load_w(w0, wrow, min(b + 2, last), half);
-        __builtin_amdgcn_sched_barrier(0);
-        if (b + 1 < a.nb) gemm_block<TS>(w1, tile, 1, col, half, acc);
-        __builtin_amdgcn_sched_barrier(0);
-        stage_store(0);
+        side_store(cur ^ 1);
+        __builtin_amdgcn_s_waitcnt(0x0070);
         __syncthreads();
     }
 
-    /* store: lanes 0-31 / 32-63 write 32 consecutive floats of two token rows */
-    const int n = nt * 128 + wave * 32 + col;
+    const int n = n0 + wave * 32 + col;
     if (n < a.N) {
         const float bias = a.bias ? a.bias[n] : 0.0f;
 #pragma unroll
-        for (int ts = 0; ts < TS; ++ts)
+        for (int ts = 0; ts < 2; ++ts)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int t = t0 + 32 * ts + 8 * (r >> 2) + 4 * half + (r & 3);
@@ -289,10 +319,11 @@ static int launch_gemm_q4k_mfma(const void *A, const void *B, const float *bias,
     GemmArgs g;
     g.A = (const uint8_t *)A; g.B = (const uint8_t *)B; g.bias = bias; g.C = C;
     g.M = M; g.N = N; g.nb = K / 256; g.ldc = ldc;
-    constexpr int TS = 2;
-    g.ntt = (M + 32 * TS - 1) / (32 * TS);
-    g.nnt = (N + 127) / 128;
+    /* lane offsets inside a tile are 32-bit */
+    if ((long long)g.nb * 292 * GEMM_BN >= (1ll << 31)) return (int)hipErrorInvalidValue;
+    g.ntt = (M + GEMM_BM - 1) / GEMM_BM;
+    g.nnt = (N + GEMM_BN - 1) / GEMM_BN;
     const int nnt8 = (g.nnt + 7) / 8 * 8;
-    hipLaunchKernelGGL((gemm_q4k_mfma_kernel<TS, CKQ_GEMM_WPE>), dim3(g.ntt * nnt8), dim3(256), 0, s, g);
+    hipLaunchKernelGGL((gemm_q4k_mfma_kernel<CKQ_GEMM_WPE>), dim3(g.ntt * nnt8), dim3(256), 0, s, g);
     return (int)hipGetLastError();
 }
