@@ -56,7 +56,8 @@ __device__ __forceinline__ int wave_in_block() { return __builtin_amdgcn_readfir
  * stores.
  */
 template <class F, int LPR, int PPL, int MT, int RPI, bool DUMP, int WPB, bool LDSX>
-__global__ void __launch_bounds__(64 * WPB) gemv_kernel(GemvArgs a)
+__global__ void __launch_bounds__(64 * WPB) __attribute__((amdgpu_waves_per_eu(MT == 1 && !DUMP && PPL == 1 && RPI == 1 ? 8 : 1)))
+gemv_kernel(GemvArgs a)
 {
     constexpr int SLOTS = 64 / LPR;
     extern __shared__ __attribute__((aligned(16))) uint8_t xs[];   /* LDSX: the MT activation rows */
@@ -70,19 +71,20 @@ __global__ void __launch_bounds__(64 * WPB) gemv_kernel(GemvArgs a)
     const int t0 = blockIdx.y * MT;
     const uint8_t *wbase = a.W + (size_t)wrow_c * a.wrow;                      /* uniform */
 
+    /* Every wave of the block reads the same activation rows: they are staged
+     * once in LDS instead of once per wave through the vector cache.  Their
+     * loads go out first, all at once (one round trip, they hit in L2), the
+     * weight loads follow, and only then are the staged values written. */
+    constexpr int XA = F::XBLOCK % 4 == 0 ? 4 : 2;
+    constexpr int XNT = 64 * WPB, XU = MT == 1 ? 2 : 4;
+    const uint8_t *xsrc = a.X + (size_t)t0 * a.xrow;
+    const int xbytes = (int)((long)min(MT, a.ntok - t0) * a.xrow), xn16 = xbytes >> 4;
+    u32 xv[XU][4];
     if (LDSX) {
-        /* every wave of the block reads the same activation rows: stage them
-         * once in LDS instead of once per wave through the vector cache */
-        const int ntok = min(MT, a.ntok - t0);
-        const uint8_t *src = a.X + (size_t)t0 * a.xrow;
-        if (F::XBLOCK % 4 == 0) {
-            const int n = (int)((long)ntok * a.xrow / 4);
-            for (int i = threadIdx.x; i < n; i += 64 * WPB)
-                reinterpret_cast<u32 *>(xs)[i] = reinterpret_cast<const u32 *>(src)[i];
-        } else {
-            const int n = (int)((long)ntok * a.xrow / 2);
-            for (int i = threadIdx.x; i < n; i += 64 * WPB)
-                reinterpret_cast<uint16_t *>(xs)[i] = reinterpret_cast<const uint16_t *>(src)[i];
+#pragma unroll
+        for (int u = 0; u < XU; ++u) {
+            const int i = u * XNT + (int)threadIdx.x;
+            if (i < xn16) ld16<XA>(xv[u], xsrc + 16u * (u32)i);
         }
     }
 
@@ -110,7 +112,30 @@ __global__ void __launch_bounds__(64 * WPB) gemv_kernel(GemvArgs a)
                 F::load_w(w[r][p], wbase, orow);
             }
         }
-        if (LDSX && p0 == 0) __syncthreads();
+        if (LDSX && p0 == 0) {
+            /* the staged activations' loads are older than the weight loads
+             * just issued, so waiting for them does not wait for the weights */
+#pragma unroll
+            for (int u = 0; u < XU; ++u) {
+                const int i = u * XNT + (int)threadIdx.x;
+                if (i < xn16) {
+                    u32 *d = reinterpret_cast<u32 *>(xs + 16u * (u32)i);
+                    d[0] = xv[u][0]; d[1] = xv[u][1]; d[2] = xv[u][2]; d[3] = xv[u][3];
+                }
+            }
+            for (int i = XNT * XU + (int)threadIdx.x; i < xn16; i += XNT) {     /* long token tiles */
+                u32 v[4];
+                ld16<XA>(v, xsrc + 16u * (u32)i);
+                u32 *d = reinterpret_cast<u32 *>(xs + 16u * (u32)i);
+                d[0] = v[0]; d[1] = v[1]; d[2] = v[2]; d[3] = v[3];
+            }
+            const int tail = (xbytes & 15) >> 1;      /* rows are a whole number of 2-byte units */
+            if ((int)threadIdx.x < tail) {
+                const u32 o = 16u * (u32)xn16 + 2u * threadIdx.x;
+                *reinterpret_cast<uint16_t *>(xs + o) = (uint16_t)ld2(xsrc + o);
+            }
+            __syncthreads();
+        }
 #pragma unroll
         for (int p = 0; p < PPL; ++p) {
             const int pos = min(p0 + p * LPR + l, a.npos - 1);
@@ -180,13 +205,21 @@ static int launch_tile(const GemvArgs &a, hipStream_t s)
 }
 
 /* Rows per wave-slot and waves per block for each token tile: one row per
- * slot and many waves for the bandwidth-bound single-token case (every load of
- * the matrix in flight at once), fewer rows in flight as the tile grows. */
+ * slot in 256-thread blocks for the bandwidth-bound single-token case (as many
+ * of the matrix's loads in flight as the CUs can hold, small barrier groups),
+ * fewer rows in flight as the tile grows. */
 template <class F, int LPR, int PPL>
 static int launch_mt(const GemvArgs &a, bool dump, int max_mt, hipStream_t s)
 {
     if (dump) return launch_one<F, LPR, PPL, 1, 1, true, 4, false>(a, s);
-    if (a.ntok == 1 || max_mt == 1) return launch_tile<F, LPR, PPL, 1, 1, 8>(a, s);
+    if (a.ntok == 1 || max_mt == 1) {
+        /* 256-thread blocks; a second row per slot once the matrix needs more
+         * than two rounds of resident waves anyway (halves the activation
+         * staging per weight byte) */
+        const long waves = ((long)(a.row1 - a.row0) * LPR + 63) / 64;
+        if (PPL == 1 && waves > 16384) return launch_tile<F, LPR, PPL, 1, 2, 4>(a, s);
+        return launch_tile<F, LPR, PPL, 1, 1, 4>(a, s);
+    }
     if (a.ntok == 2) return launch_tile<F, LPR, PPL, 2, 2, 4>(a, s);
     if (a.ntok <= 4) return launch_tile<F, LPR, PPL, 4, 2, 4>(a, s);
     return launch_tile<F, LPR, PPL, 8, 1, 4>(a, s);
