@@ -99,6 +99,51 @@ class Harness:
         return e0.elapsed_time(e1) * 1e-3 / steps, wall / steps
 
 
+    def time_read_floor(self, copies, nbytes, steps, warmup):
+        """Seconds per launch of the plain read kernel over the same rotated
+        weight buffers: what a launch costs that only pulls `nbytes` from HBM."""
+        torch, L = self.torch, self.L
+        sink = torch.zeros(4, dtype=torch.int32, device="cuda")
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        n = len(copies)
+
+        def run(count):
+            for i in range(count):
+                L.ckq_read_dev(ctypes.c_void_p(copies[i % n].data_ptr()), nbytes, ctypes.c_void_p(sink.data_ptr()), stream)
+
+        run(warmup)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        run(steps)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / steps
+
+    def time_sequence(self, layers, steps, warmup):
+        """layers: list of op lists (one per rotated weight set); a step is one
+        pass over one layer's ops.  Returns seconds per step."""
+        torch, P = self.torch, self.P
+        flat = [op for layer in layers for op in layer]
+        n = len(layers)
+
+        def run(count):
+            full, rest = divmod(count, n)
+            if full:
+                P.dev_matmul_sequence(flat, repeat=full)
+            for layer in layers[:rest]:
+                P.dev_matmul_sequence(layer, repeat=1)
+
+        run(warmup)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        run(steps)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / steps
+
+
 def cpu_baseline(rows, K, seconds_budget=12.0):
     """Q4_K x Q8_K GEMV on the host cores, same shape.  Uses the reference's
     own kernels (oracle/_ref, built from the reference checkout) when that
@@ -193,6 +238,7 @@ def main():
     bytes_ = gemv_bytes("q4_k", rows, K, M)
     gbs = bytes_ / sec / 1e9
     sec_hot, _ = H.time_gemv("q4_k", rows, K, M, copies[:1], xq_d, a.steps, a.warmup)
+    sec_read = H.time_read_floor(copies, len(W), min(a.steps, 500), 50)
 
     out = {
         "metric": "Q4_K GEMV GB/s (% HBM peak) at M=1; Q4_K x Q8_K GEMM TOPS at M=512",
@@ -206,6 +252,9 @@ def main():
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH},
         "pct_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
         "cache_resident_gbs": round(bytes_ / sec_hot / 1e9, 2),
+        # one launch of a kernel that only reads the same weight bytes from the same rotated buffers
+        "plain_read_same_bytes": {"us": round(sec_read * 1e6, 3), "gbs": round(len(W) / sec_read / 1e9, 1),
+                                  "gemv_over_read": round(sec / sec_read, 3)},
         "host_wall_ms_per_step": round(wall * 1e3, 6),
         "parity_norm_err": err,
     }
@@ -232,6 +281,57 @@ def main():
             extras[name] = {"gbs": round(b / s / 1e9, 1), "us": round(s * 1e6, 2), "frac_hbm": round(b / s / 1e9 / HBM_PEAK_GBS, 4)}
             del cps
             torch.cuda.empty_cache()
+        # a 7B decoder layer's projection set at M=1: Q,K,V,O (4096x4096 Q4_K), gate, up
+        # (11008x4096 Q4_K), down (4096x11008 Q6_K), one C call per layer, weights of
+        # successive steps distinct (4 rotated layers = 502 MB)
+        x4k = P.dev_quantize(P.to_device(T.normal(4096, seed=31)), "q8_k")
+        x11k = P.dev_quantize(P.to_device(T.normal(11008, seed=32)), "q8_k")
+        layers, keep, lbytes = [], [], 0
+        for li in range(4):
+            ops = []
+            for j, (fmt, r, k) in enumerate([("q4_k", 4096, 4096)] * 4 + [("q4_k", 11008, 4096)] * 2 + [("q6_k", 4096, 11008)]):
+                Wj = torch.from_numpy(T.synth_weights(fmt, r, k, seed=1000 + j)).cuda()
+                if li:
+                    Wj = torch.roll(Wj.view(r, -1), shifts=li * 13 + j, dims=0).contiguous().reshape(-1)
+                o = torch.empty(r, dtype=torch.float32, device="cuda")
+                keep += [Wj, o]
+                ops.append((fmt, x11k if k == 11008 else x4k, Wj, None, o, 1, r, k))
+                if li == 0:
+                    lbytes += gemv_bytes(fmt, r, k)
+            layers.append(ops)
+        s = H.time_sequence(layers, max(40, a.steps // 10), 8)
+        extras["layer_7b_projection_set_M1"] = {"us": round(s * 1e6, 2), "gbs": round(lbytes / s / 1e9, 1), "bytes": lbytes,
+                                                "frac_hbm": round(lbytes / s / 1e9 / HBM_PEAK_GBS, 4), "launches": 7}
+        del layers, keep
+        torch.cuda.empty_cache()
+
+        # small-model batched decode (Qwen2-0.5B-like: hidden 896 padded to K=1024, Q5_K
+        # projections, Q8_0 LM head 151936x896), M tokens per step
+        proj = [(896, 1024), (128, 1024), (128, 1024), (896, 1024), (4864, 1024), (4864, 1024), (896, 4864)]
+        Wp = [torch.from_numpy(T.synth_weights("q5_k", r, k, seed=2000 + i)).cuda() for i, (r, k) in enumerate(proj)]
+        _, heads = H.weight_copies("q8_0", 151936, 896, seed=2100, min_total=2 * MALL_BYTES)
+        small = {}
+        for Mb in (1, 2, 4, 8):
+            xa = P.dev_quantize(P.to_device(T.normal(Mb * 1024, seed=41)), "q8_k", rows=Mb)
+            xb = P.dev_quantize(P.to_device(T.normal(Mb * 4864, seed=42)), "q8_k", rows=Mb)
+            xh = P.dev_quantize(P.to_device(T.normal(Mb * 896, seed=43)), "q8_0", rows=Mb)
+            layers, nbytes = [], 0
+            for hi, head in enumerate(heads):
+                ops = []
+                for (r, k), Wj in zip(proj, Wp):
+                    ops.append(("q5_k", xb if k == 4864 else xa, Wj, None, torch.empty(Mb * r, dtype=torch.float32, device="cuda"), Mb, r, k))
+                    if hi == 0:
+                        nbytes += gemv_bytes("q5_k", r, k, Mb)
+                ops.append(("q8_0", xh, head, None, torch.empty(Mb * 151936, dtype=torch.float32, device="cuda"), Mb, 151936, 896))
+                if hi == 0:
+                    nbytes += gemv_bytes("q8_0", 151936, 896, Mb)
+                layers.append(ops)
+            s = H.time_sequence(layers, max(20, a.steps // 40), 4)
+            small["M%d" % Mb] = {"us": round(s * 1e6, 2), "gbs": round(nbytes / s / 1e9, 1), "tokens_per_s": round(Mb / s, 1)}
+            del layers
+        extras["small_model_decode_q5_k_layer_plus_q8_0_head"] = small
+        del heads, Wp
+        torch.cuda.empty_cache()
         out["extras"] = extras
 
     if not a.no_cpu:

@@ -690,3 +690,8 @@ int ckq_copy_dev(void *dst, const void *src, size_t bytes, void *stream)
 {
     return ckq_launch_copy(dst, src, bytes, stream);
 }
+
+int ckq_read_dev(const void *src, size_t bytes, void *sink, void *stream)
+{
+    return ckq_launch_read(src, bytes, sink, stream);
+}

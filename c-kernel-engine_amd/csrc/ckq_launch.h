@@ -41,6 +41,7 @@ int ckq_launch_quantize_q8_0(const float *x, void *y, int rows, int k, void *str
 
 /* Plain device copy kernel (calibration of the memory counters / roofline). */
 int ckq_launch_copy(void *dst, const void *src, size_t bytes, void *stream);
+int ckq_launch_read(const void *src, size_t bytes, void *sink, void *stream);
 
 #ifdef __cplusplus
 }

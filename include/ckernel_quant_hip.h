@@ -157,6 +157,12 @@ int ckq_subblock_dots_dev(int fmt, int32_t *out, const void *W, const void *x_q8
  * memory counters. */
 int ckq_copy_dev(void *dst, const void *src, size_t bytes, void *stream);
 
+/* Streaming device read of the first `bytes & ~15` bytes of src, results
+ * discarded (`sink`: 4 writable device bytes that stay untouched).  One launch
+ * of it is the time floor of a GEMV whose weights are `bytes` large; the
+ * benchmark reports it beside the GEMV figure. */
+int ckq_read_dev(const void *src, size_t bytes, void *sink, void *stream);
+
 /* ======================================================================== */
 /* Library control                                                           */
 /* ======================================================================== */
