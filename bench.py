@@ -281,6 +281,25 @@ def main():
             extras[name] = {"gbs": round(b / s / 1e9, 1), "us": round(s * 1e6, 2), "frac_hbm": round(b / s / 1e9 / HBM_PEAK_GBS, 4)}
             del cps
             torch.cuda.empty_cache()
+        # fp32-activation entry point (gemv_q4_k: weights dequantized on the fly, nothing quantized)
+        xf_d = P.to_device(xf)
+        outf = torch.empty(rows, dtype=torch.float32, device="cuda")
+        for c in copies[:4]:
+            P.dev_gemm_nt_f32act("q4_k", xf_d, c, None, 1, rows, K, out=outf)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        nf = 64 * len(copies)
+        e0.record()
+        for i in range(nf):
+            P.dev_gemm_nt_f32act("q4_k", xf_d, copies[i % len(copies)], None, 1, rows, K, out=outf)
+        e1.record()
+        torch.cuda.synchronize()
+        sf = e0.elapsed_time(e1) * 1e-3 / nf
+        bf = len(W) + 4 * K + 4 * rows
+        extras["gemv_q4_k_f32act_11008x4096"] = {"gbs": round(bf / sf / 1e9, 1), "us": round(sf * 1e6, 2),
+                                                 "frac_hbm": round(bf / sf / 1e9 / HBM_PEAK_GBS, 4),
+                                                 "note": "launched from Python one call at a time"}
+
         # a 7B decoder layer's projection set at M=1: Q,K,V,O (4096x4096 Q4_K), gate, up
         # (11008x4096 Q4_K), down (4096x11008 Q6_K), one C call per layer, weights of
         # successive steps distinct (4 rotated layers = 502 MB)

@@ -65,6 +65,15 @@ _SIGS = {
     "gemv_q8_0_q8_0_parallel_simd": (None, [_vp, _vp, _vp, _i, _i, _i, _i]),
     "gemv_q8_0": (None, [_vp, _vp, _vp, _i, _i]),
     "gemm_nt_q8_0_q8_0": (None, [_vp, _vp, _vp, _vp, _i, _i, _i]),
+    "gemv_q4_k": (None, [_vp, _vp, _vp, _i, _i]),
+    "gemm_q4_k": (None, [_vp, _vp, _vp, _i, _i, _i]),
+    "gemm_nt_q4_k": (None, [_vp, _vp, _vp, _vp, _i, _i, _i]),
+    "dot_q4_k": (_c.c_float, [_vp, _vp, _i]),
+    "gemv_q6_k": (None, [_vp, _vp, _vp, _i, _i]),
+    "gemm_q6_k": (None, [_vp, _vp, _vp, _i, _i, _i]),
+    "gemm_nt_q6_k": (None, [_vp, _vp, _vp, _vp, _i, _i, _i]),
+    "gemm_q8_0": (None, [_vp, _vp, _vp, _i, _i, _i]),
+    "gemm_nt_q8_0": (None, [_vp, _vp, _vp, _vp, _i, _i, _i]),
     "ck_test_quantize_q8_k": (None, [_vp, _vp, _i]),
     "ck_test_gemv_q4_k": (None, [_vp, _vp, _vp, _i]),
     "ck_test_gemv_q6_k": (None, [_vp, _vp, _vp, _i]),
@@ -90,6 +99,7 @@ _SIGS = {
     "ckq_gemm_nt_q5_k_q8_k_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "ckq_gemm_nt_q6_k_q8_k_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "ckq_gemm_nt_q8_0_q8_0_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "ckq_gemm_nt_f32act_dev": (_i, [_i, _vp, _vp, _vp, _vp, _i, _i, _i, _c.c_long, _vp]),
     "ckq_matmul_sequence_dev": (_i, [_vp, _i, _i, _vp]),
     "ckq_subblock_dots_dev": (_i, [_i, _vp, _vp, _vp, _i, _i, _vp]),
     "ckq_copy_dev": (_i, [_vp, _vp, _c.c_size_t, _vp]),
@@ -122,7 +132,7 @@ def declared_symbols():
     text = open(HEADER).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     text = re.sub(r"typedef\s+struct\s*\{.*?\}\s*\w+;", "", text, flags=re.S)
-    names = re.findall(r"^\s*(?:const\s+)?(?:void|int|char)\s*\*?\s*(\w+)\s*\(", text, flags=re.M)
+    names = re.findall(r"^\s*(?:const\s+)?(?:void|int|char|float)\s*\*?\s*(\w+)\s*\(", text, flags=re.M)
     return sorted(set(names))
 
 

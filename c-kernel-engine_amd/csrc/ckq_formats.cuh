@@ -47,6 +47,8 @@ __device__ __forceinline__ void k4_scale_pair(u32 u0, u32 u1, u32 u2, int g, u32
 /* ------------------------------------------------------------------------- */
 struct FmtQ4K {
     static constexpr int POS_PER_BLOCK = 4, WBLOCK = 144, XBLOCK = 292, NSUB = 2;
+    static constexpr int OCC1 = 8;            /* waves per SIMD the one-token kernel is held to */
+    static constexpr bool TOKEN_TILES = true; /* tiles of 2, 4 and 8 tokens exist */
     struct Wt  { u32 hdr[4]; u32 qs[8]; };
     struct Act { int q[16]; float d; int b_lo, b_hi; };
     struct Dec { int lo[8], hi[8]; int sc_lo, sc_hi, mn_lo, mn_hi; float d, dmin; };
@@ -77,6 +79,9 @@ struct FmtQ4K {
         a.b_lo = (int)(int16_t)(bs[0] & 0xffff) + (int)(int16_t)(bs[0] >> 16);
         a.b_hi = (int)(int16_t)(bs[1] & 0xffff) + (int)(int16_t)(bs[1] >> 16);
     }
+    /* LDS image of the staged activations: 16-byte unit u of the rows sits at unit xs_unit(u) */
+    static __device__ __forceinline__ u32 xs_unit(u32 u) { return u; }
+    static __device__ __forceinline__ void load_act_lds(Act &a, const uint8_t *xs, int pos) { load_act(a, xs, pos); }
     static __device__ __forceinline__ void decode(Dec &d, const Wt &w, int pos)
     {
         u32 sc2, mn2;
@@ -110,6 +115,8 @@ struct FmtQ4K {
 /* ------------------------------------------------------------------------- */
 struct FmtQ5K {
     static constexpr int POS_PER_BLOCK = 4, WBLOCK = 176, XBLOCK = 292, NSUB = 2;
+    static constexpr int OCC1 = 8;            /* waves per SIMD the one-token kernel is held to */
+    static constexpr bool TOKEN_TILES = true; /* tiles of 2, 4 and 8 tokens exist */
     struct Wt  { u32 hdr[4]; u32 qh[8]; u32 qs[8]; };
     typedef FmtQ4K::Act Act;
     typedef FmtQ4K::Dec Dec;
@@ -132,6 +139,9 @@ struct FmtQ5K {
         ld16<4>(w.qs + 4, row + o.qs + 16);
     }
     static __device__ __forceinline__ void load_act(Act &a, const uint8_t *x, int pos) { FmtQ4K::load_act(a, x, pos); }
+    /* LDS image of the staged activations: 16-byte unit u of the rows sits at unit xs_unit(u) */
+    static __device__ __forceinline__ u32 xs_unit(u32 u) { return u; }
+    static __device__ __forceinline__ void load_act_lds(Act &a, const uint8_t *xs, int pos) { load_act(a, xs, pos); }
     static __device__ __forceinline__ void decode(Dec &d, const Wt &w, int pos)
     {
         const int g = pos & 3;
@@ -155,6 +165,8 @@ struct FmtQ5K {
 /* ------------------------------------------------------------------------- */
 struct FmtQ6K {
     static constexpr int POS_PER_BLOCK = 4, WBLOCK = 210, XBLOCK = 292, NSUB = 4;
+    static constexpr int OCC1 = 8;            /* waves per SIMD the one-token kernel is held to */
+    static constexpr bool TOKEN_TILES = true; /* tiles of 2, 4 and 8 tokens exist */
     struct Wt  { u32 ql0[4], ql1[4], qh[4]; u32 sc[2]; u32 d; };
     struct Act { int q[16]; float d; int a32[4]; };      /* a32[r] = 32 * sum of the run's 16 quants */
     struct Dec { int q[16]; int sc[4]; float d; };
@@ -192,6 +204,9 @@ struct FmtQ6K {
             a.a32[r] = 32 * s;   /* computed from the quants: the reference's x86 routine never reads bsums here */
         }
     }
+    /* LDS image of the staged activations: 16-byte unit u of the rows sits at unit xs_unit(u) */
+    static __device__ __forceinline__ u32 xs_unit(u32 u) { return u; }
+    static __device__ __forceinline__ void load_act_lds(Act &a, const uint8_t *xs, int pos) { load_act(a, xs, pos); }
     static __device__ __forceinline__ void decode(Dec &d, const Wt &w, int pos)
     {
         const int odd = pos & 1;
@@ -231,6 +246,8 @@ struct FmtQ6K {
 /* ------------------------------------------------------------------------- */
 struct FmtQ80 {
     static constexpr int POS_PER_BLOCK = 1, WBLOCK = 34, XBLOCK = 34, NSUB = 1;
+    static constexpr int OCC1 = 8;            /* waves per SIMD the one-token kernel is held to */
+    static constexpr bool TOKEN_TILES = true; /* tiles of 2, 4 and 8 tokens exist */
     struct Wt  { u32 q[8]; u32 d; };
     struct Act { int q[8]; float d; };
     struct Dec { int q[8]; float d; };
@@ -256,6 +273,9 @@ struct FmtQ80 {
         ld16<2>(a.q, blk + 2);
         ld16<2>(a.q + 4, blk + 18);
     }
+    /* LDS image of the staged activations: 16-byte unit u of the rows sits at unit xs_unit(u) */
+    static __device__ __forceinline__ u32 xs_unit(u32 u) { return u; }
+    static __device__ __forceinline__ void load_act_lds(Act &a, const uint8_t *xs, int pos) { load_act(a, xs, pos); }
     static __device__ __forceinline__ void decode(Dec &d, const Wt &w, int)
     {
         for (int i = 0; i < 8; ++i) d.q[i] = (int)w.q[i];
@@ -275,6 +295,8 @@ struct FmtQ80 {
 /* Q8_0 weights against fp32 activations (no activation quantization). */
 struct FmtQ80F32 {
     static constexpr int POS_PER_BLOCK = 1, WBLOCK = 34, XBLOCK = 128, NSUB = 1;
+    static constexpr int OCC1 = 4;            /* 64 activation floats per lane: 128 registers */
+    static constexpr bool TOKEN_TILES = false;
     typedef FmtQ80::Wt Wt;
     typedef FmtQ80::Dec Dec;
     struct Act { float x[32]; };
@@ -292,6 +314,17 @@ struct FmtQ80F32 {
             for (int j = 0; j < 4; ++j) a.x[4 * i + j] = __builtin_bit_cast(float, t[j]);
         }
     }
+    /* A lane reads a run of consecutive 16-byte units; lanes are 128 bytes
+     * apart, so unswizzled they would all hit the same LDS banks. */
+    static __device__ __forceinline__ u32 xs_unit(u32 u) { return u ^ ((u >> 4) & 15u); }
+    static __device__ __forceinline__ void load_act_lds(Act &a, const uint8_t *xs, int pos)
+    {
+        for (int i = 0; i < 8; ++i) {
+            u32 t[4];
+            ld16<4>(t, xs + 16u * xs_unit(8u * (u32)pos + i));
+            for (int j = 0; j < 4; ++j) a.x[4 * i + j] = __builtin_bit_cast(float, t[j]);
+        }
+    }
     static __device__ __forceinline__ void decode(Dec &d, const Wt &w, int pos) { FmtQ80::decode(d, w, pos); }
     static __device__ __forceinline__ float dot(const Dec &d, const Act &a, int *sub)
     {
@@ -303,4 +336,110 @@ struct FmtQ80F32 {
     }
     static __device__ __forceinline__ int sub_index(int pos, int) { return pos; }
     static constexpr int SUBS_PER_BLOCK = 1;
+};
+
+/* Q4_K weights against fp32 activations (no activation quantization):
+ * sum (d*sc*q - dmin*m) * x (reference: gemm_kernels_q4k.c:53-101). */
+struct FmtQ4KF32 {
+    static constexpr int POS_PER_BLOCK = 4, WBLOCK = 144, XBLOCK = 1024, NSUB = 1;
+    static constexpr int OCC1 = 4;            /* 64 activation floats per lane: 128 registers */
+    static constexpr bool TOKEN_TILES = false;
+    typedef FmtQ4K::Wt Wt;
+    typedef FmtQ4K::Dec Dec;
+    struct Act { float x[64]; };
+
+    typedef FmtQ4K::Off Off;
+    static __device__ __forceinline__ Off w_off(int pos) { return FmtQ4K::w_off(pos); }
+    static __device__ __forceinline__ void off_shift(Off &o, u32 s) { FmtQ4K::off_shift(o, s); }
+    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, const Off &o) { FmtQ4K::load_w(w, row, o); }
+    static __device__ __forceinline__ void load_act(Act &a, const uint8_t *x, int pos)
+    {
+        const uint8_t *p = x + (u32)pos * 256u;      /* 64 floats per position */
+        for (int i = 0; i < 16; ++i) {
+            u32 t[4];
+            ld16<4>(t, p + 16 * i);
+            for (int j = 0; j < 4; ++j) a.x[4 * i + j] = __builtin_bit_cast(float, t[j]);
+        }
+    }
+    /* lanes are 256 bytes apart: swizzle the unit index so 16 lanes reading
+     * their i-th unit touch 16 different bank groups */
+    static __device__ __forceinline__ u32 xs_unit(u32 u) { return u ^ ((u >> 4) & 15u); }
+    static __device__ __forceinline__ void load_act_lds(Act &a, const uint8_t *xs, int pos)
+    {
+        for (int i = 0; i < 16; ++i) {
+            u32 t[4];
+            ld16<4>(t, xs + 16u * xs_unit(16u * (u32)pos + i));
+            for (int j = 0; j < 4; ++j) a.x[4 * i + j] = __builtin_bit_cast(float, t[j]);
+        }
+    }
+    static __device__ __forceinline__ void decode(Dec &d, const Wt &w, int pos) { FmtQ4K::decode(d, w, pos); }
+    static __device__ __forceinline__ float dot(const Dec &d, const Act &a, int *sub)
+    {
+        const float d1 = d.d * (float)d.sc_lo, m1 = d.dmin * (float)d.mn_lo;
+        const float d2 = d.d * (float)d.sc_hi, m2 = d.dmin * (float)d.mn_hi;
+        float s = 0.0f;
+        for (int i = 0; i < 8; ++i)
+            for (int j = 0; j < 4; ++j) {
+                s += (d1 * (float)((d.lo[i] >> (8 * j)) & 0xff) - m1) * a.x[4 * i + j];
+                s += (d2 * (float)((d.hi[i] >> (8 * j)) & 0xff) - m2) * a.x[32 + 4 * i + j];
+            }
+        sub[0] = 0;
+        return s;
+    }
+    static __device__ __forceinline__ int sub_index(int pos, int) { return pos; }
+    static constexpr int SUBS_PER_BLOCK = 4;
+};
+
+/* Q6_K weights against fp32 activations: sum (d*sc*(q-32)) * x
+ * (reference: gemm_kernels_q6k.c:39-76). */
+struct FmtQ6KF32 {
+    static constexpr int POS_PER_BLOCK = 4, WBLOCK = 210, XBLOCK = 1024, NSUB = 1;
+    static constexpr int OCC1 = 4;            /* 64 activation floats per lane: 128 registers */
+    static constexpr bool TOKEN_TILES = false;
+    typedef FmtQ6K::Wt Wt;
+    typedef FmtQ6K::Dec Dec;
+    struct Act { float x[64]; };                     /* four runs of 16: elements 128n + 32r + 16*odd + i */
+
+    typedef FmtQ6K::Off Off;
+    static __device__ __forceinline__ Off w_off(int pos) { return FmtQ6K::w_off(pos); }
+    static __device__ __forceinline__ void off_shift(Off &o, u32 s) { FmtQ6K::off_shift(o, s); }
+    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, const Off &o) { FmtQ6K::load_w(w, row, o); }
+    static __device__ __forceinline__ void load_act(Act &a, const uint8_t *x, int pos)
+    {
+        const int n = (pos >> 1) & 1, l0 = 16 * (pos & 1);
+        const uint8_t *blk = x + (u32)(pos >> 2) * 1024u + 4u * (u32)(128 * n + l0);
+        for (int r = 0; r < 4; ++r)
+            for (int i = 0; i < 4; ++i) {
+                u32 t[4];
+                ld16<4>(t, blk + 128 * r + 16 * i);
+                for (int j = 0; j < 4; ++j) a.x[16 * r + 4 * i + j] = __builtin_bit_cast(float, t[j]);
+            }
+    }
+    static __device__ __forceinline__ u32 xs_unit(u32 u) { return u ^ ((u >> 4) & 15u); }
+    static __device__ __forceinline__ void load_act_lds(Act &a, const uint8_t *xs, int pos)
+    {
+        const int n = (pos >> 1) & 1, l0 = 16 * (pos & 1);
+        const u32 u0 = 64u * (u32)(pos >> 2) + (u32)(128 * n + l0) / 4u;      /* unit of the first float */
+        for (int r = 0; r < 4; ++r)
+            for (int i = 0; i < 4; ++i) {
+                u32 t[4];
+                ld16<4>(t, xs + 16u * xs_unit(u0 + 8u * r + i));
+                for (int j = 0; j < 4; ++j) a.x[16 * r + 4 * i + j] = __builtin_bit_cast(float, t[j]);
+            }
+    }
+    static __device__ __forceinline__ void decode(Dec &d, const Wt &w, int pos) { FmtQ6K::decode(d, w, pos); }
+    static __device__ __forceinline__ float dot(const Dec &d, const Act &a, int *sub)
+    {
+        float s = 0.0f;
+        for (int r = 0; r < 4; ++r) {
+            const float ds = d.d * (float)d.sc[r];
+            for (int i = 0; i < 4; ++i)
+                for (int j = 0; j < 4; ++j)
+                    s += (ds * (float)(((d.q[4 * r + i] >> (8 * j)) & 0xff) - 32)) * a.x[16 * r + 4 * i + j];
+        }
+        sub[0] = 0;
+        return s;
+    }
+    static __device__ __forceinline__ int sub_index(int pos, int) { return pos; }
+    static constexpr int SUBS_PER_BLOCK = 4;
 };

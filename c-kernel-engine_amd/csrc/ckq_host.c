@@ -335,14 +335,22 @@ void ckq_set_parallel_whole(int enabled)
 
 static int fmt_block_elems(int fmt) { return (fmt == CKQ_FMT_Q8_0 || fmt == CKQ_KERNEL_Q80_F32) ? 32 : 256; }
 
+static int is_f32act(int fmt) { return fmt == CKQ_KERNEL_Q80_F32 || fmt == CKQ_KERNEL_Q4K_F32 || fmt == CKQ_KERNEL_Q6K_F32; }
+
+static int weight_fmt(int fmt)
+{
+    return fmt == CKQ_KERNEL_Q80_F32 ? CKQ_FMT_Q8_0 : fmt == CKQ_KERNEL_Q4K_F32 ? CKQ_FMT_Q4_K
+         : fmt == CKQ_KERNEL_Q6K_F32 ? CKQ_FMT_Q6_K : fmt;
+}
+
 static size_t weight_row_bytes(int fmt, int K)
 {
-    return ckq_row_bytes(fmt == CKQ_KERNEL_Q80_F32 ? CKQ_FMT_Q8_0 : fmt, K);
+    return ckq_row_bytes(weight_fmt(fmt), K);
 }
 
 static size_t act_row_bytes(int fmt, int K)
 {
-    if (fmt == CKQ_KERNEL_Q80_F32) return (size_t)K * 4;
+    if (is_f32act(fmt)) return (size_t)K * 4;
     if (fmt == CKQ_FMT_Q8_0) return ckq_row_bytes(CKQ_FMT_Q8_0, K);
     return ckq_row_bytes(CKQ_FMT_Q8_K, K);
 }
@@ -577,6 +585,54 @@ void gemm_nt_q8_0_q8_0(const void *A_q8, const void *B, const float *bias, float
     host_matmul(CKQ_FMT_Q8_0, A_q8, B, bias, C, M, N, K, N, 0, N);
 }
 
+/* fp32 activations used as they are (no activation quantization). */
+void gemv_q4_k(float *y, const void *W, const float *x, int M, int K)
+{
+    host_matmul(CKQ_KERNEL_Q4K_F32, x, W, NULL, y, 1, M, K, M, 0, M);
+}
+
+void gemm_q4_k(float *Y, const void *W, const float *X, int M, int N, int K)
+{
+    host_matmul(CKQ_KERNEL_Q4K_F32, X, W, NULL, Y, N, M, K, M, 0, M);
+}
+
+void gemm_nt_q4_k(const float *A, const void *B, const float *bias, float *C, int M, int N, int K)
+{
+    host_matmul(CKQ_KERNEL_Q4K_F32, A, B, bias, C, M, N, K, N, 0, N);
+}
+
+float dot_q4_k(const void *w_q4k, const float *x, int K)
+{
+    float r = 0.0f;
+    gemv_q4_k(&r, w_q4k, x, 1, K);
+    return r;
+}
+
+void gemv_q6_k(float *y, const void *W, const float *x, int M, int K)
+{
+    host_matmul(CKQ_KERNEL_Q6K_F32, x, W, NULL, y, 1, M, K, M, 0, M);
+}
+
+void gemm_q6_k(float *Y, const void *W, const float *X, int M, int N, int K)
+{
+    host_matmul(CKQ_KERNEL_Q6K_F32, X, W, NULL, Y, N, M, K, M, 0, M);
+}
+
+void gemm_nt_q6_k(const float *A, const void *B, const float *bias, float *C, int M, int N, int K)
+{
+    host_matmul(CKQ_KERNEL_Q6K_F32, A, B, bias, C, M, N, K, N, 0, N);
+}
+
+void gemm_q8_0(float *Y, const void *W, const float *X, int M, int N, int K)
+{
+    host_matmul(CKQ_KERNEL_Q80_F32, X, W, NULL, Y, N, M, K, M, 0, M);
+}
+
+void gemm_nt_q8_0(const float *A, const void *B, const float *bias, float *C, int M, int N, int K)
+{
+    host_matmul(CKQ_KERNEL_Q80_F32, A, B, bias, C, M, N, K, N, 0, N);
+}
+
 /* Parity-test wrappers (reference: src/ck_parity_api.c). */
 void ck_test_quantize_q8_k(const float *src, void *dst, int n) { quantize_row_q8_k(src, dst, n); }
 
@@ -665,6 +721,15 @@ DEFINE_DEV(q8_0_q8_0, CKQ_FMT_Q8_0)
 int ckq_gemv_q8_0_dev(float *y, const void *W, const float *x, int M, int K, void *stream)
 {
     return ckq_launch_gemv(CKQ_KERNEL_Q80_F32, y, W, x, NULL, M, K, 1, M, 0, M, NULL, stream);
+}
+
+int ckq_gemm_nt_f32act_dev(int fmt, const float *A, const void *B, const float *bias, float *C,
+                           int M, int N, int K, long ldc, void *stream)
+{
+    const int k = fmt == CKQ_FMT_Q4_K ? CKQ_KERNEL_Q4K_F32 : fmt == CKQ_FMT_Q6_K ? CKQ_KERNEL_Q6K_F32
+                : fmt == CKQ_FMT_Q8_0 ? CKQ_KERNEL_Q80_F32 : -1;
+    if (k < 0) return CKQ_EFORMAT;
+    return ckq_launch_gemv(k, C, B, A, bias, N, K, M, ldc, 0, N, NULL, stream);
 }
 
 int ckq_matmul_sequence_dev(const ckq_matmul_op *ops, int nops, int repeat, void *stream)

@@ -57,7 +57,7 @@ __device__ __forceinline__ int wave_in_block() { return __builtin_amdgcn_readfir
  * stores.
  */
 template <class F, int LPR, int PPL, int MT, int RPI, bool DUMP, int WPB, bool LDSX>
-__global__ void __launch_bounds__(64 * WPB) __attribute__((amdgpu_waves_per_eu(MT == 1 && !DUMP && PPL == 1 && RPI == 1 ? 8 : 1)))
+__global__ void __launch_bounds__(64 * WPB) __attribute__((amdgpu_waves_per_eu(MT == 1 && !DUMP && PPL == 1 && RPI == 1 ? F::OCC1 : 1)))
 gemv_kernel(GemvArgs a)
 {
     constexpr int SLOTS = 64 / LPR;
@@ -120,14 +120,14 @@ gemv_kernel(GemvArgs a)
             for (int u = 0; u < XU; ++u) {
                 const int i = u * XNT + (int)threadIdx.x;
                 if (i < xn16) {
-                    u32 *d = reinterpret_cast<u32 *>(xs + 16u * (u32)i);
+                    u32 *d = reinterpret_cast<u32 *>(xs + 16u * F::xs_unit((u32)i));
                     d[0] = xv[u][0]; d[1] = xv[u][1]; d[2] = xv[u][2]; d[3] = xv[u][3];
                 }
             }
             for (int i = XNT * XU + (int)threadIdx.x; i < xn16; i += XNT) {     /* long token tiles */
                 u32 v[4];
                 ld16<XA>(v, xsrc + 16u * (u32)i);
-                u32 *d = reinterpret_cast<u32 *>(xs + 16u * (u32)i);
+                u32 *d = reinterpret_cast<u32 *>(xs + 16u * F::xs_unit((u32)i));
                 d[0] = v[0]; d[1] = v[1]; d[2] = v[2]; d[3] = v[3];
             }
             const int tail = (xbytes & 15) >> 1;      /* rows are a whole number of 2-byte units */
@@ -144,7 +144,7 @@ gemv_kernel(GemvArgs a)
             for (int t = 0; t < MT; ++t) {
                 if (LDSX) {
                     const int tl = min(t, a.ntok - t0 - 1);                    /* uniform */
-                    F::load_act(act[t][p], xs + (u32)tl * (u32)a.xrow, pos);
+                    F::load_act_lds(act[t][p], xs + (u32)tl * (u32)a.xrow, pos);
                 } else {
                     const int tok = min(t0 + t, a.ntok - 1);                   /* uniform */
                     F::load_act(act[t][p], a.X + (size_t)tok * a.xrow, pos);
@@ -192,7 +192,8 @@ static int launch_one(const GemvArgs &a, hipStream_t s)
     constexpr int rows_per_block = WPB * (64 / LPR) * RPI;
     const int nr = a.row1 - a.row0;
     dim3 grid((nr + rows_per_block - 1) / rows_per_block, (a.ntok + MT - 1) / MT);
-    const size_t lds = LDSX ? (size_t)MT * (size_t)a.xrow : 0;
+    /* whole 256-byte groups: a format may permute the 16-byte units inside one */
+    const size_t lds = LDSX ? (((size_t)MT * (size_t)a.xrow + 255) & ~(size_t)255) : 0;
     hipLaunchKernelGGL((gemv_kernel<F, LPR, PPL, MT, RPI, DUMP, WPB, LDSX>), grid, dim3(64 * WPB), lds, s, a);
     return (int)hipGetLastError();
 }
@@ -212,7 +213,10 @@ static int launch_tile(const GemvArgs &a, hipStream_t s)
 template <class F, int LPR, int PPL>
 static int launch_mt(const GemvArgs &a, bool dump, int max_mt, hipStream_t s)
 {
-    if (dump) return launch_one<F, LPR, PPL, 1, 1, true, 4, false>(a, s);
+    if (dump) {
+        if constexpr (F::TOKEN_TILES) return launch_one<F, LPR, PPL, 1, 1, true, 4, false>(a, s);
+        return CKQ_EINVAL;
+    }
     if (a.ntok == 1 || max_mt == 1) {
         /* 256-thread blocks; a second row per slot once the matrix needs more
          * than two rounds of resident waves anyway (halves the activation
@@ -221,9 +225,12 @@ static int launch_mt(const GemvArgs &a, bool dump, int max_mt, hipStream_t s)
         if (PPL == 1 && waves > 16384) return launch_tile<F, LPR, PPL, 1, 2, 4>(a, s);
         return launch_tile<F, LPR, PPL, 1, 1, 4>(a, s);
     }
-    if (a.ntok == 2) return launch_tile<F, LPR, PPL, 2, 2, 4>(a, s);
-    if (a.ntok <= 4) return launch_tile<F, LPR, PPL, 4, 2, 4>(a, s);
-    return launch_tile<F, LPR, PPL, 8, 2, 4>(a, s);   /* two rows per slot: the staged tile serves twice the weights */
+    if constexpr (F::TOKEN_TILES) {
+        if (a.ntok == 2) return launch_tile<F, LPR, PPL, 2, 2, 4>(a, s);
+        if (a.ntok <= 4) return launch_tile<F, LPR, PPL, 4, 2, 4>(a, s);
+        return launch_tile<F, LPR, PPL, 8, 2, 4>(a, s);   /* two rows per slot: the staged tile serves twice the weights */
+    }
+    return CKQ_EINVAL;   /* formats without token tiles are always launched with max_mt == 1 */
 }
 
 template <class F>
@@ -278,6 +285,16 @@ extern "C" int ckq_launch_gemv(int fmt, float *y, const void *W, const void *X, 
         if (dump) return CKQ_EINVAL;
         a.npos = K / 32; a.wrow = (long)(K / 32) * 34; a.xrow = (long)K * 4; a.nsub_row = K / 32;
         return launch_fmt<FmtQ80F32>(a, false, 1, s);
+    case CKQ_KERNEL_Q4K_F32:
+        if (K % 256) return CKQ_ESHAPE;
+        if (dump) return CKQ_EINVAL;
+        a.npos = K / 64; a.wrow = (long)(K / 256) * 144; a.xrow = (long)K * 4; a.nsub_row = K / 64;
+        return launch_fmt<FmtQ4KF32>(a, false, 1, s);
+    case CKQ_KERNEL_Q6K_F32:
+        if (K % 256) return CKQ_ESHAPE;
+        if (dump) return CKQ_EINVAL;
+        a.npos = K / 64; a.wrow = (long)(K / 256) * 210; a.xrow = (long)K * 4; a.nsub_row = K / 64;
+        return launch_fmt<FmtQ6KF32>(a, false, 1, s);
     default:
         return CKQ_EFORMAT;
     }

@@ -19,8 +19,11 @@ extern "C" {
 #define CKQ_ESHAPE  (-2)  /* K not a multiple of the block size */
 #define CKQ_EFORMAT (-3)  /* unknown format tag */
 
-/* Weight-format tags as in ckq_blocks.h, plus the fp32-activation variant. */
+/* Weight-format tags as in ckq_blocks.h, plus the fp32-activation variants
+ * (X is then ntok rows of K floats). */
 #define CKQ_KERNEL_Q80_F32 16
+#define CKQ_KERNEL_Q4K_F32 17
+#define CKQ_KERNEL_Q6K_F32 18
 
 /*
  * y[t*ldy + row] = dot(W[row], X[t]) (+ bias[row]) for row < nrows, t < ntok.

@@ -63,6 +63,26 @@ def gemm_nt(fmt, A_q8, B, bias, M, N, K):
     return c.reshape(M, N)
 
 
+def gemv_f32act(fmt, W, x_f32, M, K):
+    """gemv_q4_k / gemv_q6_k / gemv_q8_0: fp32 activations, nothing quantized."""
+    y = np.zeros(M, dtype=np.float32)
+    getattr(lib(), "gemv_" + fmt)(_p(y), _p(W), _p(x_f32), M, K)
+    return y
+
+
+def gemm_nt_f32act(fmt, A_f32, B, bias, M, N, K):
+    c = np.zeros(M * N, dtype=np.float32)
+    getattr(lib(), "gemm_nt_" + fmt)(_p(A_f32), _p(B), _p(bias), _p(c), M, N, K)
+    return c.reshape(M, N)
+
+
+def gemm_f32act(fmt, W, X_f32, M, N, K):
+    """gemm_q4_k / gemm_q6_k / gemm_q8_0: Y[n*M + row]."""
+    y = np.zeros(N * M, dtype=np.float32)
+    getattr(lib(), "gemm_" + fmt)(_p(y), _p(W), _p(X_f32), M, N, K)
+    return y.reshape(N, M)
+
+
 # ---- device-resident path ---------------------------------------------------------
 
 def _stream():
@@ -102,6 +122,14 @@ def dev_gemv_q8_0_f32(W_t, x_t, M, K):
     y = torch.empty(M, dtype=torch.float32, device=W_t.device)
     check(lib().ckq_gemv_q8_0_dev(_dp(y), _dp(W_t), _dp(x_t), M, K, _stream()), "ckq_gemv_q8_0_dev")
     return y
+
+
+def dev_gemm_nt_f32act(fmt, A_t, B_t, bias_t, M, N, K, out=None):
+    import torch
+    c = out if out is not None else torch.empty(M * N, dtype=torch.float32, device=B_t.device)
+    check(lib().ckq_gemm_nt_f32act_dev(FMT[fmt], _dp(A_t), _dp(B_t), _dp(bias_t), _dp(c), M, N, K, N, _stream()),
+          "ckq_gemm_nt_f32act_dev")
+    return c
 
 
 def dev_subblock_dots(fmt, W_t, x_t, M, K):

@@ -85,6 +85,24 @@ void gemv_q8_0_q8_0_parallel_simd(float *y, const void *W, const void *x_q8, int
 void gemv_q8_0(float *y, const void *W, const float *x, int M, int K);
 void gemm_nt_q8_0_q8_0(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K);
 
+/* fp32 activations used as they are: the weights are dequantized on the fly,
+ * nothing is quantized.  Same naming trap as above (gemv: M rows; gemm_q*:
+ * Y[n*M + row]; gemm_nt: M tokens, N rows).  Replace gemm_kernels_q4k.c:285-297
+ * (gemv_q4_k), :461-469 (gemm_q4_k), :484-489 (dot_q4_k), :683-711
+ * (gemm_nt_q4_k); gemm_kernels_q6k.c:169-193 (gemv_q6_k), :195-210 (gemm_q6_k),
+ * :212-240 (gemm_nt_q6_k); gemm_kernels_q8_0.c:658-666 (gemm_q8_0), :683-696
+ * (gemm_nt_q8_0).  K must be a multiple of the block size (the reference reads
+ * whole blocks); otherwise nothing is written. */
+void  gemv_q4_k(float *y, const void *W, const float *x, int M, int K);
+void  gemm_q4_k(float *Y, const void *W, const float *X, int M, int N, int K);
+void  gemm_nt_q4_k(const float *A, const void *B, const float *bias, float *C, int M, int N, int K);
+float dot_q4_k(const void *w_q4k, const float *x, int K);
+void  gemv_q6_k(float *y, const void *W, const float *x, int M, int K);
+void  gemm_q6_k(float *Y, const void *W, const float *X, int M, int N, int K);
+void  gemm_nt_q6_k(const float *A, const void *B, const float *bias, float *C, int M, int N, int K);
+void  gemm_q8_0(float *Y, const void *W, const float *X, int M, int N, int K);
+void  gemm_nt_q8_0(const float *A, const void *B, const float *bias, float *C, int M, int N, int K);
+
 /* Parity-test wrappers: fp32 input is quantized, then the kernel runs.
  * Replace src/ck_parity_api.c:207-210 (quantize), :217-258 (gemv q4_k/q6_k),
  * :288-360 (gemv q8_0), :397-400 (vec_dot), :411-503 (gemm) and the size
@@ -131,6 +149,12 @@ int ckq_gemm_nt_q4_k_q8_k_dev(const void *A_q8, const void *B, const float *bias
 int ckq_gemm_nt_q5_k_q8_k_dev(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K, void *stream);
 int ckq_gemm_nt_q6_k_q8_k_dev(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K, void *stream);
 int ckq_gemm_nt_q8_0_q8_0_dev(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K, void *stream);
+
+/* fp32 activations (M rows of K floats, 16-byte aligned) against `fmt` weights
+ * (CKQ_FMT_Q4_K, _Q6_K or _Q8_0), no activation quantization: the device form
+ * of gemv_q4_k / gemm_nt_q4_k / gemm_nt_q6_k / gemm_nt_q8_0 above. */
+int ckq_gemm_nt_f32act_dev(int fmt, const float *A, const void *B, const float *bias, float *C,
+                           int M, int N, int K, long ldc, void *stream);
 
 /* A list of matmuls enqueued back-to-back, the whole list `repeat` times: the
  * per-token projection set of a decoder layer (Q/K/V/O, gate/up, down) is one

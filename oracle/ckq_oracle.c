@@ -623,6 +623,69 @@ void orc_gemv_q8_0(float *y, const void *W, const float *x, int M, int K)
     }
 }
 
+/* Q4_K weights, fp32 activations, no activation quantization:
+ * sum += (d*sc*q - dmin*m) * x per element, left to right
+ * (reference: gemm_kernels_q4k.c:53-101; gemv_q4_k at :285-297 dispatches to
+ * SIMD variants of the same sum, which differ in summation order only). */
+void orc_gemv_q4_k(float *y, const void *W, const float *x, int M, int K)
+{
+    if (!y || !W || !x || M <= 0 || K <= 0) return;
+    const int nb = K / CKQ_QK_K;
+    const ckq_block_q4_K *w = (const ckq_block_q4_K *)W;
+    for (int r = 0; r < M; ++r) {
+        float sum = 0.0f;
+        for (int b = 0; b < nb; ++b) {
+            const ckq_block_q4_K *blk = &w[(size_t)r * nb + b];
+            const float d = orc_fp16_to_fp32(blk->d), dmin = orc_fp16_to_fp32(blk->dmin);
+            uint8_t sc[8], m[8];
+            orc_unpack_scales_k4(blk->scales, sc, m);
+            for (int g = 0; g < 4; ++g) {
+                const float d1 = d * (float)sc[2 * g], m1 = dmin * (float)m[2 * g];
+                const float d2 = d * (float)sc[2 * g + 1], m2 = dmin * (float)m[2 * g + 1];
+                const uint8_t *qs = blk->qs + 32 * g;
+                const float *xp = x + (size_t)b * CKQ_QK_K + 64 * g;
+                for (int l = 0; l < 32; ++l) sum += (d1 * (float)(qs[l] & 0x0F) - m1) * xp[l];
+                for (int l = 0; l < 32; ++l) sum += (d2 * (float)(qs[l] >> 4) - m2) * xp[l + 32];
+            }
+        }
+        y[r] = sum;
+    }
+}
+
+/* Q6_K weights, fp32 activations: sum += (d*sc*q) * x, four streams per l
+ * (reference: gemm_kernels_q6k.c:39-76, gemv_q6_k at :169-193). */
+void orc_gemv_q6_k(float *y, const void *W, const float *x, int M, int K)
+{
+    if (!y || !W || !x || M <= 0 || K <= 0) return;
+    const int nb = K / CKQ_QK_K;
+    const ckq_block_q6_K *w = (const ckq_block_q6_K *)W;
+    for (int r = 0; r < M; ++r) {
+        float sum = 0.0f;
+        for (int b = 0; b < nb; ++b) {
+            const ckq_block_q6_K *blk = &w[(size_t)r * nb + b];
+            const float d = orc_fp16_to_fp32(blk->d);
+            const uint8_t *ql = blk->ql, *qh = blk->qh;
+            const int8_t *sc = blk->scales;
+            const float *xp = x + (size_t)b * CKQ_QK_K;
+            for (int n = 0; n < CKQ_QK_K; n += 128) {
+                for (int l = 0; l < 32; ++l) {
+                    const int is = l / 16;
+                    const int8_t q1 = (int8_t)((ql[l] & 0xF) | (((qh[l] >> 0) & 3) << 4)) - 32;
+                    const int8_t q2 = (int8_t)((ql[l + 32] & 0xF) | (((qh[l] >> 2) & 3) << 4)) - 32;
+                    const int8_t q3 = (int8_t)((ql[l] >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32;
+                    const int8_t q4 = (int8_t)((ql[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32;
+                    sum += (d * (float)sc[is + 0] * (float)q1) * xp[l];
+                    sum += (d * (float)sc[is + 2] * (float)q2) * xp[l + 32];
+                    sum += (d * (float)sc[is + 4] * (float)q3) * xp[l + 64];
+                    sum += (d * (float)sc[is + 6] * (float)q4) * xp[l + 96];
+                }
+                xp += 128; ql += 64; qh += 32; sc += 8;
+            }
+        }
+        y[r] = sum;
+    }
+}
+
 /* ------------------------------------------------------------------------ */
 /* GEMM                                                                      */
 /* ------------------------------------------------------------------------ */
@@ -812,4 +875,40 @@ void orc_gemv_threads(int fmt, float *y, const void *W, const void *x_q8, int M,
     }
     thr_main(&arg[0]);
     for (int t = 1; t < nth; ++t) pthread_join(tid[t], NULL);
+}
+
+/* fp32-activation GEMMs: a token loop over the GEMV, then the bias
+ * (reference: gemm_kernels_q4k.c:316-330,461-469,683-711; gemm_kernels_q6k.c:195-240;
+ * gemm_kernels_q8_0.c:658-696). */
+void orc_gemm_q4_k(float *Y, const void *W, const float *X, int M, int N, int K)
+{
+    if (!Y || !W || !X || M <= 0 || N <= 0 || K <= 0) return;
+    for (int n = 0; n < N; ++n) orc_gemv_q4_k(Y + (size_t)n * M, W, X + (size_t)n * K, M, K);
+}
+
+void orc_gemm_nt_q4_k(const float *A, const void *B, const float *bias, float *C, int M, int N, int K)
+{
+    if (!A || !B || !C || M <= 0 || N <= 0 || K <= 0) return;
+    orc_gemm_q4_k(C, B, A, N, M, K);
+    add_bias(C, bias, M, N);
+}
+
+void orc_gemm_q6_k(float *Y, const void *W, const float *X, int M, int N, int K)
+{
+    if (!Y || !W || !X || M <= 0 || N <= 0 || K <= 0) return;
+    for (int n = 0; n < N; ++n) orc_gemv_q6_k(Y + (size_t)n * M, W, X + (size_t)n * K, M, K);
+}
+
+void orc_gemm_nt_q6_k(const float *A, const void *B, const float *bias, float *C, int M, int N, int K)
+{
+    if (!A || !B || !C || M <= 0 || N <= 0 || K <= 0) return;
+    orc_gemm_q6_k(C, B, A, N, M, K);
+    add_bias(C, bias, M, N);
+}
+
+void orc_gemm_nt_q8_0(const float *A, const void *B, const float *bias, float *C, int M, int N, int K)
+{
+    if (!A || !B || !C || M <= 0 || N <= 0 || K <= 0) return;
+    for (int m = 0; m < M; ++m) orc_gemv_q8_0(C + (size_t)m * N, B, A + (size_t)m * K, N, K);
+    add_bias(C, bias, M, N);
 }

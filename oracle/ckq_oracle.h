@@ -62,6 +62,8 @@ void orc_gemv_q8_0_q8_0_lanes8(float *y, const void *W, const void *x_q8, int M,
 void orc_gemv_q8_0_q8_0_parallel(float *y, const void *W, const void *x_q8, int M, int K, int ith, int nth); /* :1263-1287 */
 void orc_vec_dot_q8_0_q8_0(int n, float *s, const void *vx, const void *vy);           /* gemm_kernels_q8_0.c:968-989 */
 void orc_gemv_q8_0(float *y, const void *W, const float *x, int M, int K);             /* gemm_kernels_q8_0.c:254-277 */
+void orc_gemv_q4_k(float *y, const void *W, const float *x, int M, int K);             /* gemm_kernels_q4k.c:53-101 (fp32 activations) */
+void orc_gemv_q6_k(float *y, const void *W, const float *x, int M, int K);             /* gemm_kernels_q6k.c:39-76,169-193 (fp32 activations) */
 
 /* ---- GEMM ---------------------------------------------------------------
  * gemm_*   : Y[n*M + row], M = output rows, N = tokens.
@@ -73,6 +75,11 @@ void orc_gemm_nt_q5_k(const float *A, const void *B, const float *bias, float *C
 void orc_gemm_q6_k_q8_k(float *Y, const void *W, const void *X_q8, int M, int N, int K);                        /* gemm_kernels_q6k_q8k.c:1209-1225 */
 void orc_gemm_nt_q6_k_q8_k(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K);  /* :1243-1268 */
 void orc_gemm_nt_q8_0_q8_0(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K);  /* gemm_batch_int8.c:87-120,582-610 */
+void orc_gemm_q4_k(float *Y, const void *W, const float *X, int M, int N, int K);                                   /* gemm_kernels_q4k.c:316-330,461-469 */
+void orc_gemm_nt_q4_k(const float *A, const void *B, const float *bias, float *C, int M, int N, int K);            /* gemm_kernels_q4k.c:683-711 */
+void orc_gemm_q6_k(float *Y, const void *W, const float *X, int M, int N, int K);                                   /* gemm_kernels_q6k.c:195-210 */
+void orc_gemm_nt_q6_k(const float *A, const void *B, const float *bias, float *C, int M, int N, int K);            /* gemm_kernels_q6k.c:212-240 */
+void orc_gemm_nt_q8_0(const float *A, const void *B, const float *bias, float *C, int M, int N, int K);            /* gemm_kernels_q8_0.c:683-696 */
 
 /* ---- exact evaluation ---------------------------------------------------
  * Same integers, block scales combined in double: the value every fp32

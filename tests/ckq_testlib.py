@@ -125,6 +125,13 @@ def oracle_gemm_nt(fmt, A, B, bias, M, N, K):
     return c.reshape(M, N)
 
 
+def oracle_gemm_nt_f32act(fmt, A_f32, B, bias, M, N, K):
+    """fp32 activations, nothing quantized (orc_gemm_nt_q4_k / _q6_k / _q8_0)."""
+    c = np.zeros(M * N, dtype=np.float32)
+    getattr(oracle(), "orc_gemm_nt_" + fmt)(ptr(A_f32), ptr(B), ptr(bias) if bias is not None else None, ptr(c), M, N, K)
+    return c.reshape(M, N)
+
+
 def oracle_exact(fmt, W, xq, M, K):
     y = np.zeros(M, dtype=np.float64)
     oracle().orc_gemv_exact_f64(FMT[fmt], ptr(y), ptr(W), ptr(xq), M, K)

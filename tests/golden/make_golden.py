@@ -192,6 +192,16 @@ def main():
                 for ith in range(5):
                     run(libs["avx2"], "gemv_q4_k_q8_k_parallel_simd", ptr(y), ptr(w), ptr(act), ROWS, K, ith, 5)
                 G["y_q4_k_%s_parallel5" % kind] = y
+            # fp32 activations, no activation quantization (both builds: they sum in different orders)
+            if fmt in ("q4_k", "q6_k", "q8_0"):
+                for tag, L in libs.items():
+                    if fmt != "q8_0":
+                        y = np.zeros(ROWS, np.float32)
+                        run(L, "gemv_" + fmt, ptr(y), ptr(w), ptr(xf), ROWS, K)
+                        G["y_%s_%s_f32w_%s" % (fmt, kind, tag)] = y
+                    c = np.zeros(TOK * ROWS, np.float32)
+                    run(L, "gemm_nt_" + fmt, ptr(xf), ptr(w), ptr(bias), ptr(c), TOK, ROWS, K)
+                    G["c_%s_%s_f32w_%s" % (fmt, kind, tag)] = c
             if fmt == "q5_k":
                 y = np.zeros(ROWS, np.float32)
                 run(libs["avx2"], gemv, ptr(y), ptr(w), ptr(xz), ROWS, K)

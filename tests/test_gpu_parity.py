@@ -321,6 +321,60 @@ def test_batched_decode_small_model_shapes(M):
         c = P.dev_gemm_nt(fmt, P.to_device(xq), P.to_device(W), None, M, rows, K).cpu().numpy()
         assert T.norm_err(c, T.oracle_gemm_nt(fmt, xq, W, None, M, rows, K)) <= TOL
 
+# ---- fp32 activations, no activation quantization -------------------------------------------
+
+F32_FMTS = ["q4_k", "q6_k", "q8_0"]
+
+
+@pytest.mark.parametrize("fmt", F32_FMTS)
+@pytest.mark.parametrize("kind", ["rand", "enc"])
+def test_f32act_golden_fixture(fmt, kind):
+    """gemv_q4_k / gemv_q6_k / gemm_nt_q4_k / _q6_k / _q8_0 through the drop-in
+    symbols (host pointers) against the reference builds' own outputs."""
+    G = T.golden()
+    M, K, TOK = (int(v) for v in G["shape"])
+    W, xf, bias = G["w_%s_%s" % (fmt, kind)], G["act_f32"], G["bias"]
+    say("f32act golden", fmt, kind)
+    c = P.gemm_nt_f32act(fmt, xf, W, bias, TOK, M, K)
+    for build in ("avx2", "avx512"):
+        assert T.norm_err(c.reshape(-1), G["c_%s_%s_f32w_%s" % (fmt, kind, build)]) <= TOL
+    if fmt != "q8_0":
+        y = P.gemv_f32act(fmt, W, xf, M, K)
+        assert T.norm_err(y, G["y_%s_%s_f32w_avx2" % (fmt, kind)]) <= TOL
+        assert ckq.lib().dot_q4_k is not None
+    Y = P.gemm_f32act(fmt, W, xf, M, TOK, K)                   # Y[n*M + row]
+    assert T.norm_err(Y, T.oracle_gemm_nt_f32act(fmt, xf, W, None, TOK, M, K)) <= TOL
+    if fmt == "q4_k":
+        import ctypes as C
+        r = ckq.lib().dot_q4_k(C.c_void_p(W.ctypes.data), C.c_void_p(xf.ctypes.data), K)
+        assert abs(r - y[0]) <= TOL * max(1.0, np.abs(y).max())
+
+
+@pytest.mark.parametrize("fmt", F32_FMTS)
+def test_f32act_vs_oracle_shapes(fmt):
+    """Ragged row counts, short and long rows, several tokens, device pointers."""
+    blk = 32 if fmt == "q8_0" else 256
+    for rows, K, M in ((1, blk, 1), (7, 2 * blk, 3), (130, 1024, 2), (257, 4096, 1), (33, 11008 if fmt != "q8_0" else 896, 5)):
+        W, xf, _ = make_case(fmt, rows, K, "rand" if rows % 2 else "enc", rows + K, tokens=M)
+        bias = T.normal(rows, 0.0, 0.5, seed=rows)
+        say("f32act", fmt, rows, K, "M", M)
+        c = P.dev_gemm_nt_f32act(fmt, P.to_device(xf), P.to_device(W), P.to_device(bias), M, rows, K).cpu().numpy()
+        assert T.norm_err(c.reshape(M, rows), T.oracle_gemm_nt_f32act(fmt, xf, W, bias, M, rows, K)) <= TOL
+        # K not a multiple of the block size: nothing is written
+    out = np.full(4, 7.0, np.float32)
+    getattr(ckq.lib(), "gemv_" + fmt)(P._p(out), P._p(np.zeros(4096, np.uint8)), P._p(np.zeros(100, np.float32)), 4, 100)
+    assert np.all(out == 7.0)
+
+
+def test_f32act_full_size():
+    """11008 x 4096 Q4_K with fp32 activations against dequantize-then-matmul in fp64."""
+    rows, K = 11008, 4096
+    W, xf, _ = make_case("q4_k", rows, K, "enc", 77)
+    say("f32act full size")
+    y = P.dev_gemm_nt_f32act("q4_k", P.to_device(xf), P.to_device(W), None, 1, rows, K).cpu().numpy().reshape(-1)
+    want = T.np_dequant("q4_k", W).reshape(rows, K).astype(np.float64) @ xf.astype(np.float64)
+    assert T.norm_err(y, want) <= TOL
+
 
 # ---- prefill GEMM on the matrix cores (Q4_K, token counts above 16) -------------------------
 

@@ -263,6 +263,40 @@ def test_lane_order_variants_bit_identical_to_avx2_build(kind):
     y = T.oracle_gemv("q8_0", G["w_q8_0_" + kind], G["act_q80"], M, K, "orc_gemv_q8_0_q8_0_lanes8")
     assert np.array_equal(y.view(np.uint32), G["y_q8_0_%s_avx2" % kind].view(np.uint32))
 
+# ---- fp32 activations, no activation quantization ----------------------------------
+
+@pytest.mark.parametrize("fmt", ["q4_k", "q6_k", "q8_0"])
+@pytest.mark.parametrize("kind", ["rand", "enc"])
+def test_fp32_activation_kernels_match_reference(fmt, kind):
+    """gemv_q4_k / gemv_q6_k / gemm_nt_q4_k / gemm_nt_q6_k / gemm_nt_q8_0: the
+    weights are dequantized on the fly and dotted with fp32 activations.  Golden
+    outputs come from both reference builds (AVX2 and AVX-512 sum in different
+    orders); the closed form is dequantize-then-matmul in fp64."""
+    G = T.golden()
+    M, K, TOK = (int(v) for v in G["shape"])
+    O = T.oracle()
+    W, xf, bias = G["w_%s_%s" % (fmt, kind)], G["act_f32"], G["bias"]
+    want = T.np_dequant(fmt, W).reshape(M, K).astype(np.float64) @ xf.reshape(TOK, K).T.astype(np.float64)   # [M, TOK]
+    if fmt != "q8_0":
+        y = np.zeros(M, np.float32)
+        getattr(O, "orc_gemv_" + fmt)(ptr(y), ptr(W), ptr(xf), M, K)
+        for build in ("avx2", "avx512"):
+            assert T.norm_err(y, G["y_%s_%s_f32w_%s" % (fmt, kind, build)]) <= 1e-5
+        assert T.norm_err(y, want[:, 0]) <= 1e-5
+        # gemm_q*_k layout: Y[n*M + row]
+        Y = np.zeros(TOK * M, np.float32)
+        getattr(O, "orc_gemm_" + fmt)(ptr(Y), ptr(W), ptr(xf), M, TOK, K)
+        assert T.norm_err(Y.reshape(TOK, M), want.T) <= 1e-5
+    c = np.zeros(TOK * M, np.float32)
+    getattr(O, "orc_gemm_nt_" + fmt)(ptr(xf), ptr(W), ptr(bias), ptr(c), TOK, M, K)
+    for build in ("avx2", "avx512"):
+        assert T.norm_err(c, G["c_%s_%s_f32w_%s" % (fmt, kind, build)]) <= 1e-5
+    assert T.norm_err(c.reshape(TOK, M), want.T + bias[None, :]) <= 1e-5
+    # a dropped min term, a wrong nibble order or a missing -32 would be far outside this
+    c0 = np.zeros(TOK * M, np.float32)
+    getattr(O, "orc_gemm_nt_" + fmt)(ptr(xf), ptr(W), None, ptr(c0), TOK, M, K)
+    assert np.allclose(c - c0, np.tile(bias, TOK), atol=1e-5 * max(1.0, np.abs(c).max()))
+
 
 # ---- exact evaluation: dequantize-then-fp64 matmul ---------------------------------
 
