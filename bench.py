@@ -300,6 +300,25 @@ def main():
                                                  "frac_hbm": round(bf / sf / 1e9 / HBM_PEAK_GBS, 4),
                                                  "note": "launched from Python one call at a time"}
 
+        # fused producer rmsnorm -> Q8_K next to the plain quantizer (launch-bound at one token)
+        gam_d = P.to_device(T.normal(K, 1.0, 0.2, seed=55))
+        prod = {}
+        for tk in (1, 512):
+            xin = P.to_device(T.normal(tk * K, 0.0, 1.0, seed=56))
+            for name, fn in (("rmsnorm_q8_k_fused", lambda: P.dev_rmsnorm_q8_k_fused(xin, gam_d, tk, K)),
+                             ("quantize_q8_k", lambda: P.dev_quantize(xin, "q8_k", rows=tk))):
+                for _ in range(5):
+                    fn()
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(100):
+                    fn()
+                e1.record()
+                torch.cuda.synchronize()
+                prod["%s_T%d_us" % (name, tk)] = round(e0.elapsed_time(e1) * 10.0, 2)
+        extras["producer_d4096"] = prod
+
         # a 7B decoder layer's projection set at M=1: Q,K,V,O (4096x4096 Q4_K), gate, up
         # (11008x4096 Q4_K), down (4096x11008 Q6_K), one C call per layer, weights of
         # successive steps distinct (4 rotated layers = 502 MB)

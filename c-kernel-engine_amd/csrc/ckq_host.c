@@ -585,6 +585,36 @@ void gemm_nt_q8_0_q8_0(const void *A_q8, const void *B, const float *bias, float
     host_matmul(CKQ_FMT_Q8_0, A_q8, B, bias, C, M, N, K, N, 0, N);
 }
 
+/* Fused producer: RMSNorm then Q8_K quantization, any pointer mix, synchronous. */
+void rmsnorm_q8_k_fused(const float *input, const float *gamma, void *vy, int tokens, int d_model,
+                        int aligned_embed_dim, float eps)
+{
+    if (!input || !gamma || !vy || tokens <= 0 || d_model <= 0 || aligned_embed_dim < d_model) return;
+    if (d_model % 256) return;
+    const size_t in_bytes = ((size_t)(tokens - 1) * aligned_embed_dim + d_model) * 4;
+    const size_t out_bytes = (size_t)tokens * ckq_row_bytes(CKQ_FMT_Q8_K, d_model);
+    pthread_mutex_lock(&g_mu);
+    do {
+        if (init_locked()) break;
+        const void *dx, *dg;
+        if (stage_in(BUF_X, input, in_bytes, &dx)) break;
+        if (stage_in(BUF_BIAS, gamma, (size_t)d_model * 4, &dg)) break;
+        const int y_on_dev = is_device_ptr(vy);
+        void *dy = vy;
+        if (!y_on_dev && buf_reserve(BUF_Y, out_bytes, &dy)) break;
+        int rc = ckq_launch_rmsnorm_q8_k_fused((const float *)dx, (const float *)dg, dy, tokens, d_model,
+                                               aligned_embed_dim, eps, g_stream);
+        if (rc) { fail(rc, "rmsnorm_q8_k_fused launch"); break; }
+        if (!y_on_dev) {
+            hipError_t e = hipMemcpyAsync(vy, dy, out_bytes, hipMemcpyDeviceToHost, g_stream);
+            if (e != hipSuccess) { fail((int)e, "copy result to host"); break; }
+        }
+        hipError_t e = hipStreamSynchronize(g_stream);
+        if (e != hipSuccess) fail((int)e, "hipStreamSynchronize");
+    } while (0);
+    pthread_mutex_unlock(&g_mu);
+}
+
 /* fp32 activations used as they are (no activation quantization). */
 void gemv_q4_k(float *y, const void *W, const float *x, int M, int K)
 {
@@ -721,6 +751,12 @@ DEFINE_DEV(q8_0_q8_0, CKQ_FMT_Q8_0)
 int ckq_gemv_q8_0_dev(float *y, const void *W, const float *x, int M, int K, void *stream)
 {
     return ckq_launch_gemv(CKQ_KERNEL_Q80_F32, y, W, x, NULL, M, K, 1, M, 0, M, NULL, stream);
+}
+
+int ckq_rmsnorm_q8_k_fused_dev(const float *input, const float *gamma, void *y, int tokens, int d_model,
+                               int aligned_embed_dim, float eps, void *stream)
+{
+    return ckq_launch_rmsnorm_q8_k_fused(input, gamma, y, tokens, d_model, aligned_embed_dim, eps, stream);
 }
 
 int ckq_gemm_nt_f32act_dev(int fmt, const float *A, const void *B, const float *bias, float *C,

@@ -8,6 +8,7 @@
  *                           with v_dot4_i32_i8, reduced with DPP.
  *   quantize_q8_k_kernel    fp32 -> Q8_K, bit-exact with the reference
  *   quantize_q8_0_kernel    fp32 -> Q8_0, bit-exact with the reference
+ *   rmsnorm_q8_k_fused_kernel  RMSNorm -> Q8_K in one pass, bit-exact with the reference's FMA build
  *   copy_kernel             plain streaming copy (counter calibration)
  *   read_kernel             plain streaming read (launch-floor calibration)
  *
@@ -412,6 +413,105 @@ extern "C" int ckq_launch_quantize_q8_0(const float *x, void *y, int rows, int k
     const long nblocks = (long)rows * (k / 32);
     hipLaunchKernelGGL(quantize_q8_0_kernel, dim3((unsigned)((nblocks * 8 + 255) / 256)), dim3(256), 0,
                        (hipStream_t)stream, x, (uint8_t *)y, nblocks);
+    return (int)hipGetLastError();
+}
+
+/*
+ * Fused producer RMSNorm -> Q8_K, one block per token (reference:
+ * src/kernels/fused/rmsnorm_q8_k_fused.c:54-142 as an FMA build compiles it).
+ * The sum of squares must be the reference's to the bit, or rstd moves by an
+ * ulp and quants flip: eight strided lanes (lane j takes x[8i+j]) each a chain
+ * of fused multiply-adds, combined as ((l0+l4)+(l1+l5)) + ((l2+l6)+(l3+l7)).
+ * Eight threads walk the chains over the row staged in LDS; every thread then
+ * derives the same rstd.  Quantization: n = (x*rstd)*gamma with two roundings,
+ * scale from the largest |n| of the block, iscale = -127/max, d = 1/iscale,
+ * q = RNE(n*iscale) saturated; one wave per 256-block, lane l owns 4l..4l+3.
+ */
+__global__ void __launch_bounds__(256) rmsnorm_q8_k_fused_kernel(const float *__restrict__ input,
+                                                                 const float *__restrict__ gamma,
+                                                                 uint8_t *__restrict__ y, int d_model, long in_stride,
+                                                                 float eps)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    float *xs = reinterpret_cast<float *>(smem);          /* d_model floats, then 8 lane sums */
+    const int tid = threadIdx.x, lane = tid & 63, wave = wave_in_block();
+    const float *x = input + (size_t)blockIdx.x * in_stride;
+    const int D = d_model, nb = D / 256;
+
+    for (int i = tid; i < D / 4; i += 256)
+        reinterpret_cast<float4 *>(xs)[i] = reinterpret_cast<const float4 *>(x)[i];
+    __syncthreads();
+    if (tid < 8) {
+        /* the chain is serial; keep 16 LDS reads in flight ahead of it (D is a multiple of 256) */
+        float acc = 0.0f, cur[16], nxt[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) cur[u] = xs[tid + 8 * u];
+        for (int d = 0; d < D; d += 128) {
+            const int dn = d + 128 < D ? d + 128 : d;
+#pragma unroll
+            for (int u = 0; u < 16; ++u) nxt[u] = xs[dn + tid + 8 * u];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) acc = __fmaf_rn(cur[u], cur[u], acc);
+#pragma unroll
+            for (int u = 0; u < 16; ++u) cur[u] = nxt[u];
+        }
+        xs[D + tid] = acc;
+    }
+    __syncthreads();
+    const float s04 = xs[D + 0] + xs[D + 4], s15 = xs[D + 1] + xs[D + 5];
+    const float s26 = xs[D + 2] + xs[D + 6], s37 = xs[D + 3] + xs[D + 7];
+    const float sum_sq = (s04 + s15) + (s26 + s37);
+    /* sqrtf and '/' are the correctly rounded ones (the __fsqrt_rn intrinsic is not) */
+    const float rstd = 1.0f / sqrtf(sum_sq / (float)D + eps);
+
+    for (int b = wave; b < nb; b += 4) {
+        const float4 xv = reinterpret_cast<const float4 *>(xs + 256 * b)[lane];
+        const float4 gv = reinterpret_cast<const float4 *>(gamma + 256 * b)[lane];
+        const float e[4] = {__fmul_rn(__fmul_rn(xv.x, rstd), gv.x), __fmul_rn(__fmul_rn(xv.y, rstd), gv.y),
+                            __fmul_rn(__fmul_rn(xv.z, rstd), gv.z), __fmul_rn(__fmul_rn(xv.w, rstd), gv.w)};
+        float amax = fmaxf(fmaxf(fabsf(e[0]), fabsf(e[1])), fmaxf(fabsf(e[2]), fabsf(e[3])));
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
+
+        uint8_t *out = y + ((size_t)blockIdx.x * nb + b) * 292;
+        if (amax == 0.0f) {
+            reinterpret_cast<u32 *>(out)[lane] = 0;
+            if (lane < 9) reinterpret_cast<u32 *>(out)[64 + lane] = 0;
+            continue;
+        }
+        const float iscale = __fdiv_rn(-127.0f, amax);
+        int q[4], sum = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            q[i] = rne_sat_i8(__fmul_rn(e[i], iscale));
+            sum += q[i];
+        }
+        reinterpret_cast<u32 *>(out + 4)[lane] =
+            (u32)(q[0] & 0xff) | ((u32)(q[1] & 0xff) << 8) | ((u32)(q[2] & 0xff) << 16) | ((u32)(q[3] & 0xff) << 24);
+        sum = group_sum<4>(sum);
+        if ((lane & 3) == 3) reinterpret_cast<int16_t *>(out + 260)[lane >> 2] = (int16_t)sum;
+        if (lane == 0) *reinterpret_cast<float *>(out) = __fdiv_rn(1.0f, iscale);
+    }
+}
+
+extern "C" int ckq_launch_rmsnorm_q8_k_fused(const float *input, const float *gamma, void *y, int tokens, int d_model,
+                                             int aligned_embed_dim, float eps, void *stream)
+{
+    if (!input || !gamma || !y || tokens <= 0 || d_model <= 0 || aligned_embed_dim < d_model) return CKQ_EINVAL;
+    if (d_model % 256 || aligned_embed_dim % 4) return CKQ_ESHAPE;
+    const size_t lds = (size_t)d_model * 4 + 32;
+    if (lds > 160 * 1024) return CKQ_ESHAPE;               /* the row is staged in LDS */
+    if (lds > 64 * 1024) {
+        static bool raised = false;                        /* opt in to more than 64 KB of dynamic LDS once */
+        if (!raised) {
+            hipError_t e = hipFuncSetAttribute((const void *)rmsnorm_q8_k_fused_kernel,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e != hipSuccess) return (int)e;
+            raised = true;
+        }
+    }
+    hipLaunchKernelGGL(rmsnorm_q8_k_fused_kernel, dim3((unsigned)tokens), dim3(256), lds, (hipStream_t)stream,
+                       input, gamma, (uint8_t *)y, d_model, (long)aligned_embed_dim, eps);
     return (int)hipGetLastError();
 }
 

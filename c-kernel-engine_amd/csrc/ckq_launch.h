@@ -42,6 +42,11 @@ int ckq_launch_gemv(int fmt, float *y, const void *W, const void *X, const float
 int ckq_launch_quantize_q8_k(const float *x, void *y, int rows, int k, void *stream);
 int ckq_launch_quantize_q8_0(const float *x, void *y, int rows, int k, void *stream);
 
+/* RMSNorm over d_model floats per token (row stride aligned_embed_dim floats),
+ * times gamma, quantized to Q8_K blocks: tokens x (d_model/256) blocks. */
+int ckq_launch_rmsnorm_q8_k_fused(const float *input, const float *gamma, void *y, int tokens, int d_model,
+                                  int aligned_embed_dim, float eps, void *stream);
+
 /* Plain device copy kernel (calibration of the memory counters / roofline). */
 int ckq_launch_copy(void *dst, const void *src, size_t bytes, void *stream);
 int ckq_launch_read(const void *src, size_t bytes, void *sink, void *stream);

@@ -63,6 +63,13 @@ def gemm_nt(fmt, A_q8, B, bias, M, N, K):
     return c.reshape(M, N)
 
 
+def rmsnorm_q8_k_fused(x, gamma, tokens, d_model, aligned=None, eps=1e-6):
+    aligned = aligned or d_model
+    out = np.zeros(tokens * row_bytes("q8_k", d_model), dtype=np.uint8)
+    lib().rmsnorm_q8_k_fused(_p(x), _p(gamma), _p(out), tokens, d_model, aligned, ctypes.c_float(eps))
+    return out
+
+
 def gemv_f32act(fmt, W, x_f32, M, K):
     """gemv_q4_k / gemv_q6_k / gemv_q8_0: fp32 activations, nothing quantized."""
     y = np.zeros(M, dtype=np.float32)
@@ -122,6 +129,15 @@ def dev_gemv_q8_0_f32(W_t, x_t, M, K):
     y = torch.empty(M, dtype=torch.float32, device=W_t.device)
     check(lib().ckq_gemv_q8_0_dev(_dp(y), _dp(W_t), _dp(x_t), M, K, _stream()), "ckq_gemv_q8_0_dev")
     return y
+
+
+def dev_rmsnorm_q8_k_fused(x_t, gamma_t, tokens, d_model, aligned=None, eps=1e-6):
+    import torch
+    aligned = aligned or d_model
+    out = torch.zeros(tokens * row_bytes("q8_k", d_model), dtype=torch.uint8, device=x_t.device)
+    check(lib().ckq_rmsnorm_q8_k_fused_dev(_dp(x_t), _dp(gamma_t), _dp(out), tokens, d_model, aligned,
+                                           ctypes.c_float(eps), _stream()), "ckq_rmsnorm_q8_k_fused_dev")
+    return out
 
 
 def dev_gemm_nt_f32act(fmt, A_t, B_t, bias_t, M, N, K, out=None):

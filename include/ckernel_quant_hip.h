@@ -103,6 +103,16 @@ void  gemm_nt_q6_k(const float *A, const void *B, const float *bias, float *C, i
 void  gemm_q8_0(float *Y, const void *W, const float *X, int M, int N, int K);
 void  gemm_nt_q8_0(const float *A, const void *B, const float *bias, float *C, int M, int N, int K);
 
+/* Fused producer of the path's activations: RMSNorm over d_model floats per
+ * token (row stride aligned_embed_dim floats) times gamma, quantized to Q8_K
+ * in the same pass; vy receives tokens x (d_model/256) blocks.  The block scale
+ * comes from the largest |value| (unlike quantize_row_q8_k's signed
+ * first-largest), so d is negative.  Bit-exact with the reference built with
+ * FMA enabled (every AVX2 host build).  d_model must be a multiple of 256.
+ * Replaces src/kernels/fused/rmsnorm_q8_k_fused.c:54-142. */
+void rmsnorm_q8_k_fused(const float *input, const float *gamma, void *vy, int tokens, int d_model,
+                        int aligned_embed_dim, float eps);
+
 /* Parity-test wrappers: fp32 input is quantized, then the kernel runs.
  * Replace src/ck_parity_api.c:207-210 (quantize), :217-258 (gemv q4_k/q6_k),
  * :288-360 (gemv q8_0), :397-400 (vec_dot), :411-503 (gemm) and the size
@@ -149,6 +159,11 @@ int ckq_gemm_nt_q4_k_q8_k_dev(const void *A_q8, const void *B, const float *bias
 int ckq_gemm_nt_q5_k_q8_k_dev(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K, void *stream);
 int ckq_gemm_nt_q6_k_q8_k_dev(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K, void *stream);
 int ckq_gemm_nt_q8_0_q8_0_dev(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K, void *stream);
+
+/* Device form of rmsnorm_q8_k_fused; input rows and gamma 16-byte aligned,
+ * d_model <= 40 000 (the row is staged in LDS). */
+int ckq_rmsnorm_q8_k_fused_dev(const float *input, const float *gamma, void *y, int tokens, int d_model,
+                               int aligned_embed_dim, float eps, void *stream);
 
 /* fp32 activations (M rows of K floats, 16-byte aligned) against `fmt` weights
  * (CKQ_FMT_Q4_K, _Q6_K or _Q8_0), no activation quantization: the device form

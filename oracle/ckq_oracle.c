@@ -687,6 +687,75 @@ void orc_gemv_q6_k(float *y, const void *W, const float *x, int M, int K)
 }
 
 /* ------------------------------------------------------------------------ */
+/* Fused producer: RMSNorm -> Q8_K                                           */
+/* ------------------------------------------------------------------------ */
+
+/* Reference: src/kernels/fused/rmsnorm_q8_k_fused.c:54-142 as an x86 build with
+ * FMA compiles it.  Per token: sum of squares in eight strided lanes (lane j
+ * takes x[8i+j]; gcc contracts the add of the product into one FMA when the
+ * build enables FMA, which every AVX2 host build does), lanes combined as
+ * ((l0+l4)+(l1+l5)) + ((l2+l6)+(l3+l7)); rstd = 1/sqrtf(sum/D + eps); then per
+ * 256-block: n = (x*rstd)*gamma (two roundings), scale from the largest
+ * |n| (NOT the signed first-largest of quantize_row_q8_k): iscale = -127/max,
+ * d = 1/iscale (negative), q = RNE(n*iscale) saturated to int8, bsums of 16.
+ * `fma` = 0 restates a build without FMA (product rounded before the add). */
+static void rmsnorm_q8_k_fused_impl(const float *input, const float *gamma, void *vy,
+                                    int tokens, int d_model, int aligned_embed_dim, float eps, int fma)
+{
+    if (!input || !gamma || !vy || tokens <= 0 || d_model <= 0) return;
+    const int D = d_model, nb = D / CKQ_QK_K;
+    ckq_block_q8_K *y = (ckq_block_q8_K *)vy;
+    for (int t = 0; t < tokens; ++t) {
+        const float *x = input + (size_t)t * aligned_embed_dim;
+        float lane[8] = {0};
+        for (int d = 0; d < D; d += 8)
+            for (int j = 0; j < 8; ++j) {
+                if (fma) lane[j] = fmaf(x[d + j], x[d + j], lane[j]);
+                else { volatile float p = x[d + j] * x[d + j]; lane[j] = lane[j] + p; }
+            }
+        const float s04 = lane[0] + lane[4], s15 = lane[1] + lane[5], s26 = lane[2] + lane[6], s37 = lane[3] + lane[7];
+        const float sum_sq = (s04 + s15) + (s26 + s37);
+        const float rstd = 1.0f / sqrtf(sum_sq / (float)D + eps);
+        for (int b = 0; b < nb; ++b) {
+            const float *xb = x + b * CKQ_QK_K, *gb = gamma + b * CKQ_QK_K;
+            ckq_block_q8_K *o = &y[(size_t)t * nb + b];
+            float n[CKQ_QK_K], amax = 0.0f;
+            for (int i = 0; i < CKQ_QK_K; ++i) {
+                volatile float u = xb[i] * rstd;
+                n[i] = u * gb[i];
+                const float a = fabsf(n[i]);
+                if (a > amax) amax = a;              /* maxps: a NaN operand never replaces the running max */
+            }
+            if (amax == 0.0f) { memset(o, 0, sizeof(*o)); continue; }
+            const float iscale = -127.0f / amax;
+            o->d = 1.0f / iscale;
+            for (int j = 0; j < CKQ_QK_K; j += 16) {
+                int bs = 0;
+                for (int i = 0; i < 16; ++i) {
+                    volatile float p = n[j + i] * iscale;
+                    const int q = rne_sat_i8(p);
+                    o->qs[j + i] = (int8_t)q;
+                    bs += q;
+                }
+                o->bsums[j / 16] = (int16_t)bs;
+            }
+        }
+    }
+}
+
+void orc_rmsnorm_q8_k_fused(const float *input, const float *gamma, void *vy,
+                            int tokens, int d_model, int aligned_embed_dim, float eps)
+{
+    rmsnorm_q8_k_fused_impl(input, gamma, vy, tokens, d_model, aligned_embed_dim, eps, 1);
+}
+
+void orc_rmsnorm_q8_k_fused_nofma(const float *input, const float *gamma, void *vy,
+                                  int tokens, int d_model, int aligned_embed_dim, float eps)
+{
+    rmsnorm_q8_k_fused_impl(input, gamma, vy, tokens, d_model, aligned_embed_dim, eps, 0);
+}
+
+/* ------------------------------------------------------------------------ */
 /* GEMM                                                                      */
 /* ------------------------------------------------------------------------ */
 

@@ -31,6 +31,9 @@ void orc_quantize_row_q8_k(const float *x, void *y, int k);                 /* q
 void orc_quantize_batch_q8_k(const float *x, void *y, int rows, int k);     /* gemm_kernels_q8_0.c:221-239 */
 void orc_quantize_row_q8_0(const float *x, void *y, int k);                 /* gemm_kernels_q8_0.c:70-146 */
 void orc_quantize_batch_q8_0(const float *x, void *y, int rows, int k);     /* gemm_kernels_q8_0.c:194-209 */
+/* fused/rmsnorm_q8_k_fused.c:54-142 (as built with FMA; _nofma: product rounded before the add) */
+void orc_rmsnorm_q8_k_fused(const float *input, const float *gamma, void *vy, int tokens, int d_model, int aligned_embed_dim, float eps);
+void orc_rmsnorm_q8_k_fused_nofma(const float *input, const float *gamma, void *vy, int tokens, int d_model, int aligned_embed_dim, float eps);
 
 /* ---- dequantizers (fp32 cross-check reference) ------------------------- */
 void orc_dequant_q4_k_row(const void *src, float *dst, size_t n);           /* dequant_kernels.c:336-385 */

@@ -230,6 +230,24 @@ def main():
                 run(libs["avx2"], "vec_dot_q8_0_q8_0", K, ptr(s), ptr(w), ptr(act))
                 G["s_q8_0_%s_vecdot" % kind] = s
 
+    # ---- fused producer rmsnorm -> Q8_K (both builds must agree: integer output) ----
+    TF, DF, AF = 3, 768, 800                       # row stride larger than d_model
+    xr = normal(S, TF * AF, 0.0, 1.5, 601)
+    xr.reshape(TF, AF)[1, 256:512] = 0.0           # a block of zeros -> zero block
+    xr.reshape(TF, AF)[2, :] *= 40.0               # large magnitudes
+    gam = normal(S, DF, 1.0, 0.4, 602)
+    gam[5] = -gam[5]
+    G["rms_in"], G["rms_gamma"] = xr, gam
+    G["rms_shape"] = np.array([TF, DF, AF], np.int32)
+    G["rms_eps"] = np.array([1e-6], np.float32)
+    outs = {}
+    for tag, L in libs.items():
+        o = np.zeros(TF * (DF // 256) * 292, np.uint8)
+        L.rmsnorm_q8_k_fused(ptr(xr), ptr(gam), ptr(o), TF, DF, AF, ctypes.c_float(1e-6))
+        outs[tag] = o
+    assert np.array_equal(outs["avx2"], outs["avx512"]), "rmsnorm_q8_k_fused differs between builds"
+    G["rms_out"] = outs["avx2"]
+
     np.savez_compressed(OUT, **G)
     print("wrote %s: %d arrays, %.1f KiB" % (OUT, len(G), os.path.getsize(OUT) / 1024.0))
 

@@ -375,6 +375,34 @@ def test_f32act_full_size():
     want = T.np_dequant("q4_k", W).reshape(rows, K).astype(np.float64) @ xf.astype(np.float64)
     assert T.norm_err(y, want) <= TOL
 
+# ---- fused producer: rmsnorm -> Q8_K, bit-exact -----------------------------------------------
+
+def test_rmsnorm_q8_k_fused_golden_host_and_device():
+    G = T.golden()
+    TF, DF, AF = (int(v) for v in G["rms_shape"])
+    x, g, eps = G["rms_in"], G["rms_gamma"], float(G["rms_eps"][0])
+    say("rmsnorm_q8_k_fused golden")
+    assert np.array_equal(P.rmsnorm_q8_k_fused(x, g, TF, DF, AF, eps), G["rms_out"])
+    out = P.dev_rmsnorm_q8_k_fused(P.to_device(x), P.to_device(g), TF, DF, AF, eps).cpu().numpy()
+    assert np.array_equal(out, G["rms_out"])
+
+
+@pytest.mark.parametrize("tokens,D,std,seed", [(1, 256, 1.0, 1), (5, 4096, 1.0, 2), (64, 1024, 30.0, 3),
+                                                (3, 11008 // 256 * 256, 1e-3, 4), (512, 4096, 2.0, 5)])
+def test_rmsnorm_q8_k_fused_bit_exact_vs_oracle(tokens, D, std, seed):
+    x = T.normal(tokens * D, 0.0, std, seed)
+    g = T.normal(D, 1.0, 0.3, seed + 50)
+    say("rmsnorm_q8_k_fused", tokens, D, std)
+    ref = np.zeros(tokens * (D // 256) * 292, np.uint8)
+    T.oracle().orc_rmsnorm_q8_k_fused(T.ptr(x), T.ptr(g), T.ptr(ref), tokens, D, D, ctypes.c_float(1e-6))
+    out = P.dev_rmsnorm_q8_k_fused(P.to_device(x), P.to_device(g), tokens, D).cpu().numpy()
+    assert np.array_equal(out, ref)
+    if tokens <= 8:
+        # feeding the GEMV: same result as quantized-activation GEMV on the oracle's blocks
+        W = T.synth_weights("q4_k", 64, D, seed + 9)
+        y = P.dev_gemm_nt("q4_k", P.to_device(out), P.to_device(W), None, tokens, 64, D).cpu().numpy()
+        assert T.norm_err(y, T.oracle_gemm_nt("q4_k", ref, W, None, tokens, 64, D)) <= TOL
+
 
 # ---- prefill GEMM on the matrix cores (Q4_K, token counts above 16) -------------------------
 

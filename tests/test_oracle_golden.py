@@ -297,6 +297,51 @@ def test_fp32_activation_kernels_match_reference(fmt, kind):
     getattr(O, "orc_gemm_nt_" + fmt)(ptr(xf), ptr(W), None, ptr(c0), TOK, M, K)
     assert np.allclose(c - c0, np.tile(bias, TOK), atol=1e-5 * max(1.0, np.abs(c).max()))
 
+# ---- fused producer: rmsnorm -> Q8_K ---------------------------------------------------
+
+def test_rmsnorm_q8_k_fused_bit_exact_vs_reference():
+    """Both reference builds produce the same bytes; the oracle reproduces them
+    (sum of squares as fused multiply-adds in eight strided lanes).  The variant
+    that rounds the product before the add is a different function: it must
+    differ somewhere on enough data, which pins the choice."""
+    G = T.golden()
+    O = T.oracle()
+    TF, DF, AF = (int(v) for v in G["rms_shape"])
+    x, g, eps = G["rms_in"], G["rms_gamma"], float(G["rms_eps"][0])
+    out = np.zeros_like(G["rms_out"])
+    O.orc_rmsnorm_q8_k_fused(ptr(x), ptr(g), ptr(out), TF, DF, AF, ctypes.c_float(eps))
+    assert np.array_equal(out, G["rms_out"])
+    blocks = out.reshape(-1, 292)
+    # the zeroed input block gives an all-zero output block
+    assert not blocks[1 * (DF // 256) + 1].any()
+    # scale from the largest magnitude: d is negative, and some quant is exactly +-127
+    d = blocks[:, :4].copy().view(np.float32).reshape(-1)
+    qs = blocks[:, 4:260].view(np.int8)
+    live = d != 0
+    assert np.all(d[live] < 0) and np.all(np.abs(qs[live]).max(axis=1) == 127)
+    # bsums are the sums of 16
+    bs = blocks[:, 260:].copy().view(np.int16)
+    assert np.array_equal(bs, qs.reshape(-1, 16, 16).sum(axis=2).astype(np.int16))
+    # closed form: dequantized output is rmsnorm(x)*gamma within half a quantization step
+    xm = x.reshape(TF, AF)[:, :DF].astype(np.float64)
+    want = xm / np.sqrt((xm ** 2).mean(axis=1, keepdims=True) + eps) * g.astype(np.float64)
+    got = (qs.astype(np.float64) * d[:, None].astype(np.float64)).reshape(TF, DF)
+    step = np.abs(d).reshape(TF, DF // 256).repeat(256, axis=1)
+    assert np.all(np.abs(got - want) <= 0.5001 * step + 1e-6 * np.abs(want))
+
+
+def test_rmsnorm_q8_k_fused_fma_choice_is_pinned():
+    O = T.oracle()
+    TF, DF = 64, 1024
+    x = T.normal(TF * DF, 0.0, 30.0, seed=77)
+    g = T.normal(DF, 1.0, 0.3, seed=78)
+    a = np.zeros(TF * (DF // 256) * 292, np.uint8)
+    b = np.zeros_like(a)
+    O.orc_rmsnorm_q8_k_fused(ptr(x), ptr(g), ptr(a), TF, DF, DF, ctypes.c_float(1e-6))
+    O.orc_rmsnorm_q8_k_fused_nofma(ptr(x), ptr(g), ptr(b), TF, DF, DF, ctypes.c_float(1e-6))
+    assert (a != b).sum() > 0          # the two restatements are distinguishable ...
+    assert (a != b).sum() < a.size // 100   # ... and differ only by rounding flips
+
 
 # ---- exact evaluation: dequantize-then-fp64 matmul ---------------------------------
 
