@@ -65,6 +65,12 @@ _SIGS = {
     "gemv_q8_0_q8_0_parallel_simd": (None, [_vp, _vp, _vp, _i, _i, _i, _i]),
     "gemv_q8_0": (None, [_vp, _vp, _vp, _i, _i]),
     "gemm_nt_q8_0_q8_0": (None, [_vp, _vp, _vp, _vp, _i, _i, _i]),
+    "dequant_q4_k_row": (None, [_vp, _vp, _c.c_size_t]),
+    "dequant_q6_k_row": (None, [_vp, _vp, _c.c_size_t]),
+    "dequant_q8_0_row": (None, [_vp, _vp, _c.c_size_t]),
+    "embedding_forward_q4_k": (None, [_vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i]),
+    "embedding_forward_q6_k": (None, [_vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i]),
+    "embedding_forward_q8_0": (None, [_vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i]),
     "rmsnorm_q8_k_fused": (None, [_vp, _vp, _vp, _i, _i, _i, _c.c_float]),
     "gemv_q4_k": (None, [_vp, _vp, _vp, _i, _i]),
     "gemm_q4_k": (None, [_vp, _vp, _vp, _i, _i, _i]),
@@ -100,6 +106,7 @@ _SIGS = {
     "ckq_gemm_nt_q5_k_q8_k_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "ckq_gemm_nt_q6_k_q8_k_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "ckq_gemm_nt_q8_0_q8_0_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "ckq_dequant_rows_dev": (_i, [_i, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp]),
     "ckq_rmsnorm_q8_k_fused_dev": (_i, [_vp, _vp, _vp, _i, _i, _i, _c.c_float, _vp]),
     "ckq_gemm_nt_f32act_dev": (_i, [_i, _vp, _vp, _vp, _vp, _i, _i, _i, _c.c_long, _vp]),
     "ckq_matmul_sequence_dev": (_i, [_vp, _i, _i, _vp]),

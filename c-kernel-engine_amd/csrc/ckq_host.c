@@ -585,6 +585,71 @@ void gemm_nt_q8_0_q8_0(const void *A_q8, const void *B, const float *bias, float
     host_matmul(CKQ_FMT_Q8_0, A_q8, B, bias, C, M, N, K, N, 0, N);
 }
 
+/* Row dequantizers and quantized embedding lookup, any pointer mix, synchronous.
+ * The table is treated like a weight matrix (uploaded once, kept resident). */
+static void host_dequant_rows(int fmt, const void *table, size_t table_rows, const int32_t *ids, int vocab,
+                              const float *pos, float *out, int n_valid, int n_row, int tokens, int n_out_rows)
+{
+    if (!table || !out || n_row <= 0 || n_out_rows <= 0) return;
+    if (n_row % (fmt == CKQ_FMT_Q8_0 ? 32 : 256)) return;
+    if (tokens < 0) tokens = 0;
+    if (tokens > n_out_rows) tokens = n_out_rows;
+    pthread_mutex_lock(&g_mu);
+    do {
+        if (init_locked()) break;
+        const void *dT, *dids = NULL, *dpos = NULL;
+        if (weights_resolve(table, table_rows * ckq_row_bytes(fmt, n_row), &dT)) break;
+        if (ids && tokens > 0 && stage_in(BUF_X, ids, (size_t)tokens * sizeof(int32_t), &dids)) break;
+        if (pos && tokens > 0 && stage_in(BUF_BIAS, pos, (size_t)tokens * n_row * sizeof(float), &dpos)) break;
+        const size_t out_bytes = (size_t)n_out_rows * n_row * sizeof(float);
+        const int on_dev = is_device_ptr(out);
+        void *dout = out;
+        if (!on_dev && buf_reserve(BUF_Y, out_bytes, &dout)) break;
+        int rc = ckq_launch_dequant_rows(fmt, dT, ids ? (const int32_t *)dids : NULL, vocab, (const float *)dpos,
+                                         (float *)dout, n_valid, n_row, tokens, n_out_rows, g_stream);
+        if (rc) { fail(rc, "ckq_launch_dequant_rows"); break; }
+        if (!on_dev) {
+            hipError_t e = hipMemcpyAsync(out, dout, out_bytes, hipMemcpyDeviceToHost, g_stream);
+            if (e != hipSuccess) { fail((int)e, "copy result to host"); break; }
+        }
+        hipError_t e = hipStreamSynchronize(g_stream);
+        if (e != hipSuccess) fail((int)e, "hipStreamSynchronize");
+    } while (0);
+    pthread_mutex_unlock(&g_mu);
+}
+
+void dequant_q4_k_row(const void *src, float *dst, size_t n_elements)
+{
+    if (n_elements == 0 || n_elements > 0x7fffff00u) return;
+    host_dequant_rows(CKQ_FMT_Q4_K, src, 1, NULL, 0, NULL, dst, (int)n_elements, (int)n_elements, 1, 1);
+}
+
+void dequant_q6_k_row(const void *src, float *dst, size_t n_elements)
+{
+    if (n_elements == 0 || n_elements > 0x7fffff00u) return;
+    host_dequant_rows(CKQ_FMT_Q6_K, src, 1, NULL, 0, NULL, dst, (int)n_elements, (int)n_elements, 1, 1);
+}
+
+void dequant_q8_0_row(const void *src, float *dst, size_t n_elements)
+{
+    if (n_elements == 0 || n_elements > 0x7fffffe0u) return;
+    host_dequant_rows(CKQ_FMT_Q8_0, src, 1, NULL, 0, NULL, dst, (int)n_elements, (int)n_elements, 1, 1);
+}
+
+#define DEFINE_EMBEDDING(NAME, FMT)                                                                              \
+    void embedding_forward_##NAME(const int32_t *token_ids, int token_count, int vocab_size,                      \
+                                  const void *token_embeddings, const float *pos_embeddings, float *output,      \
+                                  int embed_dim, int aligned_embed_dim, int context_window, int add_pos)         \
+    {                                                                                                             \
+        if (!token_ids || !token_embeddings || !output || vocab_size <= 0 || context_window <= 0) return;        \
+        host_dequant_rows(FMT, token_embeddings, (size_t)vocab_size, token_ids, vocab_size,                      \
+                          add_pos ? pos_embeddings : NULL, output, embed_dim, aligned_embed_dim, token_count,    \
+                          context_window);                                                                        \
+    }
+DEFINE_EMBEDDING(q4_k, CKQ_FMT_Q4_K)
+DEFINE_EMBEDDING(q6_k, CKQ_FMT_Q6_K)
+DEFINE_EMBEDDING(q8_0, CKQ_FMT_Q8_0)
+
 /* Fused producer: RMSNorm then Q8_K quantization, any pointer mix, synchronous. */
 void rmsnorm_q8_k_fused(const float *input, const float *gamma, void *vy, int tokens, int d_model,
                         int aligned_embed_dim, float eps)
@@ -751,6 +816,12 @@ DEFINE_DEV(q8_0_q8_0, CKQ_FMT_Q8_0)
 int ckq_gemv_q8_0_dev(float *y, const void *W, const float *x, int M, int K, void *stream)
 {
     return ckq_launch_gemv(CKQ_KERNEL_Q80_F32, y, W, x, NULL, M, K, 1, M, 0, M, NULL, stream);
+}
+
+int ckq_dequant_rows_dev(int fmt, const void *table, const int32_t *ids, int vocab, const float *pos, float *out,
+                         int n_valid, int n_row, int tokens, int n_out_rows, void *stream)
+{
+    return ckq_launch_dequant_rows(fmt, table, ids, vocab, pos, out, n_valid, n_row, tokens, n_out_rows, stream);
 }
 
 int ckq_rmsnorm_q8_k_fused_dev(const float *input, const float *gamma, void *y, int tokens, int d_model,

@@ -9,6 +9,7 @@
  *   quantize_q8_k_kernel    fp32 -> Q8_K, bit-exact with the reference
  *   quantize_q8_0_kernel    fp32 -> Q8_0, bit-exact with the reference
  *   rmsnorm_q8_k_fused_kernel  RMSNorm -> Q8_K in one pass, bit-exact with the reference's FMA build
+ *   dequant_rows_kernel     row dequantizers / quantized embedding lookup, bit-exact
  *   copy_kernel             plain streaming copy (counter calibration)
  *   read_kernel             plain streaming read (launch-floor calibration)
  *
@@ -512,6 +513,109 @@ extern "C" int ckq_launch_rmsnorm_q8_k_fused(const float *input, const float *ga
     }
     hipLaunchKernelGGL(rmsnorm_q8_k_fused_kernel, dim3((unsigned)tokens), dim3(256), lds, (hipStream_t)stream,
                        input, gamma, (uint8_t *)y, d_model, (long)aligned_embed_dim, eps);
+    return (int)hipGetLastError();
+}
+
+/* ========================================================================= */
+/* Row dequantizers and quantized embedding lookup                            */
+/* ========================================================================= */
+
+/* Four consecutive elements e..e+3 (e % 4 == 0) of a quantized row, with the
+ * reference's operation order; products and differences are rounded one by one
+ * (reference: dequant_kernels.c:276-296 Q8_0, :336-385 Q4_K, :396-430 Q6_K). */
+template <int FMT>
+__device__ __forceinline__ float4 dequant4(const uint8_t *row, u32 e)
+{
+#pragma clang fp contract(off)
+    float v[4];
+    if (FMT == CKQ_FMT_Q8_0) {
+        const uint8_t *blk = row + (e >> 5) * 34u;
+        const float d = h2f(ld2(blk));
+        const u32 q = ld2(blk + 2 + (e & 31)) | (ld2(blk + 4 + (e & 31)) << 16);
+        for (int i = 0; i < 4; ++i) v[i] = d * (float)sbyte(q, i);
+    } else if (FMT == CKQ_FMT_Q4_K) {
+        const uint8_t *blk = row + (e >> 8) * 144u;
+        const u32 w = e & 255, j = w >> 5, l = w & 31;       /* sub-block j, element l of it */
+        const u32 hdr0 = ld4<4>(blk);
+        u32 sc2, mn2;
+        k4_scale_pair(ld4<4>(blk + 4), ld4<4>(blk + 8), ld4<4>(blk + 12), (int)(j >> 1), &sc2, &mn2);
+        const u32 sc = (sc2 >> (8 * (j & 1))) & 0xff, mn = (mn2 >> (8 * (j & 1))) & 0xff;
+        const float dj = h2f(hdr0 & 0xffff) * (float)sc, mj = h2f(hdr0 >> 16) * (float)mn;
+        const u32 qs = ld4<4>(blk + 16 + 32 * (j >> 1) + l);
+        const u32 nib = (j & 1) ? (qs >> 4) & 0x0f0f0f0fu : qs & 0x0f0f0f0fu;
+        for (int i = 0; i < 4; ++i) v[i] = dj * (float)((nib >> (8 * i)) & 0xff) - mj;
+    } else { /* CKQ_FMT_Q6_K */
+        const uint8_t *blk = row + (e >> 8) * 210u;
+        const u32 w = e & 255, n = w >> 7, r = (w >> 5) & 3, l = w & 31;   /* half n, run r, element l */
+        const uint8_t *ql = blk + 64 * n + l + 32 * (r & 1);
+        const uint8_t *qh = blk + 128 + 32 * n + l;
+        const u32 lo = ld2(ql) | (ld2(ql + 2) << 16), hi = ld2(qh) | (ld2(qh + 2) << 16);
+        const u32 q4 = (r >> 1) ? (lo >> 4) & 0x0f0f0f0fu : lo & 0x0f0f0f0fu;
+        const u32 q2 = (hi >> (2 * r)) & 0x03030303u;
+        const u32 q = q4 | (q2 << 4);
+        const float d = h2f(ld2(blk + 208));
+        const float ds = d * (float)(int8_t)blk[192 + 8 * n + 2 * r + (l >> 4)];
+        for (int i = 0; i < 4; ++i) v[i] = ds * (float)((int)((q >> (8 * i)) & 0xff) - 32);
+    }
+    return make_float4(v[0], v[1], v[2], v[3]);
+}
+
+/*
+ * out[t][0..n_row) for t < n_out_rows: rows t < tokens hold the dequantized
+ * source row (ids ? clamp(ids[t]) : t), plus pos[t] where asked, zero from
+ * n_valid on; rows from `tokens` on are zero (reference:
+ * src/kernels/embedding_kernels.c:76-196).
+ */
+template <int FMT>
+__global__ void __launch_bounds__(256) dequant_rows_kernel(const uint8_t *__restrict__ table, const int32_t *__restrict__ ids,
+                                                           int vocab, const float *__restrict__ pos, float *__restrict__ out,
+                                                           int n_valid, int n_row, long row_bytes, int tokens)
+{
+    const int t = blockIdx.y;
+    const u32 e = 4u * (blockIdx.x * 256u + threadIdx.x);
+    if (e >= (u32)n_row) return;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (t < tokens) {
+        long src = t;
+        if (ids) {
+            const int id = ids[t];
+            src = (id < 0 || id >= vocab) ? 0 : id;
+        }
+        v = dequant4<FMT>(table + src * row_bytes, e);
+        if (pos) {
+            const float4 p = *reinterpret_cast<const float4 *>(pos + (size_t)t * n_row + e);
+            v.x += p.x; v.y += p.y; v.z += p.z; v.w += p.w;
+        }
+        if (e + 0 >= (u32)n_valid) v.x = 0.f;
+        if (e + 1 >= (u32)n_valid) v.y = 0.f;
+        if (e + 2 >= (u32)n_valid) v.z = 0.f;
+        if (e + 3 >= (u32)n_valid) v.w = 0.f;
+    }
+    *reinterpret_cast<float4 *>(out + (size_t)t * n_row + e) = v;
+}
+
+extern "C" int ckq_launch_dequant_rows(int fmt, const void *table, const int32_t *ids, int vocab, const float *pos,
+                                       float *out, int n_valid, int n_row, int tokens, int n_out_rows, void *stream)
+{
+    if (!table || !out || n_row <= 0 || n_out_rows <= 0 || tokens < 0 || n_valid < 0) return CKQ_EINVAL;
+    if (fmt != CKQ_FMT_Q4_K && fmt != CKQ_FMT_Q6_K && fmt != CKQ_FMT_Q8_0) return CKQ_EFORMAT;
+    if (n_row % (fmt == CKQ_FMT_Q8_0 ? 32 : 256)) return CKQ_ESHAPE;
+    if (tokens > n_out_rows) tokens = n_out_rows;
+    if (n_valid > n_row) n_valid = n_row;
+    const long rb = (long)ckq_row_bytes(fmt, n_row);
+    const dim3 grid((unsigned)((n_row / 4 + 255) / 256), (unsigned)n_out_rows), block(256);
+    hipStream_t s = (hipStream_t)stream;
+    switch (fmt) {
+    case CKQ_FMT_Q4_K:
+        hipLaunchKernelGGL(dequant_rows_kernel<CKQ_FMT_Q4_K>, grid, block, 0, s, (const uint8_t *)table, ids, vocab, pos, out, n_valid, n_row, rb, tokens);
+        break;
+    case CKQ_FMT_Q6_K:
+        hipLaunchKernelGGL(dequant_rows_kernel<CKQ_FMT_Q6_K>, grid, block, 0, s, (const uint8_t *)table, ids, vocab, pos, out, n_valid, n_row, rb, tokens);
+        break;
+    default:
+        hipLaunchKernelGGL(dequant_rows_kernel<CKQ_FMT_Q8_0>, grid, block, 0, s, (const uint8_t *)table, ids, vocab, pos, out, n_valid, n_row, rb, tokens);
+        break;
+    }
     return (int)hipGetLastError();
 }
 

@@ -47,6 +47,13 @@ int ckq_launch_quantize_q8_0(const float *x, void *y, int rows, int k, void *str
 int ckq_launch_rmsnorm_q8_k_fused(const float *input, const float *gamma, void *y, int tokens, int d_model,
                                   int aligned_embed_dim, float eps, void *stream);
 
+/* Dequantize rows of a Q4_K / Q6_K / Q8_0 table to fp32: out[t] (n_row floats,
+ * t < n_out_rows) = row (ids ? ids[t] clamped to [0,vocab) else t) for t <
+ * tokens, plus pos[t] when pos is given, zero from element n_valid on; output
+ * rows from `tokens` on are zero. */
+int ckq_launch_dequant_rows(int fmt, const void *table, const int32_t *ids, int vocab, const float *pos,
+                            float *out, int n_valid, int n_row, int tokens, int n_out_rows, void *stream);
+
 /* Plain device copy kernel (calibration of the memory counters / roofline). */
 int ckq_launch_copy(void *dst, const void *src, size_t bytes, void *stream);
 int ckq_launch_read(const void *src, size_t bytes, void *sink, void *stream);

@@ -63,6 +63,19 @@ def gemm_nt(fmt, A_q8, B, bias, M, N, K):
     return c.reshape(M, N)
 
 
+def dequant_row(fmt, src, n):
+    out = np.zeros(n, dtype=np.float32)
+    getattr(lib(), "dequant_%s_row" % fmt)(_p(src), _p(out), n)
+    return out
+
+
+def embedding_forward(fmt, ids, token_count, vocab, table, pos, embed_dim, aligned, context, add_pos, fill=0.0):
+    out = np.full(context * aligned, fill, dtype=np.float32)
+    getattr(lib(), "embedding_forward_" + fmt)(_p(ids), token_count, vocab, _p(table), _p(pos), _p(out),
+                                               embed_dim, aligned, context, add_pos)
+    return out.reshape(context, aligned)
+
+
 def rmsnorm_q8_k_fused(x, gamma, tokens, d_model, aligned=None, eps=1e-6):
     aligned = aligned or d_model
     out = np.zeros(tokens * row_bytes("q8_k", d_model), dtype=np.uint8)
@@ -129,6 +142,14 @@ def dev_gemv_q8_0_f32(W_t, x_t, M, K):
     y = torch.empty(M, dtype=torch.float32, device=W_t.device)
     check(lib().ckq_gemv_q8_0_dev(_dp(y), _dp(W_t), _dp(x_t), M, K, _stream()), "ckq_gemv_q8_0_dev")
     return y
+
+
+def dev_dequant_rows(fmt, table_t, ids_t, vocab, pos_t, n_valid, n_row, tokens, n_out_rows):
+    import torch
+    out = torch.full((n_out_rows * n_row,), 7.0, dtype=torch.float32, device=table_t.device)
+    check(lib().ckq_dequant_rows_dev(FMT[fmt], _dp(table_t), _dp(ids_t), vocab, _dp(pos_t), _dp(out), n_valid, n_row,
+                                     tokens, n_out_rows, _stream()), "ckq_dequant_rows_dev")
+    return out.view(n_out_rows, n_row)
 
 
 def dev_rmsnorm_q8_k_fused(x_t, gamma_t, tokens, d_model, aligned=None, eps=1e-6):

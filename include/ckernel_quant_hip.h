@@ -103,6 +103,27 @@ void  gemm_nt_q6_k(const float *A, const void *B, const float *bias, float *C, i
 void  gemm_q8_0(float *Y, const void *W, const float *X, int M, int N, int K);
 void  gemm_nt_q8_0(const float *A, const void *B, const float *bias, float *C, int M, int N, int K);
 
+/* Row dequantizers and the quantized embedding lookups built on them (the
+ * same block decoders, at the model's input); outputs bit-exact with the
+ * reference.  n_elements / aligned_embed_dim must be a multiple of the block
+ * size.  embedding_forward_*: out[t] = dequant(table[id[t]]) (+ pos[t] when
+ * add_pos and pos_embeddings), ids outside [0,vocab) read row 0, elements from
+ * embed_dim on and rows from token_count on are zero.  Replace
+ * dequant_kernels.c:276-296,336-385,396-430 and
+ * src/kernels/embedding_kernels.c:76-260. */
+void dequant_q4_k_row(const void *src, float *dst, size_t n_elements);
+void dequant_q6_k_row(const void *src, float *dst, size_t n_elements);
+void dequant_q8_0_row(const void *src, float *dst, size_t n_elements);
+void embedding_forward_q4_k(const int32_t *token_ids, int token_count, int vocab_size, const void *token_embeddings,
+                            const float *pos_embeddings, float *output, int embed_dim, int aligned_embed_dim,
+                            int context_window, int add_pos);
+void embedding_forward_q6_k(const int32_t *token_ids, int token_count, int vocab_size, const void *token_embeddings,
+                            const float *pos_embeddings, float *output, int embed_dim, int aligned_embed_dim,
+                            int context_window, int add_pos);
+void embedding_forward_q8_0(const int32_t *token_ids, int token_count, int vocab_size, const void *token_embeddings,
+                            const float *pos_embeddings, float *output, int embed_dim, int aligned_embed_dim,
+                            int context_window, int add_pos);
+
 /* Fused producer of the path's activations: RMSNorm over d_model floats per
  * token (row stride aligned_embed_dim floats) times gamma, quantized to Q8_K
  * in the same pass; vy receives tokens x (d_model/256) blocks.  The block scale
@@ -159,6 +180,13 @@ int ckq_gemm_nt_q4_k_q8_k_dev(const void *A_q8, const void *B, const float *bias
 int ckq_gemm_nt_q5_k_q8_k_dev(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K, void *stream);
 int ckq_gemm_nt_q6_k_q8_k_dev(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K, void *stream);
 int ckq_gemm_nt_q8_0_q8_0_dev(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K, void *stream);
+
+/* Device form of the dequantizers / embedding lookups: out[t] (n_row floats,
+ * 16-byte aligned, t < n_out_rows) = row (ids ? ids[t] clamped : t) of `table`
+ * for t < tokens, plus pos[t] when pos is non-NULL, zero from element n_valid
+ * on; rows from `tokens` on are zero.  fmt: CKQ_FMT_Q4_K, _Q6_K or _Q8_0. */
+int ckq_dequant_rows_dev(int fmt, const void *table, const int32_t *ids, int vocab, const float *pos, float *out,
+                         int n_valid, int n_row, int tokens, int n_out_rows, void *stream);
 
 /* Device form of rmsnorm_q8_k_fused; input rows and gamma 16-byte aligned,
  * d_model <= 40 000 (the row is staged in LDS). */

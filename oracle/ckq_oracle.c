@@ -302,6 +302,34 @@ void orc_dequant_q8_k_row(const void *src, float *dst, size_t n)
         for (int j = 0; j < CKQ_QK_K; ++j) dst[256 * i + j] = b[i].d * (float)b[i].qs[j];
 }
 
+/* Quantized embedding lookup (reference: src/kernels/embedding_kernels.c:76-260):
+ * out[t] = dequant(row id[t]) over aligned_embed_dim elements, + pos[t] over the
+ * first embed_dim when asked, zero from embed_dim on; ids outside [0,vocab)
+ * read row 0; rows t >= token_count (up to context_window) are zero. */
+void orc_embedding_forward(int fmt, const int32_t *token_ids, int token_count, int vocab_size,
+                           const void *token_embeddings, const float *pos_embeddings, float *output,
+                           int embed_dim, int aligned_embed_dim, int context_window, int add_pos)
+{
+    if (!token_ids || !token_embeddings || !output) return;
+    int tokens = token_count < 0 ? 0 : token_count;
+    if (tokens > context_window) tokens = context_window;
+    const size_t rb = ckq_row_bytes(fmt, (size_t)aligned_embed_dim);
+    for (int t = 0; t < tokens; ++t) {
+        int id = token_ids[t];
+        if (id < 0 || id >= vocab_size) id = 0;
+        const uint8_t *row = (const uint8_t *)token_embeddings + (size_t)id * rb;
+        float *out = output + (size_t)t * aligned_embed_dim;
+        if (fmt == CKQ_FMT_Q4_K) orc_dequant_q4_k_row(row, out, (size_t)aligned_embed_dim);
+        else if (fmt == CKQ_FMT_Q6_K) orc_dequant_q6_k_row(row, out, (size_t)aligned_embed_dim);
+        else orc_dequant_q8_0_row(row, out, (size_t)aligned_embed_dim);
+        if (add_pos && pos_embeddings)
+            for (int d = 0; d < embed_dim; ++d) out[d] += pos_embeddings[(size_t)t * aligned_embed_dim + d];
+        for (int d = embed_dim; d < aligned_embed_dim; ++d) out[d] = 0.0f;
+    }
+    for (int t = tokens; t < context_window; ++t)
+        memset(output + (size_t)t * aligned_embed_dim, 0, (size_t)aligned_embed_dim * sizeof(float));
+}
+
 /* ------------------------------------------------------------------------ */
 /* Integer sub-block dots                                                    */
 /* ------------------------------------------------------------------------ */

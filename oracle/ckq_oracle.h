@@ -41,6 +41,10 @@ void orc_dequant_q5_k_row(const void *src, float *dst, size_t n);           /* g
 void orc_dequant_q6_k_row(const void *src, float *dst, size_t n);           /* dequant_kernels.c:396-430 */
 void orc_dequant_q8_0_row(const void *src, float *dst, size_t n);           /* dequant_kernels.c:276-296 */
 void orc_dequant_q8_k_row(const void *src, float *dst, size_t n);           /* d * qs; block layout ckernel_quant.h:153-157 */
+/* src/kernels/embedding_kernels.c:76-260 (fmt: CKQ_FMT_Q4_K, _Q6_K or _Q8_0) */
+void orc_embedding_forward(int fmt, const int32_t *token_ids, int token_count, int vocab_size,
+                           const void *token_embeddings, const float *pos_embeddings, float *output,
+                           int embed_dim, int aligned_embed_dim, int context_window, int add_pos);
 
 /* ---- integer sub-block dots (bit-exact contract) ----------------------- *
  * One weight row against one activation vector.  Output counts per

@@ -248,6 +248,21 @@ def main():
     assert np.array_equal(outs["avx2"], outs["avx512"]), "rmsnorm_q8_k_fused differs between builds"
     G["rms_out"] = outs["avx2"]
 
+    # ---- quantized embedding lookup ----------------------------------------------
+    VOC, ED, AED, CTX, NTOK = 12, 500, 512, 7, 5
+    ids = np.array([3, 11, -2, 40, 0], np.int32)            # two ids outside [0, VOC) -> row 0
+    posv = normal(S, CTX * AED, 0.0, 0.1, 701)
+    G["emb_ids"], G["emb_pos"] = ids, posv
+    G["emb_shape"] = np.array([VOC, ED, AED, CTX, NTOK], np.int32)
+    for fmt in ("q4_k", "q6_k", "q8_0"):
+        tab = random_blocks(S, fmt, VOC * (AED // ELEMS[fmt]), 710 + FMT[fmt])
+        G["emb_table_" + fmt] = tab
+        for add_pos in (0, 1):
+            o = np.full(CTX * AED, 9.0, np.float32)
+            getattr(libs["avx2"], "embedding_forward_" + fmt)(ptr(ids), NTOK, VOC, ptr(tab), ptr(posv), ptr(o),
+                                                               ED, AED, CTX, add_pos)
+            G["emb_out_%s_pos%d" % (fmt, add_pos)] = o
+
     np.savez_compressed(OUT, **G)
     print("wrote %s: %d arrays, %.1f KiB" % (OUT, len(G), os.path.getsize(OUT) / 1024.0))
 

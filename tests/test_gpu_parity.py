@@ -403,6 +403,43 @@ def test_rmsnorm_q8_k_fused_bit_exact_vs_oracle(tokens, D, std, seed):
         y = P.dev_gemm_nt("q4_k", P.to_device(out), P.to_device(W), None, tokens, 64, D).cpu().numpy()
         assert T.norm_err(y, T.oracle_gemm_nt("q4_k", ref, W, None, tokens, 64, D)) <= TOL
 
+# ---- row dequantizers and quantized embedding lookup, bit-exact -----------------------------
+
+@pytest.mark.parametrize("fmt", ["q4_k", "q6_k", "q8_0"])
+def test_dequant_rows_bit_exact(fmt):
+    G = T.golden()
+    w, want = G["deq_%s_w" % fmt], G["deq_%s_out" % fmt]
+    say("dequant row golden", fmt)
+    assert np.array_equal(P.dequant_row(fmt, w, len(want)).view(np.uint32), want.view(np.uint32))
+    # larger, against the oracle
+    n = 64 * 1024
+    W = T.random_blocks(fmt, n // T.ELEMS[fmt], 91)
+    ref = np.zeros(n, np.float32)
+    getattr(T.oracle(), "orc_dequant_%s_row" % fmt)(T.ptr(W), T.ptr(ref), ctypes.c_size_t(n))
+    got = P.dev_dequant_rows(fmt, P.to_device(W), None, 0, None, n, n, 1, 1).cpu().numpy().reshape(-1)
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
+
+
+@pytest.mark.parametrize("fmt", ["q4_k", "q6_k", "q8_0"])
+@pytest.mark.parametrize("add_pos", [0, 1])
+def test_embedding_forward_golden_and_oracle(fmt, add_pos):
+    G = T.golden()
+    VOC, ED, AED, CTX, NTOK = (int(v) for v in G["emb_shape"])
+    ids, pos, tab = G["emb_ids"], G["emb_pos"], G["emb_table_" + fmt]
+    say("embedding golden", fmt, add_pos)
+    out = P.embedding_forward(fmt, ids, NTOK, VOC, tab, pos, ED, AED, CTX, add_pos, fill=9.0)
+    assert np.array_equal(out.reshape(-1).view(np.uint32), G["emb_out_%s_pos%d" % (fmt, add_pos)].view(np.uint32))
+    # a model-sized lookup on the device: 64 tokens of a 32000 x 4096 table (Q8_0: 151936 x 896)
+    voc, dim = (151936, 896) if fmt == "q8_0" else (32000, 4096)
+    tabL = T.random_blocks(fmt, voc * (dim // T.ELEMS[fmt]), 92)
+    idsL = np.random.default_rng(5).integers(-3, voc + 3, size=64).astype(np.int32)
+    posL = T.normal(80 * dim, 0.0, 0.1, seed=93)
+    ref = np.full(80 * dim, 9.0, np.float32)
+    T.oracle().orc_embedding_forward(T.FMT[fmt], T.ptr(idsL), 64, voc, T.ptr(tabL), T.ptr(posL), T.ptr(ref), dim - 8, dim, 80, add_pos)
+    got = P.dev_dequant_rows(fmt, P.to_device(tabL), P.to_device(idsL), voc, P.to_device(posL) if add_pos else None,
+                             dim - 8, dim, 64, 80).cpu().numpy().reshape(-1)
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
+
 
 # ---- prefill GEMM on the matrix cores (Q4_K, token counts above 16) -------------------------
 

@@ -342,6 +342,29 @@ def test_rmsnorm_q8_k_fused_fma_choice_is_pinned():
     assert (a != b).sum() > 0          # the two restatements are distinguishable ...
     assert (a != b).sum() < a.size // 100   # ... and differ only by rounding flips
 
+# ---- quantized embedding lookup ----------------------------------------------------------
+
+@pytest.mark.parametrize("fmt", ["q4_k", "q6_k", "q8_0"])
+@pytest.mark.parametrize("add_pos", [0, 1])
+def test_embedding_forward_bit_exact_vs_reference(fmt, add_pos):
+    G = T.golden()
+    VOC, ED, AED, CTX, NTOK = (int(v) for v in G["emb_shape"])
+    ids, pos, tab = G["emb_ids"], G["emb_pos"], G["emb_table_" + fmt]
+    out = np.full(CTX * AED, 9.0, np.float32)
+    T.oracle().orc_embedding_forward(T.FMT[fmt], ptr(ids), NTOK, VOC, ptr(tab), ptr(pos), ptr(out), ED, AED, CTX, add_pos)
+    want = G["emb_out_%s_pos%d" % (fmt, add_pos)]
+    assert np.array_equal(out.view(np.uint32), want.view(np.uint32))
+    # what the lookup must mean, from the format decoders: gathered rows, clamped ids, padding
+    o = out.reshape(CTX, AED)
+    rows = T.np_dequant(fmt, tab).reshape(VOC, AED)
+    p = pos.reshape(CTX, AED)
+    for t in range(NTOK):
+        idx = int(ids[t]) if 0 <= ids[t] < VOC else 0
+        exp = rows[idx, :ED] + (p[t, :ED] if add_pos else 0.0)
+        assert np.allclose(o[t, :ED], exp, rtol=1e-6, atol=1e-7)
+        assert np.all(o[t, ED:] == 0.0)
+    assert np.all(o[NTOK:] == 0.0)
+
 
 # ---- exact evaluation: dequantize-then-fp64 matmul ---------------------------------
 
