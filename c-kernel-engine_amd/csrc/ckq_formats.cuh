@@ -79,9 +79,21 @@ struct FmtQ4K {
         a.b_lo = (int)(int16_t)(bs[0] & 0xffff) + (int)(int16_t)(bs[0] >> 16);
         a.b_hi = (int)(int16_t)(bs[1] & 0xffff) + (int)(int16_t)(bs[1] >> 16);
     }
-    /* LDS image of the staged activations: 16-byte unit u of the rows sits at unit xs_unit(u) */
-    static __device__ __forceinline__ u32 xs_unit(u32 u) { return u; }
-    static __device__ __forceinline__ void load_act_lds(Act &a, const uint8_t *xs, int pos) { load_act(a, xs, pos); }
+    /* Staging of the token tile's activation rows in LDS: units of XS_SRC
+     * source bytes travel through XS_REGS registers; here the LDS image is a
+     * plain copy. */
+    static constexpr int XS_SRC = 16, XS_REGS = 4;
+    static __host__ __device__ __forceinline__ size_t xs_lds_bytes(size_t tile_bytes) { return tile_bytes; }
+    static __device__ __forceinline__ void xs_ld(u32 (&v)[XS_REGS], const uint8_t *p) { ld16<XBLOCK % 4 == 0 ? 4 : 2>(v, p); }
+    static __device__ __forceinline__ void xs_st(uint8_t *xs, const u32 (&v)[XS_REGS], u32 unit, u32)
+    {
+        u32 *d = reinterpret_cast<u32 *>(xs + 16u * unit);
+        d[0] = v[0]; d[1] = v[1]; d[2] = v[2]; d[3] = v[3];
+    }
+    static __device__ __forceinline__ void load_act_lds(Act &a, const uint8_t *xs, int tl, int pos, u32 xrow, int, u32)
+    {
+        load_act(a, xs + (u32)tl * xrow, pos);
+    }
     static __device__ __forceinline__ void decode(Dec &d, const Wt &w, int pos)
     {
         u32 sc2, mn2;
@@ -139,9 +151,21 @@ struct FmtQ5K {
         ld16<4>(w.qs + 4, row + o.qs + 16);
     }
     static __device__ __forceinline__ void load_act(Act &a, const uint8_t *x, int pos) { FmtQ4K::load_act(a, x, pos); }
-    /* LDS image of the staged activations: 16-byte unit u of the rows sits at unit xs_unit(u) */
-    static __device__ __forceinline__ u32 xs_unit(u32 u) { return u; }
-    static __device__ __forceinline__ void load_act_lds(Act &a, const uint8_t *xs, int pos) { load_act(a, xs, pos); }
+    /* Staging of the token tile's activation rows in LDS: units of XS_SRC
+     * source bytes travel through XS_REGS registers; here the LDS image is a
+     * plain copy. */
+    static constexpr int XS_SRC = 16, XS_REGS = 4;
+    static __host__ __device__ __forceinline__ size_t xs_lds_bytes(size_t tile_bytes) { return tile_bytes; }
+    static __device__ __forceinline__ void xs_ld(u32 (&v)[XS_REGS], const uint8_t *p) { ld16<XBLOCK % 4 == 0 ? 4 : 2>(v, p); }
+    static __device__ __forceinline__ void xs_st(uint8_t *xs, const u32 (&v)[XS_REGS], u32 unit, u32)
+    {
+        u32 *d = reinterpret_cast<u32 *>(xs + 16u * unit);
+        d[0] = v[0]; d[1] = v[1]; d[2] = v[2]; d[3] = v[3];
+    }
+    static __device__ __forceinline__ void load_act_lds(Act &a, const uint8_t *xs, int tl, int pos, u32 xrow, int, u32)
+    {
+        load_act(a, xs + (u32)tl * xrow, pos);
+    }
     static __device__ __forceinline__ void decode(Dec &d, const Wt &w, int pos)
     {
         const int g = pos & 3;
@@ -204,9 +228,21 @@ struct FmtQ6K {
             a.a32[r] = 32 * s;   /* computed from the quants: the reference's x86 routine never reads bsums here */
         }
     }
-    /* LDS image of the staged activations: 16-byte unit u of the rows sits at unit xs_unit(u) */
-    static __device__ __forceinline__ u32 xs_unit(u32 u) { return u; }
-    static __device__ __forceinline__ void load_act_lds(Act &a, const uint8_t *xs, int pos) { load_act(a, xs, pos); }
+    /* Staging of the token tile's activation rows in LDS: units of XS_SRC
+     * source bytes travel through XS_REGS registers; here the LDS image is a
+     * plain copy. */
+    static constexpr int XS_SRC = 16, XS_REGS = 4;
+    static __host__ __device__ __forceinline__ size_t xs_lds_bytes(size_t tile_bytes) { return tile_bytes; }
+    static __device__ __forceinline__ void xs_ld(u32 (&v)[XS_REGS], const uint8_t *p) { ld16<XBLOCK % 4 == 0 ? 4 : 2>(v, p); }
+    static __device__ __forceinline__ void xs_st(uint8_t *xs, const u32 (&v)[XS_REGS], u32 unit, u32)
+    {
+        u32 *d = reinterpret_cast<u32 *>(xs + 16u * unit);
+        d[0] = v[0]; d[1] = v[1]; d[2] = v[2]; d[3] = v[3];
+    }
+    static __device__ __forceinline__ void load_act_lds(Act &a, const uint8_t *xs, int tl, int pos, u32 xrow, int, u32)
+    {
+        load_act(a, xs + (u32)tl * xrow, pos);
+    }
     static __device__ __forceinline__ void decode(Dec &d, const Wt &w, int pos)
     {
         const int odd = pos & 1;
@@ -273,9 +309,31 @@ struct FmtQ80 {
         ld16<2>(a.q, blk + 2);
         ld16<2>(a.q + 4, blk + 18);
     }
-    /* LDS image of the staged activations: 16-byte unit u of the rows sits at unit xs_unit(u) */
-    static __device__ __forceinline__ u32 xs_unit(u32 u) { return u; }
-    static __device__ __forceinline__ void load_act_lds(Act &a, const uint8_t *xs, int pos) { load_act(a, xs, pos); }
+    /* Staging of the token tile's activation rows in LDS.  A 34-byte block at a
+     * 2-byte aligned address makes every 16-byte LDS read misaligned, so the
+     * tile is re-laid out: the quants of block j at byte 32 j, its scale as
+     * fp32 at 32 * total + 4 j. */
+    static constexpr int XS_SRC = 34, XS_REGS = 9;
+    static __host__ __device__ __forceinline__ size_t xs_lds_bytes(size_t tile_bytes) { return tile_bytes / 34 * 36; }
+    static __device__ __forceinline__ void xs_ld(u32 (&v)[XS_REGS], const uint8_t *p)
+    {
+        v[8] = ld2(p);
+        ld16<2>(v, p + 2);
+        ld16<2>(v + 4, p + 18);
+    }
+    static __device__ __forceinline__ void xs_st(uint8_t *xs, const u32 (&v)[XS_REGS], u32 unit, u32 total)
+    {
+        u32 *d = reinterpret_cast<u32 *>(xs + 32u * unit);
+        for (int i = 0; i < 8; ++i) d[i] = v[i];
+        *reinterpret_cast<float *>(xs + 32u * total + 4u * unit) = h2f(v[8]);
+    }
+    static __device__ __forceinline__ void load_act_lds(Act &a, const uint8_t *xs, int tl, int pos, u32, int npos, u32 total)
+    {
+        const u32 j = (u32)tl * (u32)npos + (u32)pos;
+        const u32 *q = reinterpret_cast<const u32 *>(xs + 32u * j);
+        for (int i = 0; i < 8; ++i) a.q[i] = (int)q[i];
+        a.d = *reinterpret_cast<const float *>(xs + 32u * total + 4u * j);
+    }
     static __device__ __forceinline__ void decode(Dec &d, const Wt &w, int)
     {
         for (int i = 0; i < 8; ++i) d.q[i] = (int)w.q[i];
@@ -317,7 +375,15 @@ struct FmtQ80F32 {
     /* A lane reads a run of consecutive 16-byte units; lanes are 128 bytes
      * apart, so unswizzled they would all hit the same LDS banks. */
     static __device__ __forceinline__ u32 xs_unit(u32 u) { return u ^ ((u >> 4) & 15u); }
-    static __device__ __forceinline__ void load_act_lds(Act &a, const uint8_t *xs, int pos)
+    static constexpr int XS_SRC = 16, XS_REGS = 4;
+    static __host__ __device__ __forceinline__ size_t xs_lds_bytes(size_t tile_bytes) { return (tile_bytes + 255) & ~(size_t)255; }
+    static __device__ __forceinline__ void xs_ld(u32 (&v)[XS_REGS], const uint8_t *p) { ld16<4>(v, p); }
+    static __device__ __forceinline__ void xs_st(uint8_t *xs, const u32 (&v)[XS_REGS], u32 unit, u32)
+    {
+        u32 *d = reinterpret_cast<u32 *>(xs + 16u * xs_unit(unit));
+        d[0] = v[0]; d[1] = v[1]; d[2] = v[2]; d[3] = v[3];
+    }
+    static __device__ __forceinline__ void load_act_lds(Act &a, const uint8_t *xs, int, int pos, u32, int, u32)
     {
         for (int i = 0; i < 8; ++i) {
             u32 t[4];
@@ -364,7 +430,15 @@ struct FmtQ4KF32 {
     /* lanes are 256 bytes apart: swizzle the unit index so 16 lanes reading
      * their i-th unit touch 16 different bank groups */
     static __device__ __forceinline__ u32 xs_unit(u32 u) { return u ^ ((u >> 4) & 15u); }
-    static __device__ __forceinline__ void load_act_lds(Act &a, const uint8_t *xs, int pos)
+    static constexpr int XS_SRC = 16, XS_REGS = 4;
+    static __host__ __device__ __forceinline__ size_t xs_lds_bytes(size_t tile_bytes) { return (tile_bytes + 255) & ~(size_t)255; }
+    static __device__ __forceinline__ void xs_ld(u32 (&v)[XS_REGS], const uint8_t *p) { ld16<4>(v, p); }
+    static __device__ __forceinline__ void xs_st(uint8_t *xs, const u32 (&v)[XS_REGS], u32 unit, u32)
+    {
+        u32 *d = reinterpret_cast<u32 *>(xs + 16u * xs_unit(unit));
+        d[0] = v[0]; d[1] = v[1]; d[2] = v[2]; d[3] = v[3];
+    }
+    static __device__ __forceinline__ void load_act_lds(Act &a, const uint8_t *xs, int, int pos, u32, int, u32)
     {
         for (int i = 0; i < 16; ++i) {
             u32 t[4];
@@ -416,7 +490,15 @@ struct FmtQ6KF32 {
             }
     }
     static __device__ __forceinline__ u32 xs_unit(u32 u) { return u ^ ((u >> 4) & 15u); }
-    static __device__ __forceinline__ void load_act_lds(Act &a, const uint8_t *xs, int pos)
+    static constexpr int XS_SRC = 16, XS_REGS = 4;
+    static __host__ __device__ __forceinline__ size_t xs_lds_bytes(size_t tile_bytes) { return (tile_bytes + 255) & ~(size_t)255; }
+    static __device__ __forceinline__ void xs_ld(u32 (&v)[XS_REGS], const uint8_t *p) { ld16<4>(v, p); }
+    static __device__ __forceinline__ void xs_st(uint8_t *xs, const u32 (&v)[XS_REGS], u32 unit, u32)
+    {
+        u32 *d = reinterpret_cast<u32 *>(xs + 16u * xs_unit(unit));
+        d[0] = v[0]; d[1] = v[1]; d[2] = v[2]; d[3] = v[3];
+    }
+    static __device__ __forceinline__ void load_act_lds(Act &a, const uint8_t *xs, int, int pos, u32, int, u32)
     {
         const int n = (pos >> 1) & 1, l0 = 16 * (pos & 1);
         const u32 u0 = 64u * (u32)(pos >> 2) + (u32)(128 * n + l0) / 4u;      /* unit of the first float */

@@ -59,7 +59,7 @@ __device__ __forceinline__ int wave_in_block() { return __builtin_amdgcn_readfir
  * stores.
  */
 template <class F, int LPR, int PPL, int MT, int RPI, bool DUMP, int WPB, bool LDSX>
-__global__ void __launch_bounds__(64 * WPB) __attribute__((amdgpu_waves_per_eu(MT == 1 && !DUMP && PPL == 1 && RPI == 1 ? F::OCC1 : 1)))
+__global__ void __launch_bounds__(64 * WPB) __attribute__((amdgpu_waves_per_eu(MT == 1 && !DUMP && PPL == 1 && RPI == 1 ? F::OCC1 : MT >= 4 && PPL == 1 ? 4 : 1)))
 gemv_kernel(GemvArgs a)
 {
     constexpr int SLOTS = 64 / LPR;
@@ -78,16 +78,16 @@ gemv_kernel(GemvArgs a)
      * once in LDS instead of once per wave through the vector cache.  Their
      * loads go out first, all at once (one round trip, they hit in L2), the
      * weight loads follow, and only then are the staged values written. */
-    constexpr int XA = F::XBLOCK % 4 == 0 ? 4 : 2;
     constexpr int XNT = 64 * WPB, XU = MT == 1 ? 2 : 4;
     const uint8_t *xsrc = a.X + (size_t)t0 * a.xrow;
-    const int xbytes = (int)((long)min(MT, a.ntok - t0) * a.xrow), xn16 = xbytes >> 4;
-    u32 xv[XU][4];
+    const int xbytes = (int)((long)min(MT, a.ntok - t0) * a.xrow), xn = xbytes / F::XS_SRC;   /* staging units */
+    const u32 xcap = (u32)((long)MT * a.xrow / F::XS_SRC);                                     /* units of a full tile */
+    u32 xv[XU][F::XS_REGS];
     if (LDSX) {
 #pragma unroll
         for (int u = 0; u < XU; ++u) {
             const int i = u * XNT + (int)threadIdx.x;
-            if (i < xn16) ld16<XA>(xv[u], xsrc + 16u * (u32)i);
+            if (i < xn) F::xs_ld(xv[u], xsrc + (u32)F::XS_SRC * (u32)i);
         }
     }
 
@@ -103,7 +103,7 @@ gemv_kernel(GemvArgs a)
 
     for (int p0 = 0; p0 < a.npos; p0 += LPR * PPL) {
         typename F::Wt  w[RPI][PPL];
-        typename F::Act act[MT][PPL];
+        typename F::Act act[MT >= 4 ? 1 : MT][PPL];   /* wide tiles stream their activations instead */
 #pragma unroll
         for (int p = 0; p < PPL; ++p) {
             const int pos = min(p0 + p * LPR + l, a.npos - 1);
@@ -121,24 +121,53 @@ gemv_kernel(GemvArgs a)
 #pragma unroll
             for (int u = 0; u < XU; ++u) {
                 const int i = u * XNT + (int)threadIdx.x;
-                if (i < xn16) {
-                    u32 *d = reinterpret_cast<u32 *>(xs + 16u * F::xs_unit((u32)i));
-                    d[0] = xv[u][0]; d[1] = xv[u][1]; d[2] = xv[u][2]; d[3] = xv[u][3];
+                if (i < xn) F::xs_st(xs, xv[u], (u32)i, xcap);
+            }
+            for (int i = XNT * XU + (int)threadIdx.x; i < xn; i += XNT) {       /* long token tiles */
+                u32 v[F::XS_REGS];
+                F::xs_ld(v, xsrc + (u32)F::XS_SRC * (u32)i);
+                F::xs_st(xs, v, (u32)i, xcap);
+            }
+            if (F::XS_SRC == 16) {
+                const int tail = (xbytes & 15) >> 1;  /* plain-copy images: rows are a whole number of 2-byte units */
+                if ((int)threadIdx.x < tail) {
+                    const u32 o = 16u * (u32)xn + 2u * threadIdx.x;
+                    *reinterpret_cast<uint16_t *>(xs + o) = (uint16_t)ld2(xsrc + o);
                 }
-            }
-            for (int i = XNT * XU + (int)threadIdx.x; i < xn16; i += XNT) {     /* long token tiles */
-                u32 v[4];
-                ld16<XA>(v, xsrc + 16u * (u32)i);
-                u32 *d = reinterpret_cast<u32 *>(xs + 16u * F::xs_unit((u32)i));
-                d[0] = v[0]; d[1] = v[1]; d[2] = v[2]; d[3] = v[3];
-            }
-            const int tail = (xbytes & 15) >> 1;      /* rows are a whole number of 2-byte units */
-            if ((int)threadIdx.x < tail) {
-                const u32 o = 16u * (u32)xn16 + 2u * threadIdx.x;
-                *reinterpret_cast<uint16_t *>(xs + o) = (uint16_t)ld2(xsrc + o);
             }
             __syncthreads();
         }
+        if constexpr (MT >= 4) {
+            /* wide token tiles: the weights of a position are decoded once, then
+             * the tokens' activations stream through from LDS one at a time
+             * (holding all of them in registers would leave two waves per SIMD) */
+#pragma unroll
+            for (int p = 0; p < PPL; ++p) {
+                const int  upos  = p0 + p * LPR + l;
+                const bool valid = upos < a.npos;
+                const int  pos   = min(upos, a.npos - 1);
+                typename F::Dec dec[RPI];
+#pragma unroll
+                for (int r = 0; r < RPI; ++r) F::decode(dec[r], w[r][p], pos);
+#pragma unroll
+                for (int t = 0; t < MT; ++t) {
+                    typename F::Act at;
+                    if (LDSX) {
+                        const int tl = min(t, a.ntok - t0 - 1);                    /* uniform */
+                        F::load_act_lds(at, xs, tl, pos, (u32)a.xrow, a.npos, xcap);
+                    } else {
+                        const int tok = min(t0 + t, a.ntok - 1);                   /* uniform */
+                        F::load_act(at, a.X + (size_t)tok * a.xrow, pos);
+                    }
+#pragma unroll
+                    for (int r = 0; r < RPI; ++r) {
+                        int sub[F::NSUB];
+                        const float v = F::dot(dec[r], at, sub);
+                        acc[r][t] += valid ? v : 0.0f;
+                    }
+                }
+            }
+        } else {
 #pragma unroll
         for (int p = 0; p < PPL; ++p) {
             const int pos = min(p0 + p * LPR + l, a.npos - 1);
@@ -146,7 +175,7 @@ gemv_kernel(GemvArgs a)
             for (int t = 0; t < MT; ++t) {
                 if (LDSX) {
                     const int tl = min(t, a.ntok - t0 - 1);                    /* uniform */
-                    F::load_act_lds(act[t][p], xs + (u32)tl * (u32)a.xrow, pos);
+                    F::load_act_lds(act[t][p], xs, tl, pos, (u32)a.xrow, a.npos, xcap);
                 } else {
                     const int tok = min(t0 + t, a.ntok - 1);                   /* uniform */
                     F::load_act(act[t][p], a.X + (size_t)tok * a.xrow, pos);
@@ -175,6 +204,7 @@ gemv_kernel(GemvArgs a)
                 }
             }
         }
+        }
     }
 
 #pragma unroll
@@ -194,8 +224,7 @@ static int launch_one(const GemvArgs &a, hipStream_t s)
     constexpr int rows_per_block = WPB * (64 / LPR) * RPI;
     const int nr = a.row1 - a.row0;
     dim3 grid((nr + rows_per_block - 1) / rows_per_block, (a.ntok + MT - 1) / MT);
-    /* whole 256-byte groups: a format may permute the 16-byte units inside one */
-    const size_t lds = LDSX ? (((size_t)MT * (size_t)a.xrow + 255) & ~(size_t)255) : 0;
+    const size_t lds = LDSX ? F::xs_lds_bytes((size_t)MT * (size_t)a.xrow) : 0;
     hipLaunchKernelGGL((gemv_kernel<F, LPR, PPL, MT, RPI, DUMP, WPB, LDSX>), grid, dim3(64 * WPB), lds, s, a);
     return (int)hipGetLastError();
 }
@@ -204,7 +233,7 @@ static int launch_one(const GemvArgs &a, hipStream_t s)
 template <class F, int LPR, int PPL, int MT, int RPI, int WPB>
 static int launch_tile(const GemvArgs &a, hipStream_t s)
 {
-    if ((size_t)MT * (size_t)a.xrow <= 65536) return launch_one<F, LPR, PPL, MT, RPI, false, WPB, true>(a, s);
+    if (F::xs_lds_bytes((size_t)MT * (size_t)a.xrow) <= 65536) return launch_one<F, LPR, PPL, MT, RPI, false, WPB, true>(a, s);
     return launch_one<F, LPR, PPL, MT, RPI, false, WPB, false>(a, s);
 }
 
