@@ -254,6 +254,12 @@ static int launch_mt(const GemvArgs &a, bool dump, int max_mt, hipStream_t s)
          * staging per weight byte) */
         const long waves = ((long)(a.row1 - a.row0) * LPR + 63) / 64;
         if (PPL == 1 && waves > 16384) return launch_tile<F, LPR, PPL, 1, 2, 4>(a, s);
+        /* rows longer than one pass: each staged activation row is shared
+         * between eight weight rows, as 512-thread blocks (a whole number of
+         * blocks per CU on the usual projection shapes) or, for the largest
+         * matrices, two rows per slot */
+        if (PPL > 1 && a.row1 - a.row0 >= 8192) return launch_tile<F, LPR, PPL, 1, 2, 4>(a, s);
+        if (PPL > 1 && a.row1 - a.row0 >= 2048) return launch_tile<F, LPR, PPL, 1, 1, 8>(a, s);
         return launch_tile<F, LPR, PPL, 1, 1, 4>(a, s);
     }
     if constexpr (F::TOKEN_TILES) {
