@@ -1,0 +1,266 @@
+/*
+ * ckq_gemm_q6k_mfma.cuh - prefill GEMM, Q6_K weights x Q8_K activations, on the
+ * gfx950 int8 matrix cores.
+ *
+ *   C[t][n] = sum_b (dw(n,b) * dx(t,b)) * (float) I(t,n,b)   (+ bias[n])
+ *   I = sum_{s<16} sc(n,b,s) * sum_{k in 16-run s} (q6(n,k) - 32) * q8(t,k)     (exact int32)
+ * which is the per-block arithmetic of the reference's x86 dot product
+ * (gemm_kernels_q6k_q8k.c:601-695: integer sum per block, one fp32 scale per
+ * block) under its token loop (gemm_kernels_q6k_q8k.c:1243-1268).
+ *
+ * Mapping to the hardware
+ * - v_mfma_i32_32x32x32_i8 takes 32 k per instruction; a lane supplies the 16 k
+ *   of one half, which is exactly one 16-run of a Q6_K block, so every lane
+ *   works with ONE int8 scale per instruction.
+ * - The scaled weight v = sc * (q6 - 32) needs 14 bits.  It is formed once per
+ *   weight in 16-bit lanes (v_pk_mad_u16 on byte pairs) and split into two int8
+ *   planes v = 256 * H + L, L = the signed low byte of v, H = the high byte of
+ *   v + 128; both planes are accumulated over the whole 256-block and
+ *   I = 256 * IH + IL exactly.  The split costs nothing: the two planes are the
+ *   byte lanes of the 16-bit products, gathered with v_perm_b32.
+ * - Operands reach LDS by 16-byte global->LDS loads.  A 210-byte block is
+ *   fetched as 14 chunks; the last one starts at byte 194 so that no load
+ *   reaches past the block (it carries the fp16 scale in its last two bytes).
+ *   Rows are only 2-byte aligned in memory; the loads accept that.  Quants
+ *   are laid out as in the Q4_K kernel (chunks XOR-swizzled by token).
+ * - Block = 4 waves = (32 * TH tokens) x 128 weight rows, wave w owns rows
+ *   32w..32w+31 and all TH token groups of 32.  The kernel is bound by VALU
+ *   issue (about 11 operations per 4 weights against one MFMA per 512 weight
+ *   bytes), so plane expansion of k-slab s+1 is interleaved with the MFMAs of
+ *   slab s and larger token tiles (TH = 4) amortise it where the grid is big
+ *   enough to fill the chip with them.
+ */
+#pragma once
+#include "ckq_gemm_mfma.cuh"
+
+constexpr int GEMM6_BN  = 128;   /* weight rows per tile */
+constexpr int GEMM6_ROW = 224;   /* LDS bytes per staged weight block: 14 chunks */
+
+template <int TH> struct Gemm6Stage {
+    uint8_t w[GEMM6_BN * GEMM6_ROW];   /* row r at 224 r: chunks 0-12 = block bytes 0..207, chunk 13 = bytes 194..209 */
+    uint8_t q[32 * TH * 256];          /* int8 quants: 16-byte chunk c of token t in slot c ^ (t & 15) of its 256 bytes */
+    float   d[32 * TH];                /* block scale of each token */
+};
+
+__device__ __forceinline__ u32 pk_mad_u16(u32 a, u32 b, u32 c)
+{
+    const ckq_v2u16 x = __builtin_bit_cast(ckq_v2u16, a), y = __builtin_bit_cast(ckq_v2u16, b),
+                    z = __builtin_bit_cast(ckq_v2u16, c);
+    return __builtin_bit_cast(u32, (ckq_v2u16)(x * y + z));
+}
+
+/* One 256-block of a tile: eight k-slabs of 32, each 2*TH MFMAs (TH token
+ * groups x two planes).  The planes of slab s+1 are expanded between the MFMAs
+ * of slab s; copy_one(i) issues one global->LDS copy of the next block. */
+template <int TH, int NCOPY, class CopyFn>
+__device__ __forceinline__ void gemm6_block(const Gemm6Stage<TH> &st, u32 wrow, const u32 (&aofs)[8], int half,
+                                            ckq_v16f (&acc)[TH], CopyFn copy_one)
+{
+#define CKQ_PIN() __builtin_amdgcn_sched_barrier(0)
+    auto lds16 = [&](const uint8_t *p) { return *reinterpret_cast<const ckq_v4i *>(p); };
+    const uint8_t *wr = st.w + wrow;
+
+    /* raw block of this lane's row: the 16-byte runs its k-half touches */
+    ckq_v4i ql[2][2], qh[2];
+#pragma unroll
+    for (int n = 0; n < 2; ++n) {
+#pragma unroll
+        for (int odd = 0; odd < 2; ++odd) ql[n][odd] = lds16(wr + 16 * (4 * n + 2 * odd + half));
+        qh[n] = lds16(wr + 16 * (8 + 2 * n + half));
+    }
+    const ckq_v4i scv = lds16(wr + 192);
+    const float dw = h2f(*reinterpret_cast<const uint16_t *>(wr + 222));
+    const int sh0 = 8 * half, sh1 = 16 + 8 * half;   /* scale of slab s: byte 2 (s & 1) + half of dword s >> 1 */
+
+    ckq_v4i av[2][TH];
+    auto a_read = [&](int s) {
+#pragma unroll
+        for (int ts = 0; ts < TH; ++ts) av[s & 1][ts] = lds16(&st.q[aofs[s] + 32 * 256 * ts]);
+    };
+
+    u32 scp[2], cp[2];
+    ckq_v4i pL[2], pH[2];
+    auto prep = [&](int s) {
+        const int sc = __builtin_amdgcn_sbfe(scv[s >> 1], (s & 1) ? sh1 : sh0, 8);
+        scp[s & 1] = __builtin_amdgcn_perm((u32)sc, (u32)sc, 0x05040504u);          /* sc in both 16-bit lanes */
+        cp[s & 1]  = pk_mad_u16(scp[s & 1], 0xFFE0FFE0u, 0x00800080u);              /* 128 - 32 sc */
+    };
+    auto decode = [&](int s, int i) {
+        const int n = s >> 2, g = s & 3;
+        const u32 lw = (u32)ql[n][g & 1][i], hw = (u32)qh[n][i];
+        const u32 nib = g < 2 ? (lw & 0x0f0f0f0fu) : ((lw >> 4) & 0x0f0f0f0fu);
+        const u32 hb = g == 0 ? (hw << 4) : g == 1 ? (hw << 2) : g == 2 ? hw : (hw >> 2);
+        const u32 q = (hb & 0x30303030u) | nib;                                   /* four 6-bit values */
+        const u32 e = __builtin_amdgcn_perm(0u, q, 0x0c020c00u);                  /* bytes 0, 2 in 16-bit lanes */
+        const u32 o = __builtin_amdgcn_perm(0u, q, 0x0c030c01u);                  /* bytes 1, 3 */
+        const u32 te = pk_mad_u16(e, scp[s & 1], cp[s & 1]);                      /* sc * (q - 32) + 128 */
+        const u32 to = pk_mad_u16(o, scp[s & 1], cp[s & 1]);
+        pL[s & 1][i] = (int)(__builtin_amdgcn_perm(to, te, 0x06020400u) ^ 0x80808080u);
+        pH[s & 1][i] = (int)__builtin_amdgcn_perm(to, te, 0x07030501u);
+    };
+
+    ckq_v16i iL[TH], iH[TH];
+    const ckq_v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+
+    a_read(0);
+    prep(0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) decode(0, i);
+    CKQ_PIN();
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+        if (s < 7) { a_read(s + 1); prep(s + 1); }
+#pragma unroll
+        for (int k = 0; k < 2 * TH; ++k) {
+            const int ts = k >> 1;
+            if ((k & 1) == 0) iL[ts] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[s & 1][ts], pL[s & 1], s == 0 ? zero16 : iL[ts], 0, 0, 0);
+            else              iH[ts] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[s & 1][ts], pH[s & 1], s == 0 ? zero16 : iH[ts], 0, 0, 0);
+            /* VALU work under this MFMA: a share of the next slab's planes */
+            if (s < 7) {
+                constexpr int PER = 2 * TH / 4;           /* MFMAs per decoded dword */
+                if (k % PER == 0) decode(s + 1, k / PER);
+            }
+            if (k == 0 && s < NCOPY) copy_one(s);
+            if (k == 1 && s + 8 < NCOPY) copy_one(s + 8);
+            CKQ_PIN();
+        }
+    }
+
+#pragma unroll
+    for (int ts = 0; ts < TH; ++ts) {
+        float4 dx[4];
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) dx[r4] = *reinterpret_cast<const float4 *>(&st.d[32 * ts + 8 * r4 + 4 * half]);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const float4 d4 = dx[r >> 2];
+            const float dxr = (r & 3) == 0 ? d4.x : (r & 3) == 1 ? d4.y : (r & 3) == 2 ? d4.z : d4.w;
+            const float f = (float)((iH[ts][r] << 8) + iL[ts][r]);
+            acc[ts][r] += (dw * dxr) * f;
+        }
+    }
+#undef CKQ_PIN
+}
+
+template <int TH>
+__global__ void __launch_bounds__(256, 1) gemm_q6k_mfma_kernel(GemmArgs a)
+{
+    constexpr int BM = 32 * TH;
+    __shared__ __attribute__((aligned(16))) Gemm6Stage<TH> stage[2];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = wave_in_block();
+    const int col = lane & 31, half = lane >> 5;
+
+    /* token tiles fastest inside an XCD, so each XCD's L2 sees a weight tile once */
+    const int id = blockIdx.x, xcd = id & 7, seq = id >> 3;
+    const int tt = seq % a.ntt;
+    const int nt = (seq / a.ntt) * 8 + xcd;
+    if (nt >= a.nnt) return;
+    const int t0 = tt * BM, n0 = nt * GEMM6_BN;
+    const u32 wstride = (u32)a.nb * 210u, xstride = (u32)a.nb * 292u;
+    const int last = a.nb - 1;
+    const uint8_t *wbase = a.B + (size_t)n0 * wstride;       /* uniform */
+    const uint8_t *xbase = a.A + (size_t)t0 * xstride;       /* uniform */
+
+    /* Copy roles.  One wave instruction moves 64 x 16 bytes into 1 KiB of LDS
+     * (lane l lands at byte 16 l).  Weights: 128 rows x 14 chunks = 28
+     * instructions, seven per wave.  Quants: 4 tokens per instruction. */
+    constexpr int NWI = 7, NQI = BM / 16, NCOPY = NWI + NQI;
+    static_assert(NCOPY <= 16, "two copies per k-slab at most");
+    u32 wofs_g[NWI], qofs_g[NQI];
+#pragma unroll
+    for (int i = 0; i < NWI; ++i) {
+        const int chunk = (wave + 4 * i) * 64 + lane, row = min(chunk / 14, a.N - 1 - n0), part = chunk % 14;
+        wofs_g[i] = (u32)row * wstride + (part < 13 ? 16u * part : 194u);
+    }
+#pragma unroll
+    for (int i = 0; i < NQI; ++i) {
+        const int tl = 4 * (wave + 4 * i) + (lane >> 4), c = (lane & 15) ^ (tl & 15);
+        qofs_g[i] = (u32)min(tl, a.M - 1 - t0) * xstride + 4u + 16u * c;
+    }
+    const bool st_live = tid < BM;
+    const uint8_t *st_src = xbase + (size_t)min(tid, a.M - 1 - t0) * xstride;
+    float nd = 0.f;
+
+    const uint8_t *cp_w = wbase, *cp_x = xbase;
+    int cp_buf = 0;
+    auto copy_begin = [&](int b, int buf) {
+        nd = __builtin_bit_cast(float, ld4<4>(st_src + (u32)b * 292u));
+        cp_w = wbase + (u32)b * 210u;
+        cp_x = xbase + (u32)b * 292u;
+        cp_buf = buf;
+    };
+    auto copy_one = [&](int i) {
+        if (i < NWI)
+            __builtin_amdgcn_global_load_lds((ckq_glb_void *)(cp_w + wofs_g[i]),
+                                             (ckq_lds_void *)(stage[cp_buf].w + 1024 * (wave + 4 * i)), 16, 0, 0);
+        else
+            __builtin_amdgcn_global_load_lds((ckq_glb_void *)(cp_x + qofs_g[i - NWI]),
+                                             (ckq_lds_void *)(stage[cp_buf].q + 1024 * (wave + 4 * (i - NWI))), 16, 0, 0);
+    };
+    auto side_store = [&](int buf) { if (st_live) stage[buf].d[tid] = nd; };
+
+    /* read-side offsets of this lane */
+    const u32 wrow = (u32)(32 * wave + col) * (u32)GEMM6_ROW;
+    u32 aofs[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) aofs[s] = (u32)col * 256u + 16u * (u32)((2 * s + half) ^ (col & 15));
+
+    ckq_v16f acc[TH];
+#pragma unroll
+    for (int ts = 0; ts < TH; ++ts)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[ts][r] = 0.0f;
+
+    copy_begin(0, 0);
+#pragma unroll
+    for (int i = 0; i < NCOPY; ++i) copy_one(i);
+    side_store(0);
+    __builtin_amdgcn_s_waitcnt(0x0070);   /* vmcnt(0): this wave's copies have landed */
+    __syncthreads();
+
+    for (int b = 0; b < a.nb; ++b) {
+        const int cur = b & 1;
+        copy_begin(min(b + 1, last), cur ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+        gemm6_block<TH, NCOPY>(stage[cur], wrow, aofs, half, acc, copy_one);
+        __builtin_amdgcn_sched_barrier(0);
+        side_store(cur ^ 1);
+        __builtin_amdgcn_s_waitcnt(0x0070);
+        __syncthreads();
+    }
+
+    const int n = n0 + wave * 32 + col;
+    if (n < a.N) {
+        const float bias = a.bias ? a.bias[n] : 0.0f;
+#pragma unroll
+        for (int ts = 0; ts < TH; ++ts)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int t = t0 + 32 * ts + 8 * (r >> 2) + 4 * half + (r & 3);
+                if (t < a.M) a.C[(size_t)t * a.ldc + n] = acc[ts][r] + bias;
+            }
+    }
+}
+
+static int launch_gemm_q6k_mfma(const void *A, const void *B, const float *bias, float *C,
+                                int M, int N, int K, long ldc, hipStream_t s)
+{
+    GemmArgs g;
+    g.A = (const uint8_t *)A; g.B = (const uint8_t *)B; g.bias = bias; g.C = C;
+    g.M = M; g.N = N; g.nb = K / 256; g.ldc = ldc;
+    /* lane offsets inside a tile are 32-bit */
+    if ((long long)g.nb * 292 * 128 >= (1ll << 31)) return (int)hipErrorInvalidValue;
+    g.nnt = (N + GEMM6_BN - 1) / GEMM6_BN;
+    const int nnt8 = (g.nnt + 7) / 8 * 8;
+    /* tiles of 128 tokens where they still give every CU work, else 64 */
+    const int ntt4 = (M + 127) / 128;
+    if (ntt4 * g.nnt > 128) {
+        g.ntt = ntt4;
+        hipLaunchKernelGGL((gemm_q6k_mfma_kernel<4>), dim3(g.ntt * nnt8), dim3(256), 0, s, g);
+    } else {
+        g.ntt = (M + 63) / 64;
+        hipLaunchKernelGGL((gemm_q6k_mfma_kernel<2>), dim3(g.ntt * nnt8), dim3(256), 0, s, g);
+    }
+    return (int)hipGetLastError();
+}

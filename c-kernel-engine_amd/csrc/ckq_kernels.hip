@@ -48,6 +48,7 @@ struct GemvArgs {
 __device__ __forceinline__ int wave_in_block() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
 
 #include "ckq_gemm_mfma.cuh"
+#include "ckq_gemm_q6k_mfma.cuh"
 
 /*
  * Tiled kernel (token tiles MT >= 1, and the sub-block-dot dump).  One wave
@@ -311,6 +312,8 @@ extern "C" int ckq_launch_gemv(int fmt, float *y, const void *W, const void *X, 
         return launch_fmt<FmtQ5K>(a, dump, 8, s);
     case CKQ_FMT_Q6_K:
         if (K % 256) return CKQ_ESHAPE;
+        if (!dump && ntok > CKQ_GEMM_MIN_TOKENS && row0 == 0 && row1 == nrows)
+            return launch_gemm_q6k_mfma(X, W, bias, y, ntok, nrows, K, ldy, s);
         a.npos = K / 64; a.wrow = (long)(K / 256) * 210; a.xrow = (long)(K / 256) * 292; a.nsub_row = K / 16;
         return launch_fmt<FmtQ6K>(a, dump, 8, s);
     case CKQ_FMT_Q8_0:

@@ -517,3 +517,72 @@ def test_gemm_mfma_full_prefill_shape():
     for t in (0, 63, 64, 300, 511):
         y = P.dev_gemm_nt("q4_k", P.to_device(xq[t * ab:(t + 1) * ab].copy()), Wd, None, 1, N, K).cpu().numpy().reshape(-1)
         assert T.norm_err(c[t], y) <= 2e-6, t
+
+
+# ---- prefill GEMM on the matrix cores, Q6_K (token counts above 16) --------------------------
+
+@pytest.mark.parametrize("M,N,K", [(17, 128, 256), (33, 200, 1024), (64, 96, 512), (100, 333, 2048),
+                                   (128, 1, 256), (65, 129, 4096),
+                                   (130, 8320, 256), (512, 4224, 512)])    # the last two use 128-token tiles
+def test_gemm_mfma_q6_k_vs_oracle(M, N, K):
+    bias = T.normal(N, 0.0, 0.5, seed=N)
+    for kind in ("rand", "enc"):
+        W, _, xq = make_case("q6_k", N, K, kind, 900 + M + N, tokens=M)
+        say("gemm mfma q6_k", kind, "M", M, "N", N, "K", K)
+        ref = T.oracle_gemm_nt("q6_k", xq, W, bias, M, N, K)
+        c = P.dev_gemm_nt("q6_k", P.to_device(xq), P.to_device(W), P.to_device(bias), M, N, K).cpu().numpy()
+        assert T.norm_err(c, ref) <= TOL, (M, N, K, kind)
+        # the matrix-core path and the dot4 path agree token by token
+        ab = T.row_bytes("q8_k", K)
+        for t in (0, M - 1):
+            y = P.gemv("q6_k", W, xq[t * ab:(t + 1) * ab].copy(), N, K)
+            assert T.norm_err(c[t], y + bias) <= 2e-6
+        if N <= 512:
+            ch = P.gemm_nt("q6_k", xq, W, bias, M, N, K)      # host-pointer entry point, same kernel
+            assert np.array_equal(ch, c)
+
+
+def test_gemm_mfma_q6_k_extremes():
+    """The scaled weight sc * (q - 32) spans [-4064, 4096]; the corners of that
+    range and the extreme activations stay exact through the two int8 planes."""
+    M, N, K = 64, 64, 512
+    W, _, xq = make_case("q6_k", N, K, "rand", 977, tokens=M)
+    for ql, qh, sc in ((0x00, 0x00, -128), (0xFF, 0xFF, 127), (0x00, 0x00, 127), (0xFF, 0xFF, -128)):
+        Wb = W.copy().reshape(-1, 210)
+        Wb[:, 0:128] = ql
+        Wb[:, 128:192] = qh
+        Wb[:, 192:208] = np.uint8(sc & 0xFF)
+        Wb = Wb.reshape(-1)
+        for pattern in ("alt", "max", "min"):
+            xb = xq.copy().reshape(-1, 292)
+            q = {"alt": np.where(np.arange(256) % 2 == 0, -128, 127), "max": np.full(256, 127),
+                 "min": np.full(256, -128)}[pattern].astype(np.int8)
+            xb[:, 4:260] = q.view(np.uint8)
+            xb[:, 260:292] = q.astype(np.int16).reshape(16, 16).sum(axis=1).astype(np.int16).view(np.uint8)
+            xb = xb.reshape(-1)
+            say("gemm mfma q6_k extremes", ql, sc, pattern)
+            ref = T.oracle_gemm_nt("q6_k", xb, Wb, None, M, N, K)
+            c = P.dev_gemm_nt("q6_k", P.to_device(xb), P.to_device(Wb), None, M, N, K).cpu().numpy()
+            assert T.norm_err(c, ref) <= TOL, (ql, sc, pattern)
+
+
+def test_gemm_mfma_q6_k_down_projection_shape():
+    """M=512, N=4096, K=11008: the oracle on a sample of weight rows for every
+    token, and whole rows of C against the GEMV kernel for a few tokens."""
+    M, N, K = 512, 4096, 11008
+    W = T.synth_weights("q6_k", N, K, seed=6160)
+    xf = T.normal(M * K, 0.0, 1.0, seed=6161)
+    say("gemm mfma q6_k down projection shape")
+    xq_d = P.dev_quantize(P.to_device(xf), "q8_k", rows=M)
+    xq = xq_d.cpu().numpy()
+    Wd = P.to_device(W)
+    c = P.dev_gemm_nt("q6_k", xq_d, Wd, None, M, N, K).cpu().numpy()
+    rb = T.row_bytes("q6_k", K)
+    rows = np.array([0, 1, 31, 32, 127, 128, 2047, 2048, 4094, 4095])
+    Wsub = np.ascontiguousarray(W.reshape(N, rb)[rows]).reshape(-1)
+    ref = T.oracle_gemm_nt("q6_k", xq, Wsub, None, M, len(rows), K)
+    assert T.norm_err(c[:, rows], ref) <= TOL
+    ab = T.row_bytes("q8_k", K)
+    for t in (0, 63, 64, 300, 511):
+        y = P.dev_gemm_nt("q6_k", P.to_device(xq[t * ab:(t + 1) * ab].copy()), Wd, None, 1, N, K).cpu().numpy().reshape(-1)
+        assert T.norm_err(c[t], y) <= 2e-6, t
