@@ -69,7 +69,7 @@ __device__ __forceinline__ void gemm6_block(const Gemm6Stage<TH> &st, u32 wrow, 
         qh[n] = lds16(wr + 16 * (8 + 2 * n + half));
     }
     const ckq_v4i scv = lds16(wr + 192);
-    const float dw = h2f(*reinterpret_cast<const uint16_t *>(wr + 222));
+    const u32 dw16 = *reinterpret_cast<const uint16_t *>(wr + 222);
     const int sh0 = 8 * half, sh1 = 16 + 8 * half;   /* scale of slab s: byte 2 (s & 1) + half of dword s >> 1 */
 
     ckq_v4i av[2][TH];
@@ -77,6 +77,16 @@ __device__ __forceinline__ void gemm6_block(const Gemm6Stage<TH> &st, u32 wrow, 
 #pragma unroll
         for (int ts = 0; ts < TH; ++ts) av[s & 1][ts] = lds16(&st.q[aofs[s] + 32 * 256 * ts]);
     };
+    a_read(0);
+
+    /* token scales */
+    float4 dx[TH][4];
+#pragma unroll
+    for (int ts = 0; ts < TH; ++ts)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4)
+            dx[ts][r4] = __builtin_bit_cast(float4, lds16(reinterpret_cast<const uint8_t *>(&st.d[32 * ts + 8 * r4 + 4 * half])));
+    const float dw = h2f(dw16);
 
     u32 scp[2], cp[2];
     ckq_v4i pL[2], pH[2];
@@ -101,15 +111,13 @@ __device__ __forceinline__ void gemm6_block(const Gemm6Stage<TH> &st, u32 wrow, 
 
     ckq_v16i iL[TH], iH[TH];
     const ckq_v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-
-    a_read(0);
     prep(0);
 #pragma unroll
     for (int i = 0; i < 4; ++i) decode(0, i);
     CKQ_PIN();
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
-        if (s < 7) { a_read(s + 1); prep(s + 1); }
+        if (s < 7) prep(s + 1);
 #pragma unroll
         for (int k = 0; k < 2 * TH; ++k) {
             const int ts = k >> 1;
@@ -120,25 +128,22 @@ __device__ __forceinline__ void gemm6_block(const Gemm6Stage<TH> &st, u32 wrow, 
                 constexpr int PER = 2 * TH / 4;           /* MFMAs per decoded dword */
                 if (k % PER == 0) decode(s + 1, k / PER);
             }
-            if (k == 0 && s < NCOPY) copy_one(s);
-            if (k == 1 && s + 8 < NCOPY) copy_one(s + 8);
+            if (k == 0 && s < 7) a_read(s + 1);       /* operands of the next slab, three MFMAs ahead of their use */
+            /* copies of a later block, spread over the slabs */
+            if ((k & 1) == 0 && s + 4 * k < NCOPY) copy_one(s + 4 * k);
             CKQ_PIN();
         }
     }
 
 #pragma unroll
-    for (int ts = 0; ts < TH; ++ts) {
-        float4 dx[4];
-#pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4) dx[r4] = *reinterpret_cast<const float4 *>(&st.d[32 * ts + 8 * r4 + 4 * half]);
+    for (int ts = 0; ts < TH; ++ts)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const float4 d4 = dx[r >> 2];
+            const float4 d4 = dx[ts][r >> 2];
             const float dxr = (r & 3) == 0 ? d4.x : (r & 3) == 1 ? d4.y : (r & 3) == 2 ? d4.z : d4.w;
             const float f = (float)((iH[ts][r] << 8) + iL[ts][r]);
             acc[ts][r] += (dw * dxr) * f;
         }
-    }
 #undef CKQ_PIN
 }
 
@@ -146,7 +151,12 @@ template <int TH>
 __global__ void __launch_bounds__(256, 1) gemm_q6k_mfma_kernel(GemmArgs a)
 {
     constexpr int BM = 32 * TH;
-    __shared__ __attribute__((aligned(16))) Gemm6Stage<TH> stage[2];
+    /* Blocks are fetched NST-1 iterations ahead.  The weights stream from HBM
+     * and a fetch takes about as long as one iteration of a 64-token tile, so
+     * that tile runs three stages deep (136 KB of LDS); the 128-token tile has
+     * room for two. */
+    constexpr int NST = TH == 2 ? 3 : 2;
+    __shared__ __attribute__((aligned(16))) Gemm6Stage<TH> stage[NST];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = wave_in_block();
     const int col = lane & 31, half = lane >> 5;
@@ -165,9 +175,9 @@ __global__ void __launch_bounds__(256, 1) gemm_q6k_mfma_kernel(GemmArgs a)
     /* Copy roles.  One wave instruction moves 64 x 16 bytes into 1 KiB of LDS
      * (lane l lands at byte 16 l).  Weights: 128 rows x 14 chunks = 28
      * instructions, seven per wave.  Quants: 4 tokens per instruction. */
-    constexpr int NWI = 7, NQI = BM / 16, NCOPY = NWI + NQI;
-    static_assert(NCOPY <= 16, "two copies per k-slab at most");
-    u32 wofs_g[NWI], qofs_g[NQI];
+    constexpr int NWI = 7, NQI = BM / 16, NDI = BM / 64, NCOPY = NWI + NQI + NDI;
+    static_assert(NCOPY <= 8 * TH, "one copy per pair of MFMAs at most");
+    u32 wofs_g[NWI], qofs_g[NQI], dofs_g[NDI];
 #pragma unroll
     for (int i = 0; i < NWI; ++i) {
         const int chunk = (wave + 4 * i) * 64 + lane, row = min(chunk / 14, a.N - 1 - n0), part = chunk % 14;
@@ -178,14 +188,15 @@ __global__ void __launch_bounds__(256, 1) gemm_q6k_mfma_kernel(GemmArgs a)
         const int tl = 4 * (wave + 4 * i) + (lane >> 4), c = (lane & 15) ^ (tl & 15);
         qofs_g[i] = (u32)min(tl, a.M - 1 - t0) * xstride + 4u + 16u * c;
     }
-    const bool st_live = tid < BM;
-    const uint8_t *st_src = xbase + (size_t)min(tid, a.M - 1 - t0) * xstride;
-    float nd = 0.f;
+    /* token scales: 4-byte copies, lane l fetches the scale of token 64 i + l.
+     * Every wave issues them (same bytes to the same place), which keeps the
+     * number of outstanding copies equal in all waves. */
+#pragma unroll
+    for (int i = 0; i < NDI; ++i) dofs_g[i] = (u32)min(64 * i + lane, a.M - 1 - t0) * xstride;
 
     const uint8_t *cp_w = wbase, *cp_x = xbase;
     int cp_buf = 0;
     auto copy_begin = [&](int b, int buf) {
-        nd = __builtin_bit_cast(float, ld4<4>(st_src + (u32)b * 292u));
         cp_w = wbase + (u32)b * 210u;
         cp_x = xbase + (u32)b * 292u;
         cp_buf = buf;
@@ -194,11 +205,13 @@ __global__ void __launch_bounds__(256, 1) gemm_q6k_mfma_kernel(GemmArgs a)
         if (i < NWI)
             __builtin_amdgcn_global_load_lds((ckq_glb_void *)(cp_w + wofs_g[i]),
                                              (ckq_lds_void *)(stage[cp_buf].w + 1024 * (wave + 4 * i)), 16, 0, 0);
-        else
+        else if (i < NWI + NQI)
             __builtin_amdgcn_global_load_lds((ckq_glb_void *)(cp_x + qofs_g[i - NWI]),
                                              (ckq_lds_void *)(stage[cp_buf].q + 1024 * (wave + 4 * (i - NWI))), 16, 0, 0);
+        else
+            __builtin_amdgcn_global_load_lds((ckq_glb_void *)(cp_x + dofs_g[i - NWI - NQI]),
+                                             (ckq_lds_void *)(stage[cp_buf].d + 64 * (i - NWI - NQI)), 4, 0, 0);
     };
-    auto side_store = [&](int buf) { if (st_live) stage[buf].d[tid] = nd; };
 
     /* read-side offsets of this lane */
     const u32 wrow = (u32)(32 * wave + col) * (u32)GEMM6_ROW;
@@ -212,22 +225,31 @@ __global__ void __launch_bounds__(256, 1) gemm_q6k_mfma_kernel(GemmArgs a)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[ts][r] = 0.0f;
 
-    copy_begin(0, 0);
 #pragma unroll
-    for (int i = 0; i < NCOPY; ++i) copy_one(i);
-    side_store(0);
+    for (int p = 0; p < NST - 1; ++p) {
+        copy_begin(min(p, last), p);
+#pragma unroll
+        for (int i = 0; i < NCOPY; ++i) copy_one(i);
+    }
     __builtin_amdgcn_s_waitcnt(0x0070);   /* vmcnt(0): this wave's copies have landed */
-    __syncthreads();
+    __builtin_amdgcn_s_barrier();
 
+    /* The loop holds no other memory operation than the copies, so the wait
+     * before the barrier counts them exactly: block b+1 has landed when only
+     * the copies issued during this iteration (three stages) or none (two) are
+     * still in flight.  A bare s_barrier: the block's waves exchange data only
+     * through those copies. */
+    int cur = 0, pf = NST - 1;
     for (int b = 0; b < a.nb; ++b) {
-        const int cur = b & 1;
-        copy_begin(min(b + 1, last), cur ^ 1);
+        copy_begin(min(b + NST - 1, last), pf);
         __builtin_amdgcn_sched_barrier(0);
         gemm6_block<TH, NCOPY>(stage[cur], wrow, aofs, half, acc, copy_one);
         __builtin_amdgcn_sched_barrier(0);
-        side_store(cur ^ 1);
-        __builtin_amdgcn_s_waitcnt(0x0070);
-        __syncthreads();
+        if constexpr (NST == 3) __builtin_amdgcn_s_waitcnt(0x0070 | (NCOPY & 15) | ((NCOPY >> 4) << 14));
+        else                    __builtin_amdgcn_s_waitcnt(0x0070);
+        __builtin_amdgcn_s_barrier();
+        cur = cur + 1 == NST ? 0 : cur + 1;
+        pf = pf + 1 == NST ? 0 : pf + 1;
     }
 
     const int n = n0 + wave * 32 + col;
