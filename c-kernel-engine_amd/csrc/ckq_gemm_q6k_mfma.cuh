@@ -49,55 +49,94 @@ __device__ __forceinline__ u32 pk_mad_u16(u32 a, u32 b, u32 c)
     return __builtin_bit_cast(u32, (ckq_v2u16)(x * y + z));
 }
 
-/* One 256-block of a tile: eight k-slabs of 32, each 2*TH MFMAs (TH token
- * groups x two planes).  The planes of slab s+1 are expanded between the MFMAs
- * of slab s; copy_one(i) issues one global->LDS copy of the next block. */
-template <int TH, int NCOPY, class CopyFn>
-__device__ __forceinline__ void gemm6_block(const Gemm6Stage<TH> &st, u32 wrow, const u32 (&aofs)[8], int half,
-                                            ckq_v16f (&acc)[TH], CopyFn copy_one)
+/* What a lane reads from a stage before it can start on a block: its row's
+ * raw Q6_K block (the 16-byte runs its k-half touches) and the activation
+ * operands of the first k-slab.  Read right after the barrier that publishes
+ * the stage, ahead of the previous block's fp32 combine, which hides the LDS
+ * latency. */
+template <int TH> struct Gemm6Head {
+    ckq_v4i ql[2][2], qh[2], scv, av0[TH];
+    u32 dw16;
+};
+
+template <int TH>
+__device__ __forceinline__ void gemm6_head_read(const Gemm6Stage<TH> &st, u32 wrow, u32 aofs0, int half, Gemm6Head<TH> &h)
 {
-#define CKQ_PIN() __builtin_amdgcn_sched_barrier(0)
     auto lds16 = [&](const uint8_t *p) { return *reinterpret_cast<const ckq_v4i *>(p); };
     const uint8_t *wr = st.w + wrow;
-
-    /* raw block of this lane's row: the 16-byte runs its k-half touches */
-    ckq_v4i ql[2][2], qh[2];
 #pragma unroll
     for (int n = 0; n < 2; ++n) {
 #pragma unroll
-        for (int odd = 0; odd < 2; ++odd) ql[n][odd] = lds16(wr + 16 * (4 * n + 2 * odd + half));
-        qh[n] = lds16(wr + 16 * (8 + 2 * n + half));
+        for (int odd = 0; odd < 2; ++odd) h.ql[n][odd] = lds16(wr + 16 * (4 * n + 2 * odd + half));
+        h.qh[n] = lds16(wr + 16 * (8 + 2 * n + half));
     }
-    const ckq_v4i scv = lds16(wr + 192);
-    const u32 dw16 = *reinterpret_cast<const uint16_t *>(wr + 222);
+    h.scv = lds16(wr + 192);
+    h.dw16 = *reinterpret_cast<const uint16_t *>(wr + 222);
+#pragma unroll
+    for (int ts = 0; ts < TH; ++ts) h.av0[ts] = lds16(&st.q[aofs0 + 32 * 256 * ts]);
+}
+
+/* Integer sums of one block and the scales they are combined under. */
+template <int TH> struct Gemm6Sums {
+    ckq_v16i iL[TH], iH[TH];
+    float4   dx[TH][4];
+    float    dw;
+};
+
+template <int TH>
+__device__ __forceinline__ void gemm6_combine(const Gemm6Sums<TH> &p, ckq_v16f (&acc)[TH])
+{
+#pragma unroll
+    for (int ts = 0; ts < TH; ++ts)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const float4 d4 = p.dx[ts][r >> 2];
+            const float dxr = (r & 3) == 0 ? d4.x : (r & 3) == 1 ? d4.y : (r & 3) == 2 ? d4.z : d4.w;
+            const float f = (float)((p.iH[ts][r] << 8) + p.iL[ts][r]);
+            acc[ts][r] += (p.dw * dxr) * f;
+        }
+}
+
+/* The integer part of one 256-block of a tile: eight k-slabs of 32, each 2*TH
+ * MFMAs (TH token groups x two planes).  The planes of slab s+1 are expanded
+ * between the MFMAs of slab s; copy_one(i) issues one global->LDS copy of a
+ * later block. */
+template <int TH, int NCOPY, class CopyFn>
+__device__ __forceinline__ void gemm6_slabs(const Gemm6Stage<TH> &st, const Gemm6Head<TH> &h, const u32 (&aofs)[8], int half,
+                                            Gemm6Sums<TH> &out, CopyFn copy_one)
+{
+#define CKQ_PIN() __builtin_amdgcn_sched_barrier(0)
+    auto lds16 = [&](const uint8_t *p) { return *reinterpret_cast<const ckq_v4i *>(p); };
     const int sh0 = 8 * half, sh1 = 16 + 8 * half;   /* scale of slab s: byte 2 (s & 1) + half of dword s >> 1 */
 
     ckq_v4i av[2][TH];
+#pragma unroll
+    for (int ts = 0; ts < TH; ++ts) av[0][ts] = h.av0[ts];
     auto a_read = [&](int s) {
 #pragma unroll
         for (int ts = 0; ts < TH; ++ts) av[s & 1][ts] = lds16(&st.q[aofs[s] + 32 * 256 * ts]);
     };
-    a_read(0);
 
-    /* token scales */
-    float4 dx[TH][4];
+    /* token scales: read before the first copy is issued (an LDS read of a
+     * float after a global->LDS load would wait for the load), and through the
+     * integer vector type like every other read of a stage */
 #pragma unroll
     for (int ts = 0; ts < TH; ++ts)
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4)
-            dx[ts][r4] = __builtin_bit_cast(float4, lds16(reinterpret_cast<const uint8_t *>(&st.d[32 * ts + 8 * r4 + 4 * half])));
-    const float dw = h2f(dw16);
+            out.dx[ts][r4] = __builtin_bit_cast(float4, lds16(reinterpret_cast<const uint8_t *>(&st.d[32 * ts + 8 * r4 + 4 * half])));
+    out.dw = h2f(h.dw16);
 
     u32 scp[2], cp[2];
     ckq_v4i pL[2], pH[2];
     auto prep = [&](int s) {
-        const int sc = __builtin_amdgcn_sbfe(scv[s >> 1], (s & 1) ? sh1 : sh0, 8);
+        const int sc = __builtin_amdgcn_sbfe(h.scv[s >> 1], (s & 1) ? sh1 : sh0, 8);
         scp[s & 1] = __builtin_amdgcn_perm((u32)sc, (u32)sc, 0x05040504u);          /* sc in both 16-bit lanes */
         cp[s & 1]  = pk_mad_u16(scp[s & 1], 0xFFE0FFE0u, 0x00800080u);              /* 128 - 32 sc */
     };
     auto decode = [&](int s, int i) {
         const int n = s >> 2, g = s & 3;
-        const u32 lw = (u32)ql[n][g & 1][i], hw = (u32)qh[n][i];
+        const u32 lw = (u32)h.ql[n][g & 1][i], hw = (u32)h.qh[n][i];
         const u32 nib = g < 2 ? (lw & 0x0f0f0f0fu) : ((lw >> 4) & 0x0f0f0f0fu);
         const u32 hb = g == 0 ? (hw << 4) : g == 1 ? (hw << 2) : g == 2 ? hw : (hw >> 2);
         const u32 q = (hb & 0x30303030u) | nib;                                   /* four 6-bit values */
@@ -109,7 +148,6 @@ __device__ __forceinline__ void gemm6_block(const Gemm6Stage<TH> &st, u32 wrow, 
         pH[s & 1][i] = (int)__builtin_amdgcn_perm(to, te, 0x07030501u);
     };
 
-    ckq_v16i iL[TH], iH[TH];
     const ckq_v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     prep(0);
 #pragma unroll
@@ -121,8 +159,8 @@ __device__ __forceinline__ void gemm6_block(const Gemm6Stage<TH> &st, u32 wrow, 
 #pragma unroll
         for (int k = 0; k < 2 * TH; ++k) {
             const int ts = k >> 1;
-            if ((k & 1) == 0) iL[ts] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[s & 1][ts], pL[s & 1], s == 0 ? zero16 : iL[ts], 0, 0, 0);
-            else              iH[ts] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[s & 1][ts], pH[s & 1], s == 0 ? zero16 : iH[ts], 0, 0, 0);
+            if ((k & 1) == 0) out.iL[ts] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[s & 1][ts], pL[s & 1], s == 0 ? zero16 : out.iL[ts], 0, 0, 0);
+            else              out.iH[ts] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[s & 1][ts], pH[s & 1], s == 0 ? zero16 : out.iH[ts], 0, 0, 0);
             /* VALU work under this MFMA: a share of the next slab's planes */
             if (s < 7) {
                 constexpr int PER = 2 * TH / 4;           /* MFMAs per decoded dword */
@@ -134,16 +172,6 @@ __device__ __forceinline__ void gemm6_block(const Gemm6Stage<TH> &st, u32 wrow, 
             CKQ_PIN();
         }
     }
-
-#pragma unroll
-    for (int ts = 0; ts < TH; ++ts)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const float4 d4 = dx[ts][r >> 2];
-            const float dxr = (r & 3) == 0 ? d4.x : (r & 3) == 1 ? d4.y : (r & 3) == 2 ? d4.z : d4.w;
-            const float f = (float)((iH[ts][r] << 8) + iL[ts][r]);
-            acc[ts][r] += (dw * dxr) * f;
-        }
 #undef CKQ_PIN
 }
 
@@ -240,16 +268,32 @@ __global__ void __launch_bounds__(256, 1) gemm_q6k_mfma_kernel(GemmArgs a)
      * still in flight.  A bare s_barrier: the block's waves exchange data only
      * through those copies. */
     int cur = 0, pf = NST - 1;
+    Gemm6Head<TH> head;
+    gemm6_head_read<TH>(stage[0], wrow, aofs[0], half, head);
     for (int b = 0; b < a.nb; ++b) {
         copy_begin(min(b + NST - 1, last), pf);
         __builtin_amdgcn_sched_barrier(0);
-        gemm6_block<TH, NCOPY>(stage[cur], wrow, aofs, half, acc, copy_one);
+        Gemm6Sums<TH> sums;
+        gemm6_slabs<TH, NCOPY>(stage[cur], head, aofs, half, sums, copy_one);
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (NST == 3) __builtin_amdgcn_s_waitcnt(0x0070 | (NCOPY & 15) | ((NCOPY >> 4) << 14));
         else                    __builtin_amdgcn_s_waitcnt(0x0070);
         __builtin_amdgcn_s_barrier();
         cur = cur + 1 == NST ? 0 : cur + 1;
         pf = pf + 1 == NST ? 0 : pf + 1;
+        /* The next block's first reads, then this block's fp32 combine under
+         * them (after the last block the stage holds that block again: unused).
+         * The 128-token tile has no registers to spare for that overlap. */
+        if constexpr (TH == 2) {
+            gemm6_head_read<TH>(stage[cur], wrow, aofs[0], half, head);
+            __builtin_amdgcn_sched_barrier(0);
+            gemm6_combine<TH>(sums, acc);
+        } else {
+            gemm6_combine<TH>(sums, acc);
+            __builtin_amdgcn_sched_barrier(0);
+            gemm6_head_read<TH>(stage[cur], wrow, aofs[0], half, head);
+        }
+        __builtin_amdgcn_sched_barrier(0);
     }
 
     const int n = n0 + wave * 32 + col;
