@@ -270,6 +270,18 @@ def main():
         extras["gemm_q4_k_q8_k_M512"] = {"tops": round(ops / sg / 1e12, 2), "ms": round(sg * 1e3, 4),
                                          "frac_int8_peak": round(ops / sg / 1e12 / INT8_PEAK_TOPS, 4),
                                          "ops_per_call": ops, "kernel": "two-plane int8 MFMA (v_mfma_i32_32x32x32_i8) + bf16 MFMA min term"}
+        # the same prefill step for the down projection of a Q4_K_M model: Q6_K weights, K = 11008
+        r6, k6 = 4096, 11008
+        _, cps6 = H.weight_copies("q6_k", r6, k6, seed=66, min_total=1)
+        x6 = P.dev_quantize(P.to_device(T.normal(Mg * k6, seed=67)), "q8_k", rows=Mg)
+        s6, _ = H.time_gemv("q6_k", r6, k6, Mg, cps6[:2] if len(cps6) > 1 else cps6, x6, steps_g, 2)
+        ops6 = 2.0 * Mg * r6 * k6
+        extras["gemm_q6_k_q8_k_M512_4096x11008"] = {"tops": round(ops6 / s6 / 1e12, 2), "ms": round(s6 * 1e3, 4),
+                                                    "frac_int8_peak": round(ops6 / s6 / 1e12 / INT8_PEAK_TOPS, 4),
+                                                    "ops_per_call": ops6,
+                                                    "kernel": "two-plane int8 MFMA on sc*(q-32) split by byte, three LDS stages"}
+        del cps6, x6
+        torch.cuda.empty_cache()
         for name, fmt, r, k in (("gemv_q4_k_4096x4096", "q4_k", 4096, 4096),
                                 ("lm_head_q6_k_32000x4096", "q6_k", 32000, 4096),
                                 ("down_q6_k_4096x11008", "q6_k", 4096, 11008),
