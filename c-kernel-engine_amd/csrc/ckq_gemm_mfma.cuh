@@ -145,7 +145,9 @@ __device__ __forceinline__ void gemm_block_pipe(const GemmStage &st, u32 wofs, c
     };
     auto load_dx = [&](int ts) {
 #pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4) dx[r4] = *reinterpret_cast<const float4 *>(&st.d[32 * ts + 8 * r4 + 4 * half]);
+        for (int r4 = 0; r4 < 4; ++r4)   /* through the integer vector type: an LDS read of a float after a
+                                          * global->LDS load makes the compiler wait for that load */
+            dx[r4] = __builtin_bit_cast(float4, lds16(reinterpret_cast<const uint8_t *>(&st.d[32 * ts + 8 * r4 + 4 * half])));
     };
     auto min_mfma = [&](int ts) {
         ckq_v16f zero;
