@@ -72,6 +72,8 @@ _SIGS = {
     "embedding_forward_q6_k": (None, [_vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i]),
     "embedding_forward_q8_0": (None, [_vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i]),
     "rmsnorm_q8_k_fused": (None, [_vp, _vp, _vp, _i, _i, _i, _c.c_float]),
+    "fused_mlp_swiglu_prefill_w1w2_quant": (None, [_vp, _vp, _vp, _i, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp]),
+    "fused_mlp_swiglu_prefill_w1w2_quant_scratch_size": (_c.c_size_t, [_i, _i]),
     "gemv_q4_k": (None, [_vp, _vp, _vp, _i, _i]),
     "gemm_q4_k": (None, [_vp, _vp, _vp, _i, _i, _i]),
     "gemm_nt_q4_k": (None, [_vp, _vp, _vp, _vp, _i, _i, _i]),
@@ -108,6 +110,7 @@ _SIGS = {
     "ckq_gemm_nt_q8_0_q8_0_dev": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "ckq_dequant_rows_dev": (_i, [_i, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp]),
     "ckq_rmsnorm_q8_k_fused_dev": (_i, [_vp, _vp, _vp, _i, _i, _i, _c.c_float, _vp]),
+    "ckq_swiglu_q8_k_dev": (_i, [_vp, _vp, _vp, _i, _i, _c.c_long, _vp]),
     "ckq_gemm_nt_f32act_dev": (_i, [_i, _vp, _vp, _vp, _vp, _i, _i, _i, _c.c_long, _vp]),
     "ckq_matmul_sequence_dev": (_i, [_vp, _i, _i, _vp]),
     "ckq_subblock_dots_dev": (_i, [_i, _vp, _vp, _vp, _i, _i, _vp]),
@@ -121,6 +124,7 @@ _SIGS = {
     "ckq_weights_set_cache": (None, [_i]),
     "ckq_set_parallel_whole": (None, [_i]),
     "ckq_last_error": (_i, []),
+    "ckq_clear_error": (None, []),
     "ckq_error_string": (_c.c_char_p, [_i]),
 }
 
@@ -141,7 +145,7 @@ def declared_symbols():
     text = open(HEADER).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     text = re.sub(r"typedef\s+struct\s*\{.*?\}\s*\w+;", "", text, flags=re.S)
-    names = re.findall(r"^\s*(?:const\s+)?(?:void|int|char|float)\s*\*?\s*(\w+)\s*\(", text, flags=re.M)
+    names = re.findall(r"^\s*(?:const\s+)?(?:void|int|char|float|size_t)\s*\*?\s*(\w+)\s*\(", text, flags=re.M)
     return sorted(set(names))
 
 

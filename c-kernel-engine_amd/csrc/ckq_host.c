@@ -44,7 +44,7 @@ typedef struct {
     size_t cap;
 } dev_buf;
 
-enum { BUF_X = 0, BUF_Y, BUF_BIAS, BUF_Q, BUF_COUNT };
+enum { BUF_X = 0, BUF_Y, BUF_BIAS, BUF_Q, BUF_GU, BUF_H, BUF_COUNT };
 
 static pthread_mutex_t g_mu = PTHREAD_MUTEX_INITIALIZER;
 static int          g_inited = 0;
@@ -72,6 +72,7 @@ const char *ckq_error_string(int code)
 }
 
 int ckq_last_error(void) { return g_err; }
+void ckq_clear_error(void) { g_err = 0; }
 
 static int fail(int code, const char *what)
 {
@@ -680,6 +681,98 @@ void rmsnorm_q8_k_fused(const float *input, const float *gamma, void *vy, int to
     pthread_mutex_unlock(&g_mu);
 }
 
+/* Fused prefill MLP: Q8_0 quantization, one GEMM over the stacked gate and up
+ * rows, SiLU(gate)*up quantized to Q8_K, the down GEMM.  The four kernels run
+ * back to back on the library's stream; intermediates never leave the device. */
+void fused_mlp_swiglu_prefill_w1w2_quant(const float *x, const void *W1, const float *B1, int w1_dt,
+                                         const void *W2, const float *B2, int w2_dt, float *output,
+                                         int seq_len, int embed_dim, int aligned_embed_dim,
+                                         int intermediate_dim, int aligned_intermediate_dim, void *scratch)
+{
+    if (!x || !W1 || !W2 || !output || !scratch) return;
+    if (seq_len <= 0 || embed_dim <= 0 || aligned_embed_dim <= 0 || intermediate_dim <= 0 ||
+        aligned_intermediate_dim <= 0)
+        return;
+    if (aligned_embed_dim < embed_dim || aligned_intermediate_dim < intermediate_dim) return;
+    if (aligned_embed_dim % 32 || aligned_intermediate_dim % 256) return;
+    if ((w1_dt != CKQ_CK_DT_Q8_0 && w1_dt != CKQ_CK_DT_Q5_0) || (w2_dt != CKQ_CK_DT_Q4_K && w2_dt != CKQ_CK_DT_Q6_K))
+        return;
+    if (w1_dt == CKQ_CK_DT_Q5_0) {
+        pthread_mutex_lock(&g_mu);
+        fail(CKQ_EFORMAT, "fused_mlp_swiglu_prefill_w1w2_quant: Q5_0 weights are not built");
+        pthread_mutex_unlock(&g_mu);
+        return;
+    }
+    const int E = aligned_embed_dim, I = aligned_intermediate_dim;
+    const int fmt2 = w2_dt == CKQ_CK_DT_Q4_K ? CKQ_FMT_Q4_K : CKQ_FMT_Q6_K;
+    const size_t out_bytes = (size_t)seq_len * E * 4;
+    pthread_mutex_lock(&g_mu);
+    do {
+        if (init_locked()) break;
+        const void *dx, *dW1, *dW2, *dB1 = NULL, *dB2 = NULL;
+        void *dq, *dgu, *dh;
+        if (stage_in(BUF_X, x, (size_t)seq_len * E * 4, &dx)) break;
+        if (weights_resolve(W1, (size_t)2 * I * weight_row_bytes(CKQ_FMT_Q8_0, E), &dW1)) break;
+        if (weights_resolve(W2, (size_t)E * weight_row_bytes(fmt2, I), &dW2)) break;
+        /* both biases share the bias staging buffer: B1 first, B2 behind it */
+        if (B1 || B2) {
+            const int b1_dev = B1 && is_device_ptr(B1), b2_dev = B2 && is_device_ptr(B2);
+            void *db = NULL;
+            if (((B1 && !b1_dev) || (B2 && !b2_dev)) && buf_reserve(BUF_BIAS, ((size_t)2 * I + E) * 4, &db)) break;
+            hipError_t e = hipSuccess;
+            if (B1) {
+                dB1 = B1;
+                if (!b1_dev) { e = hipMemcpyAsync(db, B1, (size_t)2 * I * 4, hipMemcpyHostToDevice, g_stream); dB1 = db; }
+            }
+            if (e == hipSuccess && B2) {
+                dB2 = B2;
+                if (!b2_dev) {
+                    e = hipMemcpyAsync((float *)db + 2 * (size_t)I, B2, (size_t)E * 4, hipMemcpyHostToDevice, g_stream);
+                    dB2 = (float *)db + 2 * (size_t)I;
+                }
+            }
+            if (e != hipSuccess) { fail((int)e, "copy biases to device"); break; }
+        }
+        if (buf_reserve(BUF_Q, (size_t)seq_len * act_row_bytes(CKQ_FMT_Q8_0, E), &dq)) break;
+        if (buf_reserve(BUF_GU, (size_t)seq_len * 2 * I * 4, &dgu)) break;
+        if (buf_reserve(BUF_H, (size_t)seq_len * act_row_bytes(fmt2, I), &dh)) break;
+        const int out_on_dev = is_device_ptr(output);
+        void *dout = output;
+        if (!out_on_dev && buf_reserve(BUF_Y, out_bytes, &dout)) break;
+        int rc = ckq_launch_quantize_q8_0((const float *)dx, dq, seq_len, E, g_stream);
+        if (rc) { fail(rc, "quantize launch"); break; }
+        rc = ckq_launch_gemv(CKQ_FMT_Q8_0, (float *)dgu, dW1, dq, (const float *)dB1, 2 * I, E, seq_len, 2L * I, 0, 2 * I,
+                             NULL, g_stream);
+        if (rc) { fail(rc, "gate/up GEMM launch"); break; }
+        rc = ckq_launch_swiglu_q8_k((const float *)dgu, (const float *)dgu + I, dh, seq_len, I, 2L * I, g_stream);
+        if (rc) { fail(rc, "swiglu launch"); break; }
+        rc = ckq_launch_gemv(fmt2, (float *)dout, dW2, dh, (const float *)dB2, E, I, seq_len, (long)E, 0, E, NULL, g_stream);
+        if (rc) { fail(rc, "down GEMM launch"); break; }
+        if (!out_on_dev) {
+            hipError_t e = hipMemcpyAsync(output, dout, out_bytes, hipMemcpyDeviceToHost, g_stream);
+            if (e != hipSuccess) { fail((int)e, "copy result to host"); break; }
+        }
+        hipError_t e = hipStreamSynchronize(g_stream);
+        if (e != hipSuccess) fail((int)e, "hipStreamSynchronize");
+    } while (0);
+    pthread_mutex_unlock(&g_mu);
+}
+
+/* What the reference asks its callers to provide (tiles of 64 tokens: Q8_0
+ * rows, gate and up tiles, Q8_K rows, each rounded up to 64 bytes), so code that
+ * sizes its arena with this call allocates the same amount. */
+size_t fused_mlp_swiglu_prefill_w1w2_quant_scratch_size(int aligned_embed_dim, int aligned_intermediate_dim)
+{
+    if (aligned_embed_dim <= 0 || aligned_intermediate_dim <= 0) return 0;
+    const size_t tile = 64;
+    const size_t q8 = tile * ((size_t)aligned_embed_dim / 32) * 34;
+    const size_t gate = tile * (size_t)aligned_intermediate_dim * 4;
+    const size_t q8k = tile * ((size_t)aligned_intermediate_dim / 256) * 292;
+#define CKQ_UP64(v) (((v) + 63) / 64 * 64)
+    return CKQ_UP64(q8) + 2 * CKQ_UP64(gate) + CKQ_UP64(q8k);
+#undef CKQ_UP64
+}
+
 /* fp32 activations used as they are (no activation quantization). */
 void gemv_q4_k(float *y, const void *W, const float *x, int M, int K)
 {
@@ -828,6 +921,11 @@ int ckq_rmsnorm_q8_k_fused_dev(const float *input, const float *gamma, void *y, 
                                int aligned_embed_dim, float eps, void *stream)
 {
     return ckq_launch_rmsnorm_q8_k_fused(input, gamma, y, tokens, d_model, aligned_embed_dim, eps, stream);
+}
+
+int ckq_swiglu_q8_k_dev(const float *gate, const float *up, void *y, int rows, int k, long ld, void *stream)
+{
+    return ckq_launch_swiglu_q8_k(gate, up, y, rows, k, ld, stream);
 }
 
 int ckq_gemm_nt_f32act_dev(int fmt, const float *A, const void *B, const float *bias, float *C,

@@ -6,7 +6,7 @@
  *                           small-batch prefill); weights are streamed once
  *                           with 128-bit loads, unpacked in registers, dotted
  *                           with v_dot4_i32_i8, reduced with DPP.
- *   quantize_q8_k_kernel    fp32 -> Q8_K, bit-exact with the reference
+ *   quantize_q8_k_kernel    fp32 -> Q8_K, bit-exact with the reference; also SiLU(gate)*up -> Q8_K
  *   quantize_q8_0_kernel    fp32 -> Q8_0, bit-exact with the reference
  *   rmsnorm_q8_k_fused_kernel  RMSNorm -> Q8_K in one pass, bit-exact with the reference's FMA build
  *   dequant_rows_kernel     row dequantizers / quantized embedding lookup, bit-exact
@@ -359,14 +359,35 @@ __device__ __forceinline__ int rne_sat_i8(float p)
  * with IEEE division; each product is rounded to fp32 and then to the nearest
  * even integer; d = 1/iscale.
  */
-__global__ void __launch_bounds__(256) quantize_q8_k_kernel(const float *__restrict__ x, uint8_t *__restrict__ y,
-                                                            long nblocks)
+/* SiLU(g) * u as the reference's fused prefill MLP forms it
+ * (fused/prefill_fused_gemm.c:904-906, 1034-1040): g / (1 + expf(-g)), then
+ * the product, each operation rounded to fp32.  exp is evaluated in double
+ * and rounded once, which agrees with a correctly rounded expf. */
+__device__ __forceinline__ float swiglu_value(float g, float u)
+{
+#pragma clang fp contract(off)
+    const float e = (float)exp(-(double)g);
+    const float s = g / (1.0f + e);
+    return s * u;
+}
+
+/* SWIGLU: the quantizer's input is SiLU(x) * up instead of x.  Rows of the
+ * input are ldx floats apart, bpr blocks of 256 per row. */
+template <bool SWIGLU>
+__global__ void __launch_bounds__(256) quantize_q8_k_kernel(const float *__restrict__ x, const float *__restrict__ up,
+                                                            uint8_t *__restrict__ y, long nblocks, int bpr, long ldx)
 {
     const int lane = threadIdx.x & 63;
     const long blk = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (blk >= nblocks) return;
-    const float4 v = reinterpret_cast<const float4 *>(x + blk * 256)[lane];
-    const float e[4] = {v.x, v.y, v.z, v.w};
+    const long src = (blk / bpr) * ldx + (blk % bpr) * 256;
+    const float4 v = reinterpret_cast<const float4 *>(x + src)[lane];
+    float e[4] = {v.x, v.y, v.z, v.w};
+    if constexpr (SWIGLU) {
+        const float4 w = reinterpret_cast<const float4 *>(up + src)[lane];
+        e[0] = swiglu_value(e[0], w.x); e[1] = swiglu_value(e[1], w.y);
+        e[2] = swiglu_value(e[2], w.z); e[3] = swiglu_value(e[3], w.w);
+    }
 
     /* first-largest |x| inside the lane, then across lanes (lower index wins ties) */
     float amax = 0.0f, smax = 0.0f;
@@ -440,8 +461,19 @@ extern "C" int ckq_launch_quantize_q8_k(const float *x, void *y, int rows, int k
     if (!x || !y || rows <= 0 || k <= 0) return CKQ_EINVAL;
     if (k % 256) return CKQ_ESHAPE;
     const long nblocks = (long)rows * (k / 256);
-    hipLaunchKernelGGL(quantize_q8_k_kernel, dim3((unsigned)((nblocks + 3) / 4)), dim3(256), 0, (hipStream_t)stream,
-                       x, (uint8_t *)y, nblocks);
+    hipLaunchKernelGGL(quantize_q8_k_kernel<false>, dim3((unsigned)((nblocks + 3) / 4)), dim3(256), 0, (hipStream_t)stream,
+                       x, (const float *)nullptr, (uint8_t *)y, nblocks, k / 256, (long)k);
+    return (int)hipGetLastError();
+}
+
+/* y[row] = Q8_K(SiLU(gate[row]) * up[row]), rows of gate and up ld floats apart. */
+extern "C" int ckq_launch_swiglu_q8_k(const float *gate, const float *up, void *y, int rows, int k, long ld, void *stream)
+{
+    if (!gate || !up || !y || rows <= 0 || k <= 0 || ld < k) return CKQ_EINVAL;
+    if (k % 256 || ld % 4 || ((uintptr_t)gate | (uintptr_t)up) % 16) return CKQ_ESHAPE;
+    const long nblocks = (long)rows * (k / 256);
+    hipLaunchKernelGGL(quantize_q8_k_kernel<true>, dim3((unsigned)((nblocks + 3) / 4)), dim3(256), 0, (hipStream_t)stream,
+                       gate, up, (uint8_t *)y, nblocks, k / 256, ld);
     return (int)hipGetLastError();
 }
 

@@ -42,6 +42,9 @@ int ckq_launch_gemv(int fmt, float *y, const void *W, const void *X, const float
 int ckq_launch_quantize_q8_k(const float *x, void *y, int rows, int k, void *stream);
 int ckq_launch_quantize_q8_0(const float *x, void *y, int rows, int k, void *stream);
 
+/* y[row] = Q8_K(SiLU(gate[row]) * up[row]), k floats per row, rows ld floats apart. */
+int ckq_launch_swiglu_q8_k(const float *gate, const float *up, void *y, int rows, int k, long ld, void *stream);
+
 /* RMSNorm over d_model floats per token (row stride aligned_embed_dim floats),
  * times gamma, quantized to Q8_K blocks: tokens x (d_model/256) blocks. */
 int ckq_launch_rmsnorm_q8_k_fused(const float *input, const float *gamma, void *y, int tokens, int d_model,

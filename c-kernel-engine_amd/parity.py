@@ -83,6 +83,20 @@ def rmsnorm_q8_k_fused(x, gamma, tokens, d_model, aligned=None, eps=1e-6):
     return out
 
 
+CK_DT = {"q4_k": 7, "q6_k": 8, "q8_0": 9, "q8_k": 10, "q5_0": 11}   # the reference's CKDataType values
+
+
+def fused_mlp_swiglu_prefill_w1w2_quant(x, W1, B1, w1_fmt, W2, B2, w2_fmt, seq_len, embed, aligned_embed,
+                                        inter, aligned_inter, output=None, scratch=True):
+    """Mirror of the reference symbol; returns the [seq_len, aligned_embed] output
+    (or the untouched `output` passed in when the call rejects its arguments)."""
+    out = output if output is not None else np.zeros(seq_len * aligned_embed, dtype=np.float32)
+    scr = np.zeros(16, dtype=np.uint8) if scratch else None
+    lib().fused_mlp_swiglu_prefill_w1w2_quant(_p(x), _p(W1), _p(B1), CK_DT[w1_fmt], _p(W2), _p(B2), CK_DT[w2_fmt],
+                                              _p(out), seq_len, embed, aligned_embed, inter, aligned_inter, _p(scr))
+    return out.reshape(seq_len, aligned_embed) if out.size == seq_len * aligned_embed else out
+
+
 def gemv_f32act(fmt, W, x_f32, M, K):
     """gemv_q4_k / gemv_q6_k / gemv_q8_0: fp32 activations, nothing quantized."""
     y = np.zeros(M, dtype=np.float32)
@@ -158,6 +172,13 @@ def dev_rmsnorm_q8_k_fused(x_t, gamma_t, tokens, d_model, aligned=None, eps=1e-6
     out = torch.zeros(tokens * row_bytes("q8_k", d_model), dtype=torch.uint8, device=x_t.device)
     check(lib().ckq_rmsnorm_q8_k_fused_dev(_dp(x_t), _dp(gamma_t), _dp(out), tokens, d_model, aligned,
                                            ctypes.c_float(eps), _stream()), "ckq_rmsnorm_q8_k_fused_dev")
+    return out
+
+
+def dev_swiglu_q8_k(gate_t, up_t, rows, k, ld):
+    import torch
+    out = torch.zeros(rows * row_bytes("q8_k", k), dtype=torch.uint8, device=gate_t.device)
+    check(lib().ckq_swiglu_q8_k_dev(_dp(gate_t), _dp(up_t), _dp(out), rows, k, ld, _stream()), "ckq_swiglu_q8_k_dev")
     return out
 
 

@@ -134,6 +134,34 @@ void embedding_forward_q8_0(const int32_t *token_ids, int token_count, int vocab
 void rmsnorm_q8_k_fused(const float *input, const float *gamma, void *vy, int tokens, int d_model,
                         int aligned_embed_dim, float eps);
 
+/* Fused prefill MLP around the quantized GEMMs: x (seq_len rows of
+ * aligned_embed_dim floats) is quantized to Q8_0, multiplied with W1 = [gate
+ * rows; up rows] (2 * aligned_intermediate_dim rows, bias B1 of the same length
+ * or NULL), SiLU(gate) * up is quantized to Q8_K and multiplied with W2
+ * (aligned_embed_dim rows, bias B2 or NULL) into output (seq_len rows of
+ * aligned_embed_dim floats).  w1_dt / w2_dt are the reference's CKDataType
+ * values (include/ckernel_dtype.h:27-50): W1 CKQ_CK_DT_Q8_0, W2 CKQ_CK_DT_Q4_K
+ * or CKQ_CK_DT_Q6_K.  The reference also accepts Q5_0 for W1; that format is
+ * not built here and the request fails like any other the library cannot
+ * serve: the process aborts, or with CKQ_ABORT_ON_ERROR=0 the call returns
+ * without touching output and ckq_last_error() reports CKQ_EFORMAT.  Other
+ * argument errors return without touching output, as the reference does.  `scratch` must be non-NULL as in
+ * the reference but is not used: intermediates stay in device memory.  Any mix
+ * of host and device pointers; synchronous.  The SiLU uses an exponential
+ * rounded once from double, so the Q8_K intermediate can differ from a glibc
+ * host's by one unit in rare quants; the output agrees within the fp32
+ * tolerance of the GEMMs.
+ * Replaces src/kernels/fused/prefill_fused_gemm.c:964-1060 and :1062-1080. */
+#define CKQ_CK_DT_Q4_K 7
+#define CKQ_CK_DT_Q6_K 8
+#define CKQ_CK_DT_Q8_0 9
+#define CKQ_CK_DT_Q5_0 11
+void fused_mlp_swiglu_prefill_w1w2_quant(const float *x, const void *W1, const float *B1, int w1_dt,
+                                         const void *W2, const float *B2, int w2_dt, float *output,
+                                         int seq_len, int embed_dim, int aligned_embed_dim,
+                                         int intermediate_dim, int aligned_intermediate_dim, void *scratch);
+size_t fused_mlp_swiglu_prefill_w1w2_quant_scratch_size(int aligned_embed_dim, int aligned_intermediate_dim);
+
 /* Parity-test wrappers: fp32 input is quantized, then the kernel runs.
  * Replace src/ck_parity_api.c:207-210 (quantize), :217-258 (gemv q4_k/q6_k),
  * :288-360 (gemv q8_0), :397-400 (vec_dot), :411-503 (gemm) and the size
@@ -193,6 +221,11 @@ int ckq_dequant_rows_dev(int fmt, const void *table, const int32_t *ids, int voc
 int ckq_rmsnorm_q8_k_fused_dev(const float *input, const float *gamma, void *y, int tokens, int d_model,
                                int aligned_embed_dim, float eps, void *stream);
 
+/* y[row] = Q8_K(SiLU(gate[row]) * up[row]): the step between the two GEMMs of
+ * the fused prefill MLP.  k floats per row (multiple of 256), rows of gate and
+ * of up ld floats apart, both 16-byte aligned. */
+int ckq_swiglu_q8_k_dev(const float *gate, const float *up, void *y, int rows, int k, long ld, void *stream);
+
 /* fp32 activations (M rows of K floats, 16-byte aligned) against `fmt` weights
  * (CKQ_FMT_Q4_K, _Q6_K or _Q8_0), no activation quantization: the device form
  * of gemv_q4_k / gemm_nt_q4_k / gemm_nt_q6_k / gemm_nt_q8_0 above. */
@@ -248,8 +281,10 @@ void ckq_weights_set_cache(int enabled);
 /* Thread-split entry points: 0 (default) = every call computes its own row
  * range; 1 = the ith==0 call computes all rows and the others return. */
 void ckq_set_parallel_whole(int enabled);
-/* Last error of the calling process (0 = none) and its text. */
+/* Last error of the calling process (0 = none), its text, and a reset for
+ * callers that run with CKQ_ABORT_ON_ERROR=0 and handle errors themselves. */
 int         ckq_last_error(void);
+void        ckq_clear_error(void);
 const char *ckq_error_string(int code);
 
 #ifdef __cplusplus

@@ -1009,3 +1009,70 @@ void orc_gemm_nt_q8_0(const float *A, const void *B, const float *bias, float *C
     for (int m = 0; m < M; ++m) orc_gemv_q8_0(C + (size_t)m * N, B, A + (size_t)m * K, N, K);
     add_bias(C, bias, M, N);
 }
+
+
+/* ------------------------------------------------------------------------ */
+/* Fused prefill MLP                                                         */
+/* ------------------------------------------------------------------------ */
+
+/* fused/prefill_fused_gemm.c:904-906 */
+static float silu_prefill(float x) { return x / (1.0f + expf(-x)); }
+
+/* The SwiGLU step and its quantization (fused/prefill_fused_gemm.c:1034-1047):
+ * g = silu(g) * u element by element, then quantize_row_q8_k of each row. */
+void orc_swiglu_q8_k(const float *gate, const float *up, void *y, int rows, int k, long ld)
+{
+    if (!gate || !up || !y || rows <= 0 || k <= 0 || k % 256) return;
+    float *row = (float *)malloc((size_t)k * sizeof(float));
+    if (!row) return;
+    const size_t rb = (size_t)(k / 256) * sizeof(ckq_block_q8_K);
+    for (int i = 0; i < rows; ++i) {
+        const float *g = gate + (size_t)i * (size_t)ld, *u = up + (size_t)i * (size_t)ld;
+        for (int j = 0; j < k; ++j) row[j] = silu_prefill(g[j]) * u[j];
+        orc_quantize_row_q8_k(row, (uint8_t *)y + (size_t)i * rb, k);
+    }
+    free(row);
+}
+
+/* fused/prefill_fused_gemm.c:964-1060.  The reference walks the sequence in
+ * tiles of 64 tokens; every step is row-wise, so the tiling does not change
+ * any value and is not restated. */
+void orc_fused_mlp_swiglu_prefill_w1w2_quant(const float *x, const void *W1, const float *B1, int w1_dt,
+                                             const void *W2, const float *B2, int w2_dt, float *output,
+                                             int seq_len, int embed_dim, int aligned_embed_dim,
+                                             int intermediate_dim, int aligned_intermediate_dim,
+                                             float *gate_up_out, void *h_q8k_out)
+{
+    enum { DT_Q4_K = 7, DT_Q6_K = 8, DT_Q8_0 = 9 };
+    if (!x || !W1 || !W2 || !output) return;
+    if (seq_len <= 0 || embed_dim <= 0 || aligned_embed_dim <= 0 || intermediate_dim <= 0 ||
+        aligned_intermediate_dim <= 0)
+        return;
+    if (aligned_embed_dim < embed_dim || aligned_intermediate_dim < intermediate_dim) return;
+    if ((aligned_embed_dim % 32) != 0 || (aligned_intermediate_dim % 256) != 0) return;
+    if (w1_dt != DT_Q8_0 || (w2_dt != DT_Q4_K && w2_dt != DT_Q6_K)) return;
+
+    const int E = aligned_embed_dim, I = aligned_intermediate_dim;
+    const size_t q8_row = (size_t)(E / 32) * sizeof(ckq_block_q8_0);
+    const size_t q8k_row = (size_t)(I / 256) * sizeof(ckq_block_q8_K);
+    uint8_t *xq = (uint8_t *)malloc((size_t)seq_len * q8_row);
+    float *gate = (float *)malloc((size_t)seq_len * I * sizeof(float));
+    float *up = (float *)malloc((size_t)seq_len * I * sizeof(float));
+    uint8_t *hq = (uint8_t *)malloc((size_t)seq_len * q8k_row);
+    if (xq && gate && up && hq) {
+        for (int t = 0; t < seq_len; ++t) orc_quantize_row_q8_0(x + (size_t)t * E, xq + (size_t)t * q8_row, E);
+        const uint8_t *w_gate = (const uint8_t *)W1, *w_up = w_gate + (size_t)I * q8_row;
+        orc_gemm_nt_q8_0_q8_0(xq, w_gate, B1, gate, seq_len, I, E);
+        orc_gemm_nt_q8_0_q8_0(xq, w_up, B1 ? B1 + I : NULL, up, seq_len, I, E);
+        orc_swiglu_q8_k(gate, up, hq, seq_len, I, I);
+        if (gate_up_out)
+            for (int t = 0; t < seq_len; ++t) {
+                for (int j = 0; j < I; ++j) gate_up_out[(size_t)t * 2 * I + j] = silu_prefill(gate[(size_t)t * I + j]) * up[(size_t)t * I + j];
+                memcpy(gate_up_out + (size_t)t * 2 * I + I, up + (size_t)t * I, (size_t)I * sizeof(float));
+            }
+        if (h_q8k_out) memcpy(h_q8k_out, hq, (size_t)seq_len * q8k_row);
+        if (w2_dt == DT_Q4_K) orc_gemm_nt_q4_k_q8_k(hq, W2, B2, output, seq_len, E, I);
+        else                  orc_gemm_nt_q6_k_q8_k(hq, W2, B2, output, seq_len, E, I);
+    }
+    free(xq); free(gate); free(up); free(hq);
+}

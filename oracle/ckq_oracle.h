@@ -88,6 +88,21 @@ void orc_gemm_q6_k(float *Y, const void *W, const float *X, int M, int N, int K)
 void orc_gemm_nt_q6_k(const float *A, const void *B, const float *bias, float *C, int M, int N, int K);            /* gemm_kernels_q6k.c:212-240 */
 void orc_gemm_nt_q8_0(const float *A, const void *B, const float *bias, float *C, int M, int N, int K);            /* gemm_kernels_q8_0.c:683-696 */
 
+/* ---- fused prefill MLP ----------------------------------------------------
+ * fused/prefill_fused_gemm.c:964-1060: Q8_0(x) x W1 (gate rows then up rows),
+ * SiLU(gate)*up with the C library's expf, Q8_K of that, x W2.  w1_dt / w2_dt
+ * are the reference's CKDataType values (Q8_0 = 9; Q4_K = 7, Q6_K = 8); other
+ * types return without writing.  gate_up_out (seq_len x 2*aligned_intermediate
+ * floats: gate, already multiplied, then up) and h_q8k_out receive the
+ * intermediates when non-NULL.                                              */
+void orc_fused_mlp_swiglu_prefill_w1w2_quant(const float *x, const void *W1, const float *B1, int w1_dt,
+                                             const void *W2, const float *B2, int w2_dt, float *output,
+                                             int seq_len, int embed_dim, int aligned_embed_dim,
+                                             int intermediate_dim, int aligned_intermediate_dim,
+                                             float *gate_up_out, void *h_q8k_out);
+/* Q8_K of SiLU(gate)*up, rows ld floats apart (fused/prefill_fused_gemm.c:904-906,1034-1047). */
+void orc_swiglu_q8_k(const float *gate, const float *up, void *y, int rows, int k, long ld);
+
 /* ---- exact evaluation ---------------------------------------------------
  * Same integers, block scales combined in double: the value every fp32
  * summation order approximates.  fmt is a ckq_format weight tag; the

@@ -20,6 +20,8 @@ vp = ctypes.c_void_p
 
 
 def ptr(a):
+    if a is None:
+        return None
     assert a.flags["C_CONTIGUOUS"]
     return a.ctypes.data_as(vp)
 
@@ -130,6 +132,20 @@ def oracle_gemm_nt_f32act(fmt, A_f32, B, bias, M, N, K):
     c = np.zeros(M * N, dtype=np.float32)
     getattr(oracle(), "orc_gemm_nt_" + fmt)(ptr(A_f32), ptr(B), ptr(bias) if bias is not None else None, ptr(c), M, N, K)
     return c.reshape(M, N)
+
+
+CK_DT = {"q4_k": 7, "q6_k": 8, "q8_0": 9, "q8_k": 10, "q5_0": 11}   # the reference's CKDataType values
+
+
+def oracle_fused_mlp(x, W1, B1, W2, B2, w2_fmt, seq, embed, aembed, inter, ainter, want_intermediates=False):
+    out = np.zeros(seq * aembed, dtype=np.float32)
+    gu = np.zeros(seq * 2 * ainter, dtype=np.float32) if want_intermediates else None
+    hq = np.zeros(seq * row_bytes("q8_k", ainter), dtype=np.uint8) if want_intermediates else None
+    oracle().orc_fused_mlp_swiglu_prefill_w1w2_quant(ptr(x), ptr(W1), ptr(B1), CK_DT["q8_0"], ptr(W2), ptr(B2),
+                                                     CK_DT[w2_fmt], ptr(out), seq, embed, aembed, inter, ainter,
+                                                     ptr(gu), ptr(hq))
+    out = out.reshape(seq, aembed)
+    return (out, gu.reshape(seq, 2 * ainter), hq) if want_intermediates else out
 
 
 def oracle_exact(fmt, W, xq, M, K):

@@ -263,6 +263,32 @@ def main():
                                                                ED, AED, CTX, add_pos)
             G["emb_out_%s_pos%d" % (fmt, add_pos)] = o
 
+    # ---- fused prefill MLP (Q8_0 gate/up, Q4_K or Q6_K down) -------------------------
+    # 70 tokens: the reference walks tiles of 64, so the second tile is ragged
+    SEQ, ED2, AED2, ID2, AID2 = 70, 60, 64, 250, 256
+    xm = normal(S, SEQ * AED2, 0.0, 1.0, 801)
+    w1 = synth_weights(S, "q8_0", 2 * AID2, AED2, 802)
+    # synth weights are N(0, 0.02): scale the block scales up so gate values spread over the SiLU's knee
+    w1v = w1.reshape(-1, 34)
+    d16 = w1v[:, 0:2].copy().view(np.float16).astype(np.float32) * 12.0
+    w1v[:, 0:2] = d16.astype(np.float16).view(np.uint8)
+    b1 = normal(S, 2 * AID2, 0.0, 0.3, 803)
+    b2 = normal(S, AED2, 0.0, 0.3, 804)
+    G["mlp_x"], G["mlp_w1"], G["mlp_b1"], G["mlp_b2"] = xm, w1, b1, b2
+    G["mlp_shape"] = np.array([SEQ, ED2, AED2, ID2, AID2], np.int32)
+    DT = {"q4_k": 7, "q6_k": 8, "q8_0": 9}
+    for fmt in ("q4_k", "q6_k"):
+        w2 = synth_weights(S, fmt, AED2, AID2, 805 + FMT[fmt])
+        G["mlp_w2_" + fmt] = w2
+        for tag, L in libs.items():
+            L.fused_mlp_swiglu_prefill_w1w2_quant_scratch_size.restype = ctypes.c_size_t
+            scr = np.zeros(L.fused_mlp_swiglu_prefill_w1w2_quant_scratch_size(AED2, AID2), np.uint8)
+            o = np.zeros(SEQ * AED2, np.float32)
+            L.fused_mlp_swiglu_prefill_w1w2_quant(ptr(xm), ptr(w1), ptr(b1), DT["q8_0"], ptr(w2), ptr(b2), DT[fmt],
+                                                  ptr(o), SEQ, ED2, AED2, ID2, AID2, ptr(scr))
+            G["mlp_out_%s_%s" % (fmt, tag)] = o
+        G["mlp_scratch_size"] = np.array([len(scr)], np.int64)
+
     np.savez_compressed(OUT, **G)
     print("wrote %s: %d arrays, %.1f KiB" % (OUT, len(G), os.path.getsize(OUT) / 1024.0))
 

@@ -366,6 +366,48 @@ def test_embedding_forward_bit_exact_vs_reference(fmt, add_pos):
     assert np.all(o[NTOK:] == 0.0)
 
 
+# ---- fused prefill MLP ----------------------------------------------------------------------
+
+@pytest.mark.parametrize("fmt", ["q4_k", "q6_k"])
+def test_fused_mlp_swiglu_prefill_vs_reference(fmt):
+    """The compiled reference (70 tokens: one full tile of 64 and a ragged one)
+    against the restatement, and the restatement's stages against what they must
+    mean: SiLU(gate)*up in float64, Q8_K of it, the down GEMM of that."""
+    G = T.golden()
+    SEQ, ED, AED, ID, AID = (int(v) for v in G["mlp_shape"])
+    x, w1, b1, b2, w2 = G["mlp_x"], G["mlp_w1"], G["mlp_b1"], G["mlp_b2"], G["mlp_w2_" + fmt]
+    out, gu, hq = T.oracle_fused_mlp(x, w1, b1, w2, b2, fmt, SEQ, ED, AED, ID, AID, want_intermediates=True)
+    for tag in ("avx2", "avx512"):
+        want = G["mlp_out_%s_%s" % (fmt, tag)].reshape(SEQ, AED)
+        assert T.norm_err(out, want) <= 2e-6, tag
+    # stage 1: gate and up are the Q8_0 GEMM of the quantized input (already pinned on its own)
+    xq = T.oracle_quantize(x, "q8_0", rows=SEQ)
+    c = T.oracle_gemm_nt("q8_0", xq, w1, b1, SEQ, 2 * AID, AED)
+    up = gu[:, AID:]
+    assert np.array_equal(up.view(np.uint32), c[:, AID:].view(np.uint32))
+    # stage 2: the activation, against float64
+    g64 = c[:, :AID].astype(np.float64)
+    want_h = g64 / (1.0 + np.exp(-g64)) * up.astype(np.float64)
+    assert np.all(np.abs(gu[:, :AID] - want_h) <= 4e-7 * np.abs(want_h) + 1e-30)
+    # stage 3: Q8_K of exactly those floats
+    assert np.array_equal(hq, T.oracle_quantize(np.ascontiguousarray(gu[:, :AID]).reshape(-1), "q8_k", rows=SEQ))
+    # stage 4: the down GEMM of exactly those blocks
+    assert np.array_equal(out.view(np.uint32), T.oracle_gemm_nt(fmt, hq, w2, b2, SEQ, AED, AID).view(np.uint32))
+
+
+def test_fused_mlp_rejects_what_the_reference_rejects():
+    G = T.golden()
+    SEQ, ED, AED, ID, AID = (int(v) for v in G["mlp_shape"])
+    O = T.oracle()
+    x, w1, w2 = G["mlp_x"], G["mlp_w1"], G["mlp_w2_q4_k"]
+    for bad in (dict(w1=T.CK_DT["q4_k"]), dict(w2=T.CK_DT["q8_0"]), dict(aed=AED + 8), dict(aid=AID + 32), dict(seq=0)):
+        out = np.full(SEQ * AED, 7.0, np.float32)
+        O.orc_fused_mlp_swiglu_prefill_w1w2_quant(ptr(x), ptr(w1), None, bad.get("w1", T.CK_DT["q8_0"]), ptr(w2), None,
+                                                  bad.get("w2", T.CK_DT["q4_k"]), ptr(out), bad.get("seq", SEQ), ED,
+                                                  bad.get("aed", AED), ID, bad.get("aid", AID), None, None)
+        assert np.all(out == 7.0), bad
+
+
 # ---- exact evaluation: dequantize-then-fp64 matmul ---------------------------------
 
 @pytest.mark.parametrize("fmt", ["q4_k", "q5_k", "q6_k", "q8_0"])
