@@ -28,7 +28,7 @@ __device__ __forceinline__ int wave_in_block();
 /* GEMV                                                                       */
 /* ========================================================================= */
 
-/* Token counts above this use the MFMA GEMM (Q4_K); at or below it the
+/* Token counts above this use the MFMA GEMMs (Q4_K, Q6_K, Q8_0); at or below it the
  * weight-streaming dot4 kernel with 8-token tiles reads the weights once or
  * twice and is faster. */
 #define CKQ_GEMM_MIN_TOKENS 16
@@ -49,6 +49,7 @@ __device__ __forceinline__ int wave_in_block() { return __builtin_amdgcn_readfir
 
 #include "ckq_gemm_mfma.cuh"
 #include "ckq_gemm_q6k_mfma.cuh"
+#include "ckq_gemm_q80_mfma.cuh"
 
 /*
  * Tiled kernel (token tiles MT >= 1, and the sub-block-dot dump).  One wave
@@ -318,6 +319,8 @@ extern "C" int ckq_launch_gemv(int fmt, float *y, const void *W, const void *X, 
         return launch_fmt<FmtQ6K>(a, dump, 8, s);
     case CKQ_FMT_Q8_0:
         if (K % 32) return CKQ_ESHAPE;
+        if (!dump && ntok > CKQ_GEMM_MIN_TOKENS && row0 == 0 && row1 == nrows)
+            return launch_gemm_q80_mfma(X, W, bias, y, ntok, nrows, K, ldy, s);
         a.npos = K / 32; a.wrow = (long)(K / 32) * 34; a.xrow = (long)(K / 32) * 34; a.nsub_row = K / 32;
         return launch_fmt<FmtQ80>(a, dump, 8, s);
     case CKQ_KERNEL_Q80_F32:

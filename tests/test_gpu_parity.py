@@ -724,3 +724,51 @@ def test_fused_mlp_argument_errors_leave_output_untouched():
         else:
             os.environ["CKQ_ABORT_ON_ERROR"] = old
     assert int(ckq.lib().fused_mlp_swiglu_prefill_w1w2_quant_scratch_size(AED, AID)) == int(G["mlp_scratch_size"][0])
+
+
+# ---- prefill GEMM on the matrix cores, Q8_0 (token counts above 16) --------------------------
+
+@pytest.mark.parametrize("M,N,K", [(17, 128, 128), (33, 200, 96), (64, 96, 160), (100, 333, 896), (128, 1, 32),
+                                   (65, 129, 4096), (130, 1030, 64), (512, 512, 416)])
+def test_gemm_mfma_q8_0_vs_oracle(M, N, K):
+    bias = T.normal(N, 0.0, 0.5, seed=N)
+    for kind in ("rand", "enc"):
+        W, _, xq = make_case("q8_0", N, K, kind, 1100 + M + N, tokens=M)
+        say("gemm mfma q8_0", kind, "M", M, "N", N, "K", K)
+        ref = T.oracle_gemm_nt("q8_0", xq, W, bias, M, N, K)
+        c = P.dev_gemm_nt("q8_0", P.to_device(xq), P.to_device(W), P.to_device(bias), M, N, K).cpu().numpy()
+        assert T.norm_err(c, ref) <= TOL, (M, N, K, kind)
+        # the matrix-core path and the dot4 path agree token by token
+        ab = T.row_bytes("q8_0", K)
+        for t in (0, M - 1):
+            y = P.gemv("q8_0", W, xq[t * ab:(t + 1) * ab].copy(), N, K)
+            assert T.norm_err(c[t], y + bias) <= 2e-6
+        if N <= 512:
+            ch = P.gemm_nt("q8_0", xq, W, None, M, N, K)      # host-pointer entry point, same kernel, no bias
+            assert T.norm_err(ch, ref - bias) <= TOL
+            ldc = N + 3                                        # unaligned row pitch: scalar stores
+            cd = P.to_device(np.full(M * ldc, 5.0, np.float32))
+            xq_d, W_d = P.to_device(xq), P.to_device(W)        # kept alive across the call
+            P.check(ckq.lib().ckq_gemm_nt_dev(P.FMT["q8_0"], P._dp(xq_d), P._dp(W_d), None, P._dp(cd),
+                                              M, N, K, ldc, P._stream()), "ckq_gemm_nt_dev")
+            cdn = cd.cpu().numpy().reshape(M, ldc)
+            assert np.array_equal(cdn[:, :N], ch) and np.all(cdn[:, N:] == 5.0)
+
+
+def test_gemm_mfma_q8_0_extremes():
+    """All quants at -128 / 127 on both sides and the largest finite fp16 scales
+    that keep the result finite: the int32 block sums are exact."""
+    M, N, K = 64, 64, 256
+    W, _, xq = make_case("q8_0", N, K, "rand", 1177, tokens=M)
+    for wq, xqv in ((127, 127), (-128, -128), (-128, 127)):
+        Wb = W.copy().reshape(-1, 34)
+        Wb[:, 2:] = np.uint8(wq & 0xFF)
+        Wb[:, 0:2] = np.array([1.5], np.float16).view(np.uint8)
+        xb = xq.copy().reshape(-1, 34)
+        xb[:, 2:] = np.uint8(xqv & 0xFF)
+        xb[:, 0:2] = np.array([0.75], np.float16).view(np.uint8)
+        say("gemm mfma q8_0 extremes", wq, xqv)
+        ref = T.oracle_gemm_nt("q8_0", xb.reshape(-1), Wb.reshape(-1), None, M, N, K)
+        c = P.dev_gemm_nt("q8_0", P.to_device(xb.reshape(-1)), P.to_device(Wb.reshape(-1)), None, M, N, K).cpu().numpy()
+        assert np.array_equal(c, ref)        # every term is exact in fp32 here
+        assert c[0, 0] == np.float32(1.5 * 0.75 * wq * xqv * 32 * (K // 32))
