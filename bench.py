@@ -282,6 +282,38 @@ def main():
                                                     "kernel": "two-plane int8 MFMA on sc*(q-32) split by byte, three LDS stages"}
         del cps6, x6
         torch.cuda.empty_cache()
+        # and for a Q8_0 model's gate/up projection (small model: K = 896) and a 7B-sized one
+        for name8, r8, k8 in (("gemm_q8_0_q8_0_M512_9728x896", 9728, 896), ("gemm_q8_0_q8_0_M512_11008x4096", 11008, 4096)):
+            _, cps8 = H.weight_copies("q8_0", r8, k8, seed=88, min_total=1)
+            x8 = P.dev_quantize(P.to_device(T.normal(Mg * k8, seed=89)), "q8_0", rows=Mg)
+            s8, _ = H.time_gemv("q8_0", r8, k8, Mg, cps8[:2], x8, steps_g, 2)
+            ops8 = 2.0 * Mg * r8 * k8
+            extras[name8] = {"tops": round(ops8 / s8 / 1e12, 2), "ms": round(s8 * 1e3, 4),
+                             "frac_int8_peak": round(ops8 / s8 / 1e12 / INT8_PEAK_TOPS, 4), "ops_per_call": ops8,
+                             "kernel": "one int8 MFMA per 32-block, fp16 scale products on the VALU"}
+            del cps8, x8
+            torch.cuda.empty_cache()
+        # the fused prefill MLP of a small model (E = 896, I = 4864): Q8_0 gate/up, Q4_K down, device pointers
+        Em, Im = 896, 4864
+        xm = P.to_device(T.normal(Mg * Em, seed=90))
+        w1m = P.to_device(T.synth_weights("q8_0", 2 * Im, Em, seed=91, std=0.25))
+        w2m = P.to_device(T.synth_weights("q4_k", Em, Im, seed=92))
+        outm = torch.empty(Mg * Em, dtype=torch.float32, device="cuda")
+        scr = torch.zeros(16, dtype=torch.uint8, device="cuda")
+        def mlp():
+            H.L.fused_mlp_swiglu_prefill_w1w2_quant(P._dp(xm), P._dp(w1m), None, P.CK_DT["q8_0"], P._dp(w2m), None,
+                                                    P.CK_DT["q4_k"], P._dp(outm), Mg, Em, Em, Im, Im, P._dp(scr))
+        mlp(); mlp()
+        import time as _t
+        t0 = _t.perf_counter()
+        for _ in range(10):
+            mlp()                                   # synchronous entry point
+        tm = (_t.perf_counter() - t0) / 10
+        opsm = 2.0 * Mg * (2 * Im * Em + Em * Im)
+        extras["fused_mlp_prefill_M512_E896_I4864"] = {"ms": round(tm * 1e3, 4), "tops": round(opsm / tm / 1e12, 2),
+                                                       "note": "synchronous call: four kernels and a stream sync"}
+        del xm, w1m, w2m, outm
+        torch.cuda.empty_cache()
         for name, fmt, r, k in (("gemv_q4_k_4096x4096", "q4_k", 4096, 4096),
                                 ("lm_head_q6_k_32000x4096", "q6_k", 32000, 4096),
                                 ("down_q6_k_4096x11008", "q6_k", 4096, 11008),
