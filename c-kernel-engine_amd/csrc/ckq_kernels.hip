@@ -28,7 +28,7 @@ __device__ __forceinline__ int wave_in_block();
 /* GEMV                                                                       */
 /* ========================================================================= */
 
-/* Token counts above this use the MFMA GEMMs (Q4_K, Q6_K, Q8_0); at or below it the
+/* Token counts above this use the MFMA GEMMs; at or below it the
  * weight-streaming dot4 kernel with 8-token tiles reads the weights once or
  * twice and is faster. */
 #define CKQ_GEMM_MIN_TOKENS 16
@@ -50,6 +50,7 @@ __device__ __forceinline__ int wave_in_block() { return __builtin_amdgcn_readfir
 #include "ckq_gemm_mfma.cuh"
 #include "ckq_gemm_q6k_mfma.cuh"
 #include "ckq_gemm_q80_mfma.cuh"
+#include "ckq_gemm_q5k_mfma.cuh"
 
 /*
  * Tiled kernel (token tiles MT >= 1, and the sub-block-dot dump).  One wave
@@ -309,6 +310,10 @@ extern "C" int ckq_launch_gemv(int fmt, float *y, const void *W, const void *X, 
         return launch_fmt<FmtQ4K>(a, dump, 8, s);
     case CKQ_FMT_Q5_K:
         if (K % 256) return CKQ_ESHAPE;
+        /* the min term and the 16-bit scale products make this kernel's fixed
+         * cost per block higher: the token tiles stay ahead up to 64 tokens */
+        if (!dump && ntok > 4 * CKQ_GEMM_MIN_TOKENS && row0 == 0 && row1 == nrows)
+            return launch_gemm_q5k_mfma(X, W, bias, y, ntok, nrows, K, ldy, s);
         a.npos = K / 64; a.wrow = (long)(K / 256) * 176; a.xrow = (long)(K / 256) * 292; a.nsub_row = K / 32;
         return launch_fmt<FmtQ5K>(a, dump, 8, s);
     case CKQ_FMT_Q6_K:

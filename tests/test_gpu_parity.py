@@ -772,3 +772,55 @@ def test_gemm_mfma_q8_0_extremes():
         c = P.dev_gemm_nt("q8_0", P.to_device(xb.reshape(-1)), P.to_device(Wb.reshape(-1)), None, M, N, K).cpu().numpy()
         assert np.array_equal(c, ref)        # every term is exact in fp32 here
         assert c[0, 0] == np.float32(1.5 * 0.75 * wq * xqv * 32 * (K // 32))
+
+
+# ---- prefill GEMM on the matrix cores, Q5_K (token counts above 16) --------------------------
+
+@pytest.mark.parametrize("M,N,K", [(65, 128, 256), (70, 200, 1024), (66, 96, 512), (100, 333, 2048),
+                                   (128, 1, 256), (97, 129, 4864), (512, 896, 1024)])
+def test_gemm_mfma_q5_k_vs_oracle(M, N, K):
+    bias = T.normal(N, 0.0, 0.5, seed=N)
+    for kind in ("rand", "enc"):
+        W, _, xq = make_case("q5_k", N, K, kind, 1300 + M + N, tokens=M)
+        say("gemm mfma q5_k", kind, "M", M, "N", N, "K", K)
+        ref = T.oracle_gemm_nt("q5_k", xq, W, bias, M, N, K)
+        c = P.dev_gemm_nt("q5_k", P.to_device(xq), P.to_device(W), P.to_device(bias), M, N, K).cpu().numpy()
+        assert T.norm_err(c, ref) <= TOL, (M, N, K, kind)
+        # the matrix-core path and the dot4 path agree token by token
+        ab = T.row_bytes("q8_k", K)
+        for t in (0, M - 1):
+            y = P.gemv("q5_k", W, xq[t * ab:(t + 1) * ab].copy(), N, K)
+            assert T.norm_err(c[t], y + bias) <= 2e-6
+        if N <= 512:
+            ch = P.gemm_nt("q5_k", xq, W, bias, M, N, K)      # host-pointer entry point, same kernel
+            assert np.array_equal(ch, c)
+
+
+def test_gemm_mfma_q5_k_stored_bsums_and_extremes():
+    """Stored bsums are consumed (zeroed bsums drop the min term), and the
+    extreme values (5-bit value 31, scale and min 63, q8 = -128 / 127, bsums at
+    both ends of their range) stay exact through the byte-split operands."""
+    M, N, K = 96, 64, 512
+    W, _, xq = make_case("q5_k", N, K, "rand", 1311, tokens=M)
+    xz = xq.copy().reshape(-1, 292)
+    xz[:, 260:292] = 0
+    xz = xz.reshape(-1)
+    say("gemm mfma q5_k zeroed bsums")
+    ref = T.oracle_gemm_nt("q5_k", xz, W, None, M, N, K)
+    c = P.dev_gemm_nt("q5_k", P.to_device(xz), P.to_device(W), None, M, N, K).cpu().numpy()
+    assert T.norm_err(c, ref) <= TOL
+    Wb = W.copy().reshape(-1, 176)
+    Wb[:, 4:16] = 0xFF          # all scales and mins 63
+    Wb[:, 16:] = 0xFF           # all fifth bits and nibbles set: every value 31
+    Wb = Wb.reshape(-1)
+    for pattern in ("alt", "max", "min"):
+        xb = xq.copy().reshape(-1, 292)
+        q = {"alt": np.where(np.arange(256) % 2 == 0, -128, 127), "max": np.full(256, 127),
+             "min": np.full(256, -128)}[pattern].astype(np.int8)
+        xb[:, 4:260] = q.view(np.uint8)
+        xb[:, 260:292] = q.astype(np.int16).reshape(16, 16).sum(axis=1).astype(np.int16).view(np.uint8)
+        xb = xb.reshape(-1)
+        say("gemm mfma q5_k extremes", pattern)
+        ref = T.oracle_gemm_nt("q5_k", xb, Wb, None, M, N, K)
+        c = P.dev_gemm_nt("q5_k", P.to_device(xb), P.to_device(Wb), None, M, N, K).cpu().numpy()
+        assert T.norm_err(c, ref) <= TOL, pattern
