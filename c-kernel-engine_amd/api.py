@@ -119,6 +119,8 @@ _SIGS = {
     "ckq_init": (_i, []),
     "ckq_synchronize": (_i, []),
     "ckq_weights_register": (_i, [_vp, _c.c_size_t]),
+    "ckq_weights_register_manifest": (_i, [_vp, _c.c_char_p]),
+    "ckq_weights_resident": (_i, [_vp]),
     "ckq_weights_invalidate": (None, [_vp]),
     "ckq_weights_clear": (None, []),
     "ckq_weights_set_cache": (None, [_i]),

@@ -37,6 +37,7 @@ typedef struct {
     size_t      bytes;
     uint64_t    fp;
     void       *dev;
+    int         pinned;   /* registered by the caller: serves any sub-range, content is not re-checked */
 } weight_entry;
 
 typedef struct {
@@ -213,6 +214,14 @@ static int weights_lookup(const void *W, size_t bytes, const void **out)
         *out = W;
         return 0;
     }
+    /* registered regions first: any range inside one is resident as it stands */
+    for (size_t i = 0; i < g_nw; ++i) {
+        const uint8_t *h = (const uint8_t *)g_w[i].host, *w = (const uint8_t *)W;
+        if (g_w[i].pinned && w >= h && w + bytes <= h + g_w[i].bytes) {
+            *out = (const uint8_t *)g_w[i].dev + (w - h);
+            return 0;
+        }
+    }
     const uint64_t fp = fingerprint(W, bytes);
     for (size_t i = 0; i < g_nw; ++i) {
         if (g_w[i].host == W && g_w[i].bytes == bytes) {
@@ -241,6 +250,7 @@ static int weights_lookup(const void *W, size_t bytes, const void **out)
     g_w[g_nw].bytes = bytes;
     g_w[g_nw].fp = fp;
     g_w[g_nw].dev = d;
+    g_w[g_nw].pinned = 0;
     g_nw++;
     *out = d;
     return 0;
@@ -276,19 +286,88 @@ static int weights_resolve(const void *W, size_t bytes, const void **out)
     return weights_lookup(W, bytes, out);
 }
 
+static int register_locked(const void *W, size_t bytes)
+{
+    const void *d;
+    int rc = weights_lookup(W, bytes, &d);
+    if (rc) return rc;
+    for (size_t i = 0; i < g_nw; ++i)
+        if (g_w[i].host == W && g_w[i].bytes == bytes) g_w[i].pinned = 1;
+    return 0;
+}
+
 int ckq_weights_register(const void *W, size_t bytes)
 {
     if (!W || bytes == 0) return CKQ_EINVAL;
+    if (is_device_ptr(W)) return 0;
     pthread_mutex_lock(&g_mu);
     int rc = init_locked();
-    const void *d;
-    if (rc == 0) rc = weights_lookup(W, bytes, &d);
+    if (rc == 0) rc = register_locked(W, bytes);
     if (rc == 0) {
         hipError_t e = hipStreamSynchronize(g_stream);
         if (e != hipSuccess) rc = fail((int)e, "hipStreamSynchronize");
     }
     pthread_mutex_unlock(&g_mu);
     return rc;
+}
+
+/* Loader hook: walk a weights manifest (one tensor per line,
+ * name|dtype|file_offset|size|runtime_offset, '#' comments and blank lines
+ * skipped, numbers in any C base) and register every tensor of a quantized
+ * weight format this library computes with, at base + runtime_offset. */
+int ckq_weights_register_manifest(const void *base, const char *manifest_path)
+{
+    if (!base || !manifest_path) return CKQ_EINVAL;
+    FILE *mf = fopen(manifest_path, "r");
+    if (!mf) return CKQ_EINVAL;
+    static const char *const quant[] = {"q4_k", "q4k", "q5_k", "q5k", "q6_k", "q6k", "q8_0"};
+    char line[4096];
+    int n = 0, rc = 0, inited = 0;
+    while (rc == 0 && fgets(line, sizeof line, mf)) {
+        char *p = line;
+        while (*p == ' ' || *p == '\t') ++p;
+        if (*p == '#' || *p == '\n' || *p == '\r' || *p == 0) continue;
+        char *f[5];
+        int nf = 0;
+        for (char *q = p; nf < 5; ++nf) {
+            f[nf] = q;
+            char *bar = strchr(q, '|');
+            if (!bar) { ++nf; break; }
+            *bar = 0;
+            q = bar + 1;
+        }
+        if (nf < 5) { rc = CKQ_EINVAL; break; }        /* malformed line */
+        int is_quant = 0;
+        for (size_t i = 0; i < sizeof quant / sizeof quant[0]; ++i) is_quant |= strcmp(f[1], quant[i]) == 0;
+        if (!is_quant) continue;
+        const unsigned long long size = strtoull(f[3], NULL, 0), off = strtoull(f[4], NULL, 0);
+        if (size == 0) continue;
+        pthread_mutex_lock(&g_mu);
+        if (!inited) { rc = init_locked(); inited = 1; }
+        if (rc == 0) rc = register_locked((const uint8_t *)base + off, (size_t)size);
+        pthread_mutex_unlock(&g_mu);
+        if (rc == 0) ++n;
+    }
+    fclose(mf);
+    if (rc == 0 && inited) {
+        pthread_mutex_lock(&g_mu);
+        hipError_t e = hipStreamSynchronize(g_stream);
+        if (e != hipSuccess) rc = fail((int)e, "hipStreamSynchronize");
+        pthread_mutex_unlock(&g_mu);
+    }
+    return rc ? rc : n;
+}
+
+/* Number of resident weight regions; their total size through *bytes. */
+int ckq_weights_resident(size_t *bytes)
+{
+    pthread_mutex_lock(&g_mu);
+    size_t b = 0;
+    for (size_t i = 0; i < g_nw; ++i) b += g_w[i].bytes;
+    const int n = (int)g_nw;
+    pthread_mutex_unlock(&g_mu);
+    if (bytes) *bytes = b;
+    return n;
 }
 
 static void drop_entry(size_t i)

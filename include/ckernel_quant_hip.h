@@ -272,9 +272,22 @@ int ckq_init(void);
 /* Wait for all work the host-pointer entry points enqueued. */
 int ckq_synchronize(void);
 /* Weight residency: host weight matrices are uploaded on first use and cached
- * by (address, bytes, fingerprint).  register = upload now; invalidate = drop
- * one; clear = drop all; set_cache(0) = upload on every call. */
+ * by (address, bytes, fingerprint).  invalidate = drop the region starting at W;
+ * clear = drop all; set_cache(0) = upload on every call.
+ * register = upload now and pin: a registered region serves every later call
+ * whose weights lie anywhere inside it (a whole weight arena can be registered
+ * once) and its content is not re-checked until it is invalidated.
+ * register_manifest is the loader hook: it reads the weights manifest the
+ * reference's loader reads (one tensor per line,
+ * name|dtype|file_offset|size|runtime_offset; version/v7/src/
+ * ckernel_model_load_v7.c:17-35, 330-377) and registers every q4_k / q5_k /
+ * q6_k / q8_0 tensor at base + runtime_offset, base being the arena
+ * ck_load_weights filled.  Returns the number of tensors registered or a
+ * negative CKQ_E* code (unreadable file, malformed line).
+ * resident = number of resident regions, total size through *bytes. */
 int  ckq_weights_register(const void *W, size_t bytes);
+int  ckq_weights_register_manifest(const void *base, const char *manifest_path);
+int  ckq_weights_resident(size_t *bytes);
 void ckq_weights_invalidate(const void *W);
 void ckq_weights_clear(void);
 void ckq_weights_set_cache(int enabled);

@@ -84,6 +84,27 @@ def test_dev_entry_points_reject_bad_shapes(L):
     assert b"multiple" in L.ckq_error_string(-2)
 
 
+def test_manifest_hook_parses_without_touching_a_device(L, tmp_path):
+    """The loader hook reads the reference's manifest format; tensors of other
+    dtypes are skipped, so a manifest without quantized weights needs no device;
+    unreadable files and malformed lines are reported as argument errors."""
+    base = np.zeros(64, np.uint8)
+    p = lambda a: a.ctypes.data_as(ctypes.c_void_p)
+    m = tmp_path / "weights_manifest.map"
+    m.write_text("# name|dtype|file_offset|size|runtime_offset\n\n"
+                 "model.norm.weight|fp32|8|3584|0\n"
+                 "model.rope.cache|f16|0x1000|128|4096\n")
+    assert L.ckq_weights_register_manifest(p(base), str(m).encode()) == 0
+    assert L.ckq_weights_register_manifest(p(base), str(tmp_path / "missing.map").encode()) == -1
+    assert L.ckq_weights_register_manifest(None, str(m).encode()) == -1
+    bad = tmp_path / "bad.map"
+    bad.write_text("model.norm.weight|fp32|8|3584\n")
+    assert L.ckq_weights_register_manifest(p(base), str(bad).encode()) == -1
+    assert L.ckq_last_error() == 0
+    nbytes = ctypes.c_size_t(7)
+    assert L.ckq_weights_resident(ctypes.byref(nbytes)) == 0 and nbytes.value == 0
+
+
 def test_no_device_fails_loudly():
     """Without a GPU a compute call must not succeed silently: the library
     reports the HIP error and aborts the process."""

@@ -824,3 +824,49 @@ def test_gemm_mfma_q5_k_stored_bsums_and_extremes():
         ref = T.oracle_gemm_nt("q5_k", xb, Wb, None, M, N, K)
         c = P.dev_gemm_nt("q5_k", P.to_device(xb), P.to_device(Wb), None, M, N, K).cpu().numpy()
         assert T.norm_err(c, ref) <= TOL, pattern
+
+
+# ---- loader hook: registered weight regions ---------------------------------------------------
+
+def test_weights_register_manifest_and_ranges(tmp_path):
+    """A weight arena laid out by a manifest (as the reference's loader fills it):
+    the hook uploads the quantized tensors once; calls with host pointers into
+    the arena - whole tensors, row ranges of them, the gate or up half of a
+    stacked matrix - are served from those regions without new uploads."""
+    L = ckq.lib()
+    L.ckq_weights_clear()
+    N, K = 48, 512
+    wa = T.synth_weights("q4_k", N, K, seed=9101)
+    wb = T.synth_weights("q6_k", N, K, seed=9102)
+    arena = np.zeros(4096 + len(wa) + 64 + len(wb) + 512, np.uint8)
+    oa, ob = 4096, 4096 + len(wa) + 64
+    arena[oa:oa + len(wa)] = wa
+    arena[ob:ob + len(wb)] = wb
+    arena[:4096].view(np.float32)[:] = 1.0                       # an fp32 tensor the hook must skip
+    m = tmp_path / "weights_manifest.map"
+    m.write_text("# name|dtype|file_offset|size|runtime_offset\n"
+                 "model.norm.weight|fp32|8|4096|0\n"
+                 "model.layers.0.wq|q4_k|4104|%d|%d\n"
+                 "model.layers.0.wdown|q6k|0x%x|%d|%d\n" % (len(wa), oa, 4104 + len(wa), len(wb), ob))
+    say("ckq_weights_register_manifest")
+    assert L.ckq_weights_register_manifest(T.ptr(arena), str(m).encode()) == 2
+    nbytes = ctypes.c_size_t(0)
+    assert L.ckq_weights_resident(ctypes.byref(nbytes)) == 2 and nbytes.value == len(wa) + len(wb)
+    xq = T.oracle_quantize(T.normal(K, seed=9103), "q8_k")
+    ya = P.gemv("q4_k", arena[oa:oa + len(wa)], xq, N, K)          # views: host pointers into the arena
+    yb = P.gemv("q6_k", arena[ob:ob + len(wb)], xq, N, K)
+    assert T.norm_err(ya, T.oracle_gemv("q4_k", wa, xq, N, K)) <= TOL
+    assert T.norm_err(yb, T.oracle_gemv("q6_k", wb, xq, N, K)) <= TOL
+    rb = T.row_bytes("q4_k", K)
+    ysub = P.gemv("q4_k", arena[oa + 8 * rb:oa + 40 * rb], xq, 32, K)   # rows 8..39 of the first tensor
+    assert np.array_equal(ysub, ya[8:40])
+    assert L.ckq_weights_resident(None) == 2                       # nothing new was uploaded
+    # a registered region is not re-checked: new content needs invalidate
+    arena[oa:oa + len(wa)] = T.synth_weights("q4_k", N, K, seed=9104)
+    assert np.array_equal(P.gemv("q4_k", arena[oa:oa + len(wa)], xq, N, K), ya)
+    L.ckq_weights_invalidate(T.ptr(arena[oa:]))
+    assert L.ckq_weights_resident(None) == 1
+    y2 = P.gemv("q4_k", arena[oa:oa + len(wa)], xq, N, K)
+    assert T.norm_err(y2, T.oracle_gemv("q4_k", arena[oa:oa + len(wa)].copy(), xq, N, K)) <= TOL
+    L.ckq_weights_clear()
+    assert L.ckq_weights_resident(None) == 0
