@@ -56,7 +56,97 @@ struct GemmArgs {
     int  M, N, nb;
     long ldc;
     int  ntt, nnt;        /* token tiles, weight-row tiles */
+    /* split K: blockIdx.y = s handles K-steps [s * k_per, min(k_steps, (s + 1) * k_per)) and
+     * writes its partial tile, without bias, to part + s * M * N (row pitch N) */
+    int    splits, k_per;
+    float *part;
 };
+
+/* Where a block of a (possibly K-split) GEMM writes, and whether it adds the bias. */
+struct GemmOut { float *C; long ldc; const float *bias; };
+__device__ __forceinline__ GemmOut gemm_out(const GemmArgs &a)
+{
+    if (a.splits <= 1) return {a.C, a.ldc, a.bias};
+    return {a.part + (size_t)blockIdx.y * (size_t)a.M * (size_t)a.N, (long)a.N, nullptr};
+}
+
+/* C = bias + partial 0 + partial 1 + ... in that order: the result does not
+ * depend on which block finished first.  One thread per output. */
+__global__ void __launch_bounds__(256) gemm_splitk_reduce_kernel(float *__restrict__ C, long ldc, const float *__restrict__ part,
+                                                                 const float *__restrict__ bias, int M, int N, int splits)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x, mn = (size_t)M * (size_t)N;
+    if (i >= mn) return;
+    const int t = (int)(i / (size_t)N), n = (int)(i % (size_t)N);
+    float v = part[i];
+    for (int s = 1; s < splits; ++s) v += part[(size_t)s * mn + i];
+    C[(size_t)t * ldc + n] = bias ? v + bias[n] : v;
+}
+
+/* Split K when the tile grid leaves most of the chip idle: `tiles` blocks of
+ * `k_steps` loop iterations each.  Returns the number of splits (1 = none) so
+ * that tiles * splits approaches the CU count while every split keeps at
+ * least four iterations. */
+static int gemm_choose_splits(int tiles, int k_steps)
+{
+    if (tiles >= 160 || k_steps < 8) return 1;
+    int s = 256 / tiles;
+    if (s > k_steps / 4) s = k_steps / 4;
+    if (s > 16) s = 16;
+    return s < 2 ? 1 : s;
+}
+
+/* Scratch for the partial tiles of K-split launches: one grow-only device
+ * buffer per stream (work on one stream is ordered, so consecutive launches
+ * may share it).  Growing it allocates and therefore synchronises. */
+#include <mutex>
+static int gemm_workspace(hipStream_t s, size_t bytes, float **out)
+{
+    struct Slot { hipStream_t s; void *p; size_t cap; bool used; };
+    static Slot slots[16];
+    static std::mutex mu;
+    std::lock_guard<std::mutex> lock(mu);
+    Slot *sl = nullptr;
+    for (auto &c : slots) if (c.used && c.s == s) { sl = &c; break; }
+    if (!sl) for (auto &c : slots) if (!c.used) { sl = &c; c.used = true; c.s = s; c.p = nullptr; c.cap = 0; break; }
+    if (!sl) return (int)hipErrorOutOfMemory;
+    if (sl->cap < bytes) {
+        if (sl->p) {
+            hipError_t e = hipStreamSynchronize(s);
+            if (e != hipSuccess) return (int)e;
+            (void)hipFree(sl->p);
+            sl->p = nullptr; sl->cap = 0;
+        }
+        const size_t cap = bytes + bytes / 2;
+        hipError_t e = hipMalloc(&sl->p, cap);
+        if (e != hipSuccess) return (int)e;
+        sl->cap = cap;
+    }
+    *out = (float *)sl->p;
+    return 0;
+}
+
+/* Common launch tail: sets up the split, launches `kernel` on grid (x, splits)
+ * and, when split, the ordered reduction. */
+template <class Kernel>
+static int gemm_launch_split(Kernel kernel, GemmArgs &g, unsigned grid_x, int k_steps, hipStream_t s)
+{
+    g.splits = gemm_choose_splits(g.ntt * g.nnt, k_steps);
+    g.k_per = (k_steps + g.splits - 1) / g.splits;
+    g.splits = (k_steps + g.k_per - 1) / g.k_per;          /* no empty split */
+    g.part = nullptr;
+    if (g.splits > 1) {
+        int rc = gemm_workspace(s, (size_t)g.splits * (size_t)g.M * (size_t)g.N * sizeof(float), &g.part);
+        if (rc) return rc;
+    }
+    hipLaunchKernelGGL(kernel, dim3(grid_x, (unsigned)g.splits), dim3(256), 0, s, g);
+    if (g.splits > 1) {
+        const size_t mn = (size_t)g.M * (size_t)g.N;
+        hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, s,
+                           g.C, g.ldc, g.part, g.bias, g.M, g.N, g.splits);
+    }
+    return (int)hipGetLastError();
+}
 
 #ifndef CKQ_GEMM_WPE
 #define CKQ_GEMM_WPE 2          /* waves per SIMD the register budget is sized for */
@@ -213,7 +303,8 @@ __global__ void __launch_bounds__(256, WPE) gemm_q4k_mfma_kernel(GemmArgs a)
     if (nt >= a.nnt) return;
     const int t0 = tt * BM, n0 = nt * GEMM_BN;
     const u32 wstride = (u32)a.nb * 144u, xstride = (u32)a.nb * 292u;
-    const int last = a.nb - 1;
+    const int b0 = a.splits > 1 ? (int)blockIdx.y * a.k_per : 0;
+    const int b1 = a.splits > 1 ? min(a.nb, b0 + a.k_per) : a.nb, last = b1 - 1;
     const uint8_t *wbase = a.B + (size_t)n0 * wstride;       /* uniform */
     const uint8_t *xbase = a.A + (size_t)t0 * xstride;       /* uniform */
 
@@ -284,15 +375,15 @@ __global__ void __launch_bounds__(256, WPE) gemm_q4k_mfma_kernel(GemmArgs a)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[ts][r] = 0.0f;
 
-    copy_begin(0, 0);
+    copy_begin(b0, 0);
 #pragma unroll
     for (int i = 0; i < NWI + NQI; ++i) copy_one(i);
     side_store(0);
     __builtin_amdgcn_s_waitcnt(0x0070);   /* vmcnt(0): this wave's copies have landed */
     __syncthreads();
 
-    for (int b = 0; b < a.nb; ++b) {
-        const int cur = b & 1;
+    for (int b = b0; b < b1; ++b) {
+        const int cur = (b - b0) & 1;
         copy_begin(min(b + 1, last), cur ^ 1);
         __builtin_amdgcn_sched_barrier(0);
         gemm_block_pipe(stage[cur], wofs_l, aofs, col, half, acc, copy_one);
@@ -302,15 +393,16 @@ __global__ void __launch_bounds__(256, WPE) gemm_q4k_mfma_kernel(GemmArgs a)
         __syncthreads();
     }
 
+    const GemmOut o = gemm_out(a);
     const int n = n0 + wave * 32 + col;
     if (n < a.N) {
-        const float bias = a.bias ? a.bias[n] : 0.0f;
+        const float bias = o.bias ? o.bias[n] : 0.0f;
 #pragma unroll
         for (int ts = 0; ts < 2; ++ts)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int t = t0 + 32 * ts + 8 * (r >> 2) + 4 * half + (r & 3);
-                if (t < a.M) a.C[(size_t)t * a.ldc + n] = acc[ts][r] + bias;
+                if (t < a.M) o.C[(size_t)t * o.ldc + n] = acc[ts][r] + bias;
             }
     }
 }
@@ -326,6 +418,5 @@ static int launch_gemm_q4k_mfma(const void *A, const void *B, const float *bias,
     g.ntt = (M + GEMM_BM - 1) / GEMM_BM;
     g.nnt = (N + GEMM_BN - 1) / GEMM_BN;
     const int nnt8 = (g.nnt + 7) / 8 * 8;
-    hipLaunchKernelGGL((gemm_q4k_mfma_kernel<CKQ_GEMM_WPE>), dim3(g.ntt * nnt8), dim3(256), 0, s, g);
-    return (int)hipGetLastError();
+    return gemm_launch_split(gemm_q4k_mfma_kernel<CKQ_GEMM_WPE>, g, (unsigned)(g.ntt * nnt8), g.nb, s);
 }

@@ -186,7 +186,8 @@ __global__ void __launch_bounds__(256, 1) gemm_q5k_mfma_kernel(GemmArgs a)
     if (nt >= a.nnt) return;
     const int t0 = tt * BM, n0 = nt * GEMM5_BN;
     const u32 wstride = (u32)a.nb * 176u, xstride = (u32)a.nb * 292u;
-    const int last = a.nb - 1;
+    const int b0 = a.splits > 1 ? (int)blockIdx.y * a.k_per : 0;
+    const int b1 = a.splits > 1 ? min(a.nb, b0 + a.k_per) : a.nb, last = b1 - 1;
     const uint8_t *wbase = a.B + (size_t)n0 * wstride;       /* uniform */
     const uint8_t *xbase = a.A + (size_t)t0 * xstride;       /* uniform */
 
@@ -249,7 +250,7 @@ __global__ void __launch_bounds__(256, 1) gemm_q5k_mfma_kernel(GemmArgs a)
 
 #pragma unroll
     for (int p = 0; p < NST - 1; ++p) {
-        copy_begin(min(p, last), p);
+        copy_begin(min(b0 + p, last), p);
 #pragma unroll
         for (int i = 0; i < NCOPY; ++i) copy_one(i);
     }
@@ -260,7 +261,7 @@ __global__ void __launch_bounds__(256, 1) gemm_q5k_mfma_kernel(GemmArgs a)
      * are still in flight; the block's waves exchange data only through those
      * copies, so a bare s_barrier follows. */
     int cur = 0, pf = NST - 1;
-    for (int b = 0; b < a.nb; ++b) {
+    for (int b = b0; b < b1; ++b) {
         copy_begin(min(b + NST - 1, last), pf);
         __builtin_amdgcn_sched_barrier(0);
         gemm5_block<NCOPY>(stage[cur], wrow, aofs, col, half, acc, copy_one);
@@ -271,15 +272,16 @@ __global__ void __launch_bounds__(256, 1) gemm_q5k_mfma_kernel(GemmArgs a)
         pf = pf + 1 == NST ? 0 : pf + 1;
     }
 
+    const GemmOut o = gemm_out(a);
     const int n = n0 + wave * 32 + col;
     if (n < a.N) {
-        const float bias = a.bias ? a.bias[n] : 0.0f;
+        const float bias = o.bias ? o.bias[n] : 0.0f;
 #pragma unroll
         for (int ts = 0; ts < 2; ++ts)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int t = t0 + 32 * ts + 8 * (r >> 2) + 4 * half + (r & 3);
-                if (t < a.M) a.C[(size_t)t * a.ldc + n] = acc[ts][r] + bias;
+                if (t < a.M) o.C[(size_t)t * o.ldc + n] = acc[ts][r] + bias;
             }
     }
 }
@@ -295,6 +297,5 @@ static int launch_gemm_q5k_mfma(const void *A, const void *B, const float *bias,
     g.ntt = (M + GEMM5_BM - 1) / GEMM5_BM;
     g.nnt = (N + GEMM5_BN - 1) / GEMM5_BN;
     const int nnt8 = (g.nnt + 7) / 8 * 8;
-    hipLaunchKernelGGL(gemm_q5k_mfma_kernel, dim3(g.ntt * nnt8), dim3(256), 0, s, g);
-    return (int)hipGetLastError();
+    return gemm_launch_split(gemm_q5k_mfma_kernel, g, (unsigned)(g.ntt * nnt8), g.nb, s);
 }

@@ -196,7 +196,8 @@ __global__ void __launch_bounds__(256, 1) gemm_q6k_mfma_kernel(GemmArgs a)
     if (nt >= a.nnt) return;
     const int t0 = tt * BM, n0 = nt * GEMM6_BN;
     const u32 wstride = (u32)a.nb * 210u, xstride = (u32)a.nb * 292u;
-    const int last = a.nb - 1;
+    const int b0 = a.splits > 1 ? (int)blockIdx.y * a.k_per : 0;
+    const int b1 = a.splits > 1 ? min(a.nb, b0 + a.k_per) : a.nb, last = b1 - 1;
     const uint8_t *wbase = a.B + (size_t)n0 * wstride;       /* uniform */
     const uint8_t *xbase = a.A + (size_t)t0 * xstride;       /* uniform */
 
@@ -255,7 +256,7 @@ __global__ void __launch_bounds__(256, 1) gemm_q6k_mfma_kernel(GemmArgs a)
 
 #pragma unroll
     for (int p = 0; p < NST - 1; ++p) {
-        copy_begin(min(p, last), p);
+        copy_begin(min(b0 + p, last), p);
 #pragma unroll
         for (int i = 0; i < NCOPY; ++i) copy_one(i);
     }
@@ -270,7 +271,7 @@ __global__ void __launch_bounds__(256, 1) gemm_q6k_mfma_kernel(GemmArgs a)
     int cur = 0, pf = NST - 1;
     Gemm6Head<TH> head;
     gemm6_head_read<TH>(stage[0], wrow, aofs[0], half, head);
-    for (int b = 0; b < a.nb; ++b) {
+    for (int b = b0; b < b1; ++b) {
         copy_begin(min(b + NST - 1, last), pf);
         __builtin_amdgcn_sched_barrier(0);
         Gemm6Sums<TH> sums;
@@ -296,15 +297,16 @@ __global__ void __launch_bounds__(256, 1) gemm_q6k_mfma_kernel(GemmArgs a)
         __builtin_amdgcn_sched_barrier(0);
     }
 
+    const GemmOut o = gemm_out(a);
     const int n = n0 + wave * 32 + col;
     if (n < a.N) {
-        const float bias = a.bias ? a.bias[n] : 0.0f;
+        const float bias = o.bias ? o.bias[n] : 0.0f;
 #pragma unroll
         for (int ts = 0; ts < TH; ++ts)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int t = t0 + 32 * ts + 8 * (r >> 2) + 4 * half + (r & 3);
-                if (t < a.M) a.C[(size_t)t * a.ldc + n] = acc[ts][r] + bias;
+                if (t < a.M) o.C[(size_t)t * o.ldc + n] = acc[ts][r] + bias;
             }
     }
 }
@@ -323,10 +325,8 @@ static int launch_gemm_q6k_mfma(const void *A, const void *B, const float *bias,
     const int ntt4 = (M + 127) / 128;
     if (ntt4 * g.nnt > 128) {
         g.ntt = ntt4;
-        hipLaunchKernelGGL((gemm_q6k_mfma_kernel<4>), dim3(g.ntt * nnt8), dim3(256), 0, s, g);
-    } else {
-        g.ntt = (M + 63) / 64;
-        hipLaunchKernelGGL((gemm_q6k_mfma_kernel<2>), dim3(g.ntt * nnt8), dim3(256), 0, s, g);
+        return gemm_launch_split(gemm_q6k_mfma_kernel<4>, g, (unsigned)(g.ntt * nnt8), g.nb, s);
     }
-    return (int)hipGetLastError();
+    g.ntt = (M + 63) / 64;
+    return gemm_launch_split(gemm_q6k_mfma_kernel<2>, g, (unsigned)(g.ntt * nnt8), g.nb, s);
 }

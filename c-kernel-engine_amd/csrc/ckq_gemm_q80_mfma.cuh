@@ -68,7 +68,9 @@ __global__ void __launch_bounds__(256, 2) gemm_q80_mfma_kernel(GemmArgs a)
     const int t0 = tt * BM, n0 = nt * BN;
     const int nblk = a.nb;                                  /* 32-blocks per row */
     const u32 stride = (u32)nblk * 34u;                     /* bytes per weight row and per activation row */
-    const int niter = (nblk + KB - 1) / KB;
+    const int niter_all = (nblk + KB - 1) / KB;
+    const int it0 = a.splits > 1 ? (int)blockIdx.y * a.k_per : 0;
+    const int niter = a.splits > 1 ? min(niter_all, it0 + a.k_per) : niter_all;   /* this block runs iterations [it0, niter) */
     const uint8_t *wbase = a.B + (size_t)n0 * stride;       /* uniform */
     const uint8_t *xbase = a.A + (size_t)t0 * stride;       /* uniform */
 
@@ -148,7 +150,7 @@ __global__ void __launch_bounds__(256, 2) gemm_q80_mfma_kernel(GemmArgs a)
 
 #pragma unroll
     for (int p = 0; p < NST - 1; ++p) {
-        copy_begin(min(p, niter - 1), p);
+        copy_begin(min(it0 + p, niter - 1), p);
 #pragma unroll
         for (int i = 0; i < NCOPY; ++i) copy_one(i);
     }
@@ -159,7 +161,7 @@ __global__ void __launch_bounds__(256, 2) gemm_q80_mfma_kernel(GemmArgs a)
     const ckq_v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 
     int cur = 0;
-    for (int it = 0; it < niter; ++it) {
+    for (int it = it0; it < niter; ++it) {
         const Gemm8Stage &st = stage[cur];
         const int valid = min(KB, nblk - it * KB);
         /* Operands of block j (read one block ahead of their use, through the
@@ -210,7 +212,8 @@ __global__ void __launch_bounds__(256, 2) gemm_q80_mfma_kernel(GemmArgs a)
     }
 
     /* lane: token t0 + col + 32 ts, rows n0 + 32 wave + 8 q + 4 half + (0..3) */
-    const bool vec_ok = (a.ldc % 4 == 0) && (((uintptr_t)a.C) % 16 == 0) && (n0 + BN <= a.N);
+    const GemmOut o = gemm_out(a);
+    const bool vec_ok = (o.ldc % 4 == 0) && (((uintptr_t)o.C) % 16 == 0) && (n0 + BN <= a.N);
 #pragma unroll
     for (int ts = 0; ts < 2; ++ts) {
         const int t = t0 + col + 32 * ts;
@@ -220,8 +223,8 @@ __global__ void __launch_bounds__(256, 2) gemm_q80_mfma_kernel(GemmArgs a)
             const int n = n0 + 32 * wave + 8 * q + 4 * half;
             float v[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) v[i] = acc[ts][4 * q + i] + ((a.bias && n + i < a.N) ? a.bias[n + i] : 0.0f);
-            float *dst = a.C + (size_t)t * a.ldc + n;
+            for (int i = 0; i < 4; ++i) v[i] = acc[ts][4 * q + i] + ((o.bias && n + i < a.N) ? o.bias[n + i] : 0.0f);
+            float *dst = o.C + (size_t)t * o.ldc + n;
             if (vec_ok) *reinterpret_cast<float4 *>(dst) = make_float4(v[0], v[1], v[2], v[3]);
             else {
 #pragma unroll
@@ -242,6 +245,5 @@ static int launch_gemm_q80_mfma(const void *A, const void *B, const float *bias,
     g.ntt = (M + GEMM8_BM - 1) / GEMM8_BM;
     g.nnt = (N + GEMM8_BN - 1) / GEMM8_BN;
     const int nnt8 = (g.nnt + 7) / 8 * 8;
-    hipLaunchKernelGGL(gemm_q80_mfma_kernel, dim3(g.ntt * nnt8), dim3(256), 0, s, g);
-    return (int)hipGetLastError();
+    return gemm_launch_split(gemm_q80_mfma_kernel, g, (unsigned)(g.ntt * nnt8), (g.nb + GEMM8_KB - 1) / GEMM8_KB, s);
 }

@@ -870,3 +870,29 @@ def test_weights_register_manifest_and_ranges(tmp_path):
     assert T.norm_err(y2, T.oracle_gemv("q4_k", arena[oa:oa + len(wa)].copy(), xq, N, K)) <= TOL
     L.ckq_weights_clear()
     assert L.ckq_weights_resident(None) == 0
+
+
+# ---- K-split prefill GEMMs ----------------------------------------------------------------------
+
+@pytest.mark.parametrize("fmt", ["q4_k", "q5_k", "q6_k", "q8_0"])
+def test_gemm_split_k_is_deterministic_and_matches_oracle(fmt):
+    """Few tiles and a long K: the launch splits K over several blocks per tile
+    and sums the partial tiles in a fixed order.  Same bits on every run, the
+    oracle's values within the fp32 tolerance, bias added once."""
+    M, N, K = 96, 200, 19 * 256          # 4 tiles, 19 (or 38) K-steps: a ragged last split
+    bias = T.normal(N, 0.0, 0.5, seed=77)
+    W, _, xq = make_case(fmt, N, K, "enc", 1500 + T.FMT[fmt], tokens=M)
+    say("split-K gemm", fmt)
+    xq_d, W_d, b_d = P.to_device(xq), P.to_device(W), P.to_device(bias)
+    c0 = P.dev_gemm_nt(fmt, xq_d, W_d, b_d, M, N, K).cpu().numpy()
+    ref = T.oracle_gemm_nt(fmt, xq, W, bias, M, N, K)
+    assert T.norm_err(c0, ref) <= TOL
+    for _ in range(3):
+        assert np.array_equal(P.dev_gemm_nt(fmt, xq_d, W_d, b_d, M, N, K).cpu().numpy(), c0)
+    # a second stream gets its own scratch
+    import torch
+    st = torch.cuda.Stream()
+    with torch.cuda.stream(st):
+        c1 = P.dev_gemm_nt(fmt, xq_d, W_d, b_d, M, N, K)
+    st.synchronize()
+    assert np.array_equal(c1.cpu().numpy(), c0)
