@@ -98,14 +98,15 @@ static int gemm_choose_splits(int tiles, int k_steps)
 
 /* Scratch for the partial tiles of K-split launches: one grow-only device
  * buffer per stream (work on one stream is ordered, so consecutive launches
- * may share it).  Growing it allocates and therefore synchronises. */
+ * may share it).  Growing it allocates and therefore synchronises.  The
+ * caller holds g_split_mu from here until the reduction is enqueued, so two
+ * host threads launching on one stream cannot interleave their kernel pairs. */
 #include <mutex>
+static std::mutex g_split_mu;
 static int gemm_workspace(hipStream_t s, size_t bytes, float **out)
 {
     struct Slot { hipStream_t s; void *p; size_t cap; bool used; };
     static Slot slots[16];
-    static std::mutex mu;
-    std::lock_guard<std::mutex> lock(mu);
     Slot *sl = nullptr;
     for (auto &c : slots) if (c.used && c.s == s) { sl = &c; break; }
     if (!sl) for (auto &c : slots) if (!c.used) { sl = &c; c.used = true; c.s = s; c.p = nullptr; c.cap = 0; break; }
@@ -129,22 +130,23 @@ static int gemm_workspace(hipStream_t s, size_t bytes, float **out)
 /* Common launch tail: sets up the split, launches `kernel` on grid (x, splits)
  * and, when split, the ordered reduction. */
 template <class Kernel>
-static int gemm_launch_split(Kernel kernel, GemmArgs &g, unsigned grid_x, int k_steps, hipStream_t s)
+static int gemm_launch_split(Kernel kernel, GemmArgs &g, unsigned grid_x, int k_steps, hipStream_t s, unsigned threads = 256)
 {
     g.splits = gemm_choose_splits(g.ntt * g.nnt, k_steps);
     g.k_per = (k_steps + g.splits - 1) / g.splits;
     g.splits = (k_steps + g.k_per - 1) / g.k_per;          /* no empty split */
     g.part = nullptr;
-    if (g.splits > 1) {
-        int rc = gemm_workspace(s, (size_t)g.splits * (size_t)g.M * (size_t)g.N * sizeof(float), &g.part);
-        if (rc) return rc;
+    if (g.splits <= 1) {
+        hipLaunchKernelGGL(kernel, dim3(grid_x, 1u), dim3(threads), 0, s, g);
+        return (int)hipGetLastError();
     }
-    hipLaunchKernelGGL(kernel, dim3(grid_x, (unsigned)g.splits), dim3(256), 0, s, g);
-    if (g.splits > 1) {
-        const size_t mn = (size_t)g.M * (size_t)g.N;
-        hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, s,
-                           g.C, g.ldc, g.part, g.bias, g.M, g.N, g.splits);
-    }
+    std::lock_guard<std::mutex> lock(g_split_mu);
+    int rc = gemm_workspace(s, (size_t)g.splits * (size_t)g.M * (size_t)g.N * sizeof(float), &g.part);
+    if (rc) return rc;
+    hipLaunchKernelGGL(kernel, dim3(grid_x, (unsigned)g.splits), dim3(threads), 0, s, g);
+    const size_t mn = (size_t)g.M * (size_t)g.N;
+    hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, s,
+                       g.C, g.ldc, g.part, g.bias, g.M, g.N, g.splits);
     return (int)hipGetLastError();
 }
 
@@ -288,14 +290,24 @@ __device__ __forceinline__ void gemm_block_pipe(const GemmStage &st, u32 wofs, c
 #undef CKQ_PIN
 }
 
-template <int WPE>
-__global__ void __launch_bounds__(256, WPE) gemm_q4k_mfma_kernel(GemmArgs a)
+/* KG = 2: the block is two groups of four waves on the same tile; group g takes
+ * the K-blocks b0+g, b0+g+2, ... through its own pair of LDS stages, and the two
+ * partial tiles are added through LDS at the end (group 0 + group 1, a fixed
+ * order).  One such block fills a CU (two waves per SIMD) with ONE tile, so a
+ * grid of T tiles takes ceil(T / 256) rounds of half-length tiles instead of
+ * ceil(T / 512) rounds of full-length ones: 688 tiles need 3 x 0.5 instead of
+ * 2 x 1. */
+template <int WPE, int KG>
+__global__ void __launch_bounds__(256 * KG, KG == 2 ? 1 : WPE) gemm_q4k_mfma_kernel(GemmArgs a)
 {
     constexpr int BM = GEMM_BM;
-    __shared__ __attribute__((aligned(16))) GemmStage stage[2];
+    __shared__ __attribute__((aligned(16))) GemmStage stage_all[KG][2];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = wave_in_block();
+    const int wave_all = wave_in_block();
+    const int grp = KG == 2 ? wave_all >> 2 : 0, wave = wave_all & 3;
+    const int tid = threadIdx.x & 255, lane = tid & 63;
     const int col = lane & 31, half = lane >> 5;
+    GemmStage *const stage = stage_all[grp];
 
     const int id = blockIdx.x, xcd = id & 7, seq = id >> 3;
     const int tt = seq % a.ntt;
@@ -375,22 +387,43 @@ __global__ void __launch_bounds__(256, WPE) gemm_q4k_mfma_kernel(GemmArgs a)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[ts][r] = 0.0f;
 
-    copy_begin(b0, 0);
+    copy_begin(min(b0 + grp, last), 0);
 #pragma unroll
     for (int i = 0; i < NWI + NQI; ++i) copy_one(i);
     side_store(0);
     __builtin_amdgcn_s_waitcnt(0x0070);   /* vmcnt(0): this wave's copies have landed */
     __syncthreads();
 
-    for (int b = b0; b < b1; ++b) {
-        const int cur = (b - b0) & 1;
-        copy_begin(min(b + 1, last), cur ^ 1);
+    /* both groups run the same number of iterations (the barrier is the
+     * block's); a group without a block in the last one only keeps step */
+    const int niter = (b1 - b0 + KG - 1) / KG;
+    for (int it = 0; it < niter; ++it) {
+        const int b = b0 + grp + KG * it, cur = it & 1;
+        copy_begin(min(b + KG, last), cur ^ 1);
         __builtin_amdgcn_sched_barrier(0);
-        gemm_block_pipe(stage[cur], wofs_l, aofs, col, half, acc, copy_one);
+        if (KG == 1 || b < b1) gemm_block_pipe(stage[cur], wofs_l, aofs, col, half, acc, copy_one);
         __builtin_amdgcn_sched_barrier(0);
         side_store(cur ^ 1);
         __builtin_amdgcn_s_waitcnt(0x0070);
         __syncthreads();
+    }
+
+    if constexpr (KG == 2) {
+        /* partial tile of group 1 through LDS (every stage is idle now) */
+        float *red = reinterpret_cast<float *>(&stage_all[0][0]);
+        static_assert(sizeof(GemmStage) >= 32 * 256 * sizeof(float), "the reduction buffer fits one stage");
+        if (grp == 1) {
+#pragma unroll
+            for (int ts = 0; ts < 2; ++ts)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) red[(ts * 16 + r) * 256 + tid] = acc[ts][r];
+        }
+        __syncthreads();
+        if (grp == 1) return;
+#pragma unroll
+        for (int ts = 0; ts < 2; ++ts)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[ts][r] += red[(ts * 16 + r) * 256 + tid];
     }
 
     const GemmOut o = gemm_out(a);
@@ -418,5 +451,13 @@ static int launch_gemm_q4k_mfma(const void *A, const void *B, const float *bias,
     g.ntt = (M + GEMM_BM - 1) / GEMM_BM;
     g.nnt = (N + GEMM_BN - 1) / GEMM_BN;
     const int nnt8 = (g.nnt + 7) / 8 * 8;
-    return gemm_launch_split(gemm_q4k_mfma_kernel<CKQ_GEMM_WPE>, g, (unsigned)(g.ntt * nnt8), g.nb, s);
+    /* One tile per CU at most (with the K split the launch will choose) and a
+     * long enough K: two groups of waves per tile put a second wave on every
+     * SIMD (4096x11008 at M = 512: 80 -> 70 us).  With more tiles than CUs two
+     * independent blocks per CU interleave better than two groups in lockstep
+     * (11008x4096: 78 us against 88). */
+    const int tiles = g.ntt * g.nnt, sp = gemm_choose_splits(tiles, g.nb);
+    if (tiles * sp <= 256 && (g.nb + sp - 1) / sp >= 8)
+        return gemm_launch_split(gemm_q4k_mfma_kernel<CKQ_GEMM_WPE, 2>, g, (unsigned)(g.ntt * nnt8), g.nb, s, 512);
+    return gemm_launch_split(gemm_q4k_mfma_kernel<CKQ_GEMM_WPE, 1>, g, (unsigned)(g.ntt * nnt8), g.nb, s, 256);
 }

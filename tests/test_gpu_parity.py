@@ -896,3 +896,30 @@ def test_gemm_split_k_is_deterministic_and_matches_oracle(fmt):
         c1 = P.dev_gemm_nt(fmt, xq_d, W_d, b_d, M, N, K)
     st.synchronize()
     assert np.array_equal(c1.cpu().numpy(), c0)
+
+
+def test_gemm_mfma_q4_k_two_wave_groups_per_tile():
+    """160 tiles and nine K-blocks: one tile per CU, so the launch gives every
+    tile two groups of waves that take alternate K-blocks (five and four) and
+    add their partial tiles in a fixed order.  The oracle on a sample of weight
+    rows for every token, whole rows against the GEMV kernel for a few tokens,
+    and the same bits on a second run."""
+    M, N, K = 512, 2560, 2304
+    W = T.synth_weights("q4_k", N, K, seed=5250)
+    xf = T.normal(M * K, 0.0, 1.0, seed=5251)
+    bias = T.normal(N, 0.0, 0.5, seed=5252)
+    say("gemm mfma q4_k two wave groups")
+    xq_d = P.dev_quantize(P.to_device(xf), "q8_k", rows=M)
+    xq = xq_d.cpu().numpy()
+    Wd, bd = P.to_device(W), P.to_device(bias)
+    c = P.dev_gemm_nt("q4_k", xq_d, Wd, bd, M, N, K).cpu().numpy()
+    rb = T.row_bytes("q4_k", K)
+    rows = np.array([0, 1, 31, 32, 127, 128, 1279, 1280, 2558, 2559])
+    Wsub = np.ascontiguousarray(W.reshape(N, rb)[rows]).reshape(-1)
+    ref = T.oracle_gemm_nt("q4_k", xq, Wsub, np.ascontiguousarray(bias[rows]), M, len(rows), K)
+    assert T.norm_err(c[:, rows], ref) <= TOL
+    ab = T.row_bytes("q8_k", K)
+    for t in (0, 63, 64, 300, 511):
+        y = P.dev_gemm_nt("q4_k", P.to_device(xq[t * ab:(t + 1) * ab].copy()), Wd, bd, 1, N, K).cpu().numpy().reshape(-1)
+        assert T.norm_err(c[t], y) <= 2e-6, t
+    assert np.array_equal(P.dev_gemm_nt("q4_k", xq_d, Wd, bd, M, N, K).cpu().numpy(), c)
