@@ -923,3 +923,33 @@ def test_gemm_mfma_q4_k_two_wave_groups_per_tile():
         y = P.dev_gemm_nt("q4_k", P.to_device(xq[t * ab:(t + 1) * ab].copy()), Wd, bd, 1, N, K).cpu().numpy().reshape(-1)
         assert T.norm_err(c[t], y) <= 2e-6, t
     assert np.array_equal(P.dev_gemm_nt("q4_k", xq_d, Wd, bd, M, N, K).cpu().numpy(), c)
+
+
+# ---- matrix-core GEMMs on seeded random shapes ---------------------------------------------------
+
+@pytest.mark.parametrize("fmt", ["q4_k", "q5_k", "q6_k", "q8_0"])
+def test_gemm_mfma_random_shapes(fmt):
+    """Ragged token counts, row counts that are no multiple of the 32-row wave
+    slice or the 128-row tile, K from one block up, with and without bias and
+    with a row pitch wider than N: every combination a tile edge can meet."""
+    import torch
+    rng = np.random.default_rng(20240 + T.FMT[fmt])
+    lo = 65 if fmt == "q5_k" else 17
+    for case in range(10):
+        M = int(rng.integers(lo, 210))
+        N = int(rng.integers(1, 300))
+        K = int(rng.integers(1, 21)) * 32 if fmt == "q8_0" else int(rng.integers(1, 7)) * 256
+        use_bias = bool(case & 1)
+        ldc = N + int(rng.integers(0, 9)) if case % 3 == 0 else N
+        W, _, xq = make_case(fmt, N, K, "enc" if case & 2 else "rand", 7000 + 31 * case + T.FMT[fmt], tokens=M)
+        bias = T.normal(N, 0.0, 0.5, seed=case) if use_bias else None
+        say("gemm mfma random", fmt, "M", M, "N", N, "K", K, "ldc", ldc, "bias", use_bias)
+        ref = T.oracle_gemm_nt(fmt, xq, W, bias, M, N, K)
+        xq_d, W_d = P.to_device(xq), P.to_device(W)
+        b_d = P.to_device(bias) if use_bias else None
+        c_d = torch.full((M * ldc,), 3.0, dtype=torch.float32, device="cuda")
+        P.check(ckq.lib().ckq_gemm_nt_dev(P.FMT[fmt], P._dp(xq_d), P._dp(W_d), P._dp(b_d), P._dp(c_d), M, N, K, ldc,
+                                          P._stream()), "ckq_gemm_nt_dev")
+        c = c_d.cpu().numpy().reshape(M, ldc)
+        assert T.norm_err(c[:, :N], ref) <= TOL, (fmt, M, N, K, ldc)
+        assert np.all(c[:, N:] == 3.0), (fmt, M, N, K, ldc)         # nothing written beyond a row's N outputs
