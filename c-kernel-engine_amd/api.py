@@ -10,9 +10,9 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 HEADER = os.path.join(ROOT, "include", "ckernel_quant_hip.h")
 
-FMT = {"q4_k": 0, "q5_k": 1, "q6_k": 2, "q8_0": 3, "q8_k": 4}
-BLOCK_BYTES = {"q4_k": 144, "q5_k": 176, "q6_k": 210, "q8_0": 34, "q8_k": 292}
-BLOCK_ELEMS = {"q4_k": 256, "q5_k": 256, "q6_k": 256, "q8_0": 32, "q8_k": 256}
+FMT = {"q4_k": 0, "q5_k": 1, "q6_k": 2, "q8_0": 3, "q8_k": 4, "q5_0": 5}
+BLOCK_BYTES = {"q4_k": 144, "q5_k": 176, "q6_k": 210, "q8_0": 34, "q8_k": 292, "q5_0": 22}
+BLOCK_ELEMS = {"q4_k": 256, "q5_k": 256, "q6_k": 256, "q8_0": 32, "q8_k": 256, "q5_0": 32}
 
 
 class CkqError(RuntimeError):
@@ -72,6 +72,10 @@ _SIGS = {
     "embedding_forward_q6_k": (None, [_vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i]),
     "embedding_forward_q8_0": (None, [_vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i]),
     "rmsnorm_q8_k_fused": (None, [_vp, _vp, _vp, _i, _i, _i, _c.c_float]),
+    "vec_dot_q5_0_q8_0": (None, [_i, _vp, _vp, _vp]),
+    "gemv_q5_0_q8_0": (None, [_vp, _vp, _vp, _i, _i]),
+    "gemv_q5_0_q8_0_parallel_simd": (None, [_vp, _vp, _vp, _i, _i, _i, _i]),
+    "gemm_nt_q5_0_q8_0": (None, [_vp, _vp, _vp, _vp, _i, _i, _i]),
     "fused_mlp_swiglu_prefill_w1w2_quant": (None, [_vp, _vp, _vp, _i, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp]),
     "fused_mlp_swiglu_prefill_w1w2_quant_scratch_size": (_c.c_size_t, [_i, _i]),
     "gemv_q4_k": (None, [_vp, _vp, _vp, _i, _i]),

@@ -350,6 +350,42 @@ struct FmtQ80 {
     static constexpr int SUBS_PER_BLOCK = 1;
 };
 
+/* Q5_0 weights against Q8_0 activations: 22-byte blocks (fp16 d, 32 fifth bits,
+ * 16 nibble bytes), values q - 16 in [-16, 15]; everything on the activation
+ * side is FmtQ80's.  Reference: gemm_kernels_q5_0.c:901-939. */
+struct FmtQ50 : FmtQ80 {
+    static constexpr int WBLOCK = 22;
+    struct Wt { u32 qs[4]; u32 qh; u32 d; };
+    static __device__ __forceinline__ Off w_off(int pos)
+    {
+        Off o;
+        o.blk = (u32)pos * WBLOCK;
+        return o;
+    }
+    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, const Off &o)
+    {
+        w.d = ld2(row + o.blk);
+        w.qh = ld4<2>(row + o.blk + 2);
+        ld16<2>(w.qs, row + o.blk + 6);
+    }
+    /* four 5-bit values (nibbles in n, their fifth bits in the low four bits
+     * of h) minus 16, as packed int8 */
+    static __device__ __forceinline__ int q5_bytes(u32 n, u32 h)
+    {
+        const u32 spread = ((h & 15u) * 0x00204081u) & 0x01010101u;      /* bit k -> byte k */
+        const u32 v = n | (spread << 4);                                  /* 0..31 per byte */
+        return (int)((((v | 0x80808080u) - 0x10101010u)) ^ 0x80808080u);  /* - 16 per byte, no borrows */
+    }
+    static __device__ __forceinline__ void decode(Dec &d, const Wt &w, int)
+    {
+        for (int i = 0; i < 4; ++i) {
+            d.q[i]     = q5_bytes(w.qs[i] & 0x0f0f0f0fu, w.qh >> (4 * i));
+            d.q[4 + i] = q5_bytes((w.qs[i] >> 4) & 0x0f0f0f0fu, w.qh >> (16 + 4 * i));
+        }
+        d.d = h2f(w.d);
+    }
+};
+
 /* Q8_0 weights against fp32 activations (no activation quantization). */
 struct FmtQ80F32 {
     static constexpr int POS_PER_BLOCK = 1, WBLOCK = 34, XBLOCK = 128, NSUB = 1;

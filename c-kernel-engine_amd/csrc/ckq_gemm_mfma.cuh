@@ -102,14 +102,15 @@ static int gemm_choose_splits(int tiles, int k_steps)
  * caller holds g_split_mu from here until the reduction is enqueued, so two
  * host threads launching on one stream cannot interleave their kernel pairs. */
 #include <mutex>
-static std::mutex g_split_mu;
-static int gemm_workspace(hipStream_t s, size_t bytes, float **out)
+static std::recursive_mutex g_split_mu;
+/* kind 0: partial tiles of a K split; kind 1: weights rewritten for another kernel */
+static int gemm_workspace(int kind, hipStream_t s, size_t bytes, float **out)
 {
-    struct Slot { hipStream_t s; void *p; size_t cap; bool used; };
-    static Slot slots[16];
+    struct Slot { hipStream_t s; int kind; void *p; size_t cap; bool used; };
+    static Slot slots[32];
     Slot *sl = nullptr;
-    for (auto &c : slots) if (c.used && c.s == s) { sl = &c; break; }
-    if (!sl) for (auto &c : slots) if (!c.used) { sl = &c; c.used = true; c.s = s; c.p = nullptr; c.cap = 0; break; }
+    for (auto &c : slots) if (c.used && c.s == s && c.kind == kind) { sl = &c; break; }
+    if (!sl) for (auto &c : slots) if (!c.used) { sl = &c; c.used = true; c.s = s; c.kind = kind; c.p = nullptr; c.cap = 0; break; }
     if (!sl) return (int)hipErrorOutOfMemory;
     if (sl->cap < bytes) {
         if (sl->p) {
@@ -140,8 +141,8 @@ static int gemm_launch_split(Kernel kernel, GemmArgs &g, unsigned grid_x, int k_
         hipLaunchKernelGGL(kernel, dim3(grid_x, 1u), dim3(threads), 0, s, g);
         return (int)hipGetLastError();
     }
-    std::lock_guard<std::mutex> lock(g_split_mu);
-    int rc = gemm_workspace(s, (size_t)g.splits * (size_t)g.M * (size_t)g.N * sizeof(float), &g.part);
+    std::lock_guard<std::recursive_mutex> lock(g_split_mu);
+    int rc = gemm_workspace(0, s, (size_t)g.splits * (size_t)g.M * (size_t)g.N * sizeof(float), &g.part);
     if (rc) return rc;
     hipLaunchKernelGGL(kernel, dim3(grid_x, (unsigned)g.splits), dim3(threads), 0, s, g);
     const size_t mn = (size_t)g.M * (size_t)g.N;

@@ -413,7 +413,7 @@ void ckq_set_parallel_whole(int enabled)
 /* Shapes                                                                    */
 /* ------------------------------------------------------------------------ */
 
-static int fmt_block_elems(int fmt) { return (fmt == CKQ_FMT_Q8_0 || fmt == CKQ_KERNEL_Q80_F32) ? 32 : 256; }
+static int fmt_block_elems(int fmt) { return (fmt == CKQ_FMT_Q8_0 || fmt == CKQ_FMT_Q5_0 || fmt == CKQ_KERNEL_Q80_F32) ? 32 : 256; }
 
 static int is_f32act(int fmt) { return fmt == CKQ_KERNEL_Q80_F32 || fmt == CKQ_KERNEL_Q4K_F32 || fmt == CKQ_KERNEL_Q6K_F32; }
 
@@ -431,7 +431,7 @@ static size_t weight_row_bytes(int fmt, int K)
 static size_t act_row_bytes(int fmt, int K)
 {
     if (is_f32act(fmt)) return (size_t)K * 4;
-    if (fmt == CKQ_FMT_Q8_0) return ckq_row_bytes(CKQ_FMT_Q8_0, K);
+    if (fmt == CKQ_FMT_Q8_0 || fmt == CKQ_FMT_Q5_0) return ckq_row_bytes(CKQ_FMT_Q8_0, K);
     return ckq_row_bytes(CKQ_FMT_Q8_K, K);
 }
 
@@ -655,6 +655,28 @@ void vec_dot_q8_0_q8_0(int n, float *s, const void *vx, const void *vy)
     host_matmul(CKQ_FMT_Q8_0, vy, vx, NULL, s, 1, 1, n, 1, 0, 1);
 }
 
+/* Q5_0 weights (the format of rows too short for K-quants) against Q8_0 activations. */
+void vec_dot_q5_0_q8_0(int n, float *s, const void *vx, const void *vy)
+{
+    if (!s || !vx || !vy || n <= 0) return;
+    host_matmul(CKQ_FMT_Q5_0, vy, vx, NULL, s, 1, 1, n, 1, 0, 1);
+}
+
+void gemv_q5_0_q8_0(float *y, const void *W, const void *x_q8, int M, int K)
+{
+    host_matmul(CKQ_FMT_Q5_0, x_q8, W, NULL, y, 1, M, K, M, 0, M);
+}
+
+void gemv_q5_0_q8_0_parallel_simd(float *y, const void *W, const void *x_q8, int M, int K, int ith, int nth)
+{
+    host_gemv_split(CKQ_FMT_Q5_0, y, W, x_q8, M, K, ith, nth);
+}
+
+void gemm_nt_q5_0_q8_0(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K)
+{
+    host_matmul(CKQ_FMT_Q5_0, A_q8, B, bias, C, M, N, K, N, 0, N);
+}
+
 void gemv_q8_0(float *y, const void *W, const float *x, int M, int K)
 {
     host_matmul(CKQ_KERNEL_Q80_F32, x, W, NULL, y, 1, M, K, M, 0, M);
@@ -776,12 +798,7 @@ void fused_mlp_swiglu_prefill_w1w2_quant(const float *x, const void *W1, const f
     if (aligned_embed_dim % 32 || aligned_intermediate_dim % 256) return;
     if ((w1_dt != CKQ_CK_DT_Q8_0 && w1_dt != CKQ_CK_DT_Q5_0) || (w2_dt != CKQ_CK_DT_Q4_K && w2_dt != CKQ_CK_DT_Q6_K))
         return;
-    if (w1_dt == CKQ_CK_DT_Q5_0) {
-        pthread_mutex_lock(&g_mu);
-        fail(CKQ_EFORMAT, "fused_mlp_swiglu_prefill_w1w2_quant: Q5_0 weights are not built");
-        pthread_mutex_unlock(&g_mu);
-        return;
-    }
+    const int fmt1 = w1_dt == CKQ_CK_DT_Q8_0 ? CKQ_FMT_Q8_0 : CKQ_FMT_Q5_0;
     const int E = aligned_embed_dim, I = aligned_intermediate_dim;
     const int fmt2 = w2_dt == CKQ_CK_DT_Q4_K ? CKQ_FMT_Q4_K : CKQ_FMT_Q6_K;
     const size_t out_bytes = (size_t)seq_len * E * 4;
@@ -791,7 +808,7 @@ void fused_mlp_swiglu_prefill_w1w2_quant(const float *x, const void *W1, const f
         const void *dx, *dW1, *dW2, *dB1 = NULL, *dB2 = NULL;
         void *dq, *dgu, *dh;
         if (stage_in(BUF_X, x, (size_t)seq_len * E * 4, &dx)) break;
-        if (weights_resolve(W1, (size_t)2 * I * weight_row_bytes(CKQ_FMT_Q8_0, E), &dW1)) break;
+        if (weights_resolve(W1, (size_t)2 * I * weight_row_bytes(fmt1, E), &dW1)) break;
         if (weights_resolve(W2, (size_t)E * weight_row_bytes(fmt2, I), &dW2)) break;
         /* both biases share the bias staging buffer: B1 first, B2 behind it */
         if (B1 || B2) {
@@ -820,7 +837,7 @@ void fused_mlp_swiglu_prefill_w1w2_quant(const float *x, const void *W1, const f
         if (!out_on_dev && buf_reserve(BUF_Y, out_bytes, &dout)) break;
         int rc = ckq_launch_quantize_q8_0((const float *)dx, dq, seq_len, E, g_stream);
         if (rc) { fail(rc, "quantize launch"); break; }
-        rc = ckq_launch_gemv(CKQ_FMT_Q8_0, (float *)dgu, dW1, dq, (const float *)dB1, 2 * I, E, seq_len, 2L * I, 0, 2 * I,
+        rc = ckq_launch_gemv(fmt1, (float *)dgu, dW1, dq, (const float *)dB1, 2 * I, E, seq_len, 2L * I, 0, 2 * I,
                              NULL, g_stream);
         if (rc) { fail(rc, "gate/up GEMM launch"); break; }
         rc = ckq_launch_swiglu_q8_k((const float *)dgu, (const float *)dgu + I, dh, seq_len, I, 2L * I, g_stream);
@@ -965,7 +982,8 @@ int ckq_quantize_q8_0_dev(const float *x, void *y, int num_rows, int k, void *st
 int ckq_gemm_nt_dev(int fmt, const void *A_q8, const void *B, const float *bias, float *C,
                     int M, int N, int K, long ldc, void *stream)
 {
-    if (fmt != CKQ_FMT_Q4_K && fmt != CKQ_FMT_Q5_K && fmt != CKQ_FMT_Q6_K && fmt != CKQ_FMT_Q8_0) return CKQ_EFORMAT;
+    if (fmt != CKQ_FMT_Q4_K && fmt != CKQ_FMT_Q5_K && fmt != CKQ_FMT_Q6_K && fmt != CKQ_FMT_Q8_0 && fmt != CKQ_FMT_Q5_0)
+        return CKQ_EFORMAT;
     return ckq_launch_gemv(fmt, C, B, A_q8, bias, N, K, M, ldc, 0, N, NULL, stream);
 }
 
@@ -1031,7 +1049,8 @@ int ckq_matmul_sequence_dev(const ckq_matmul_op *ops, int nops, int repeat, void
 int ckq_subblock_dots_dev(int fmt, int32_t *out, const void *W, const void *x_q8, int M, int K, void *stream)
 {
     if (!out) return CKQ_EINVAL;
-    if (fmt != CKQ_FMT_Q4_K && fmt != CKQ_FMT_Q5_K && fmt != CKQ_FMT_Q6_K && fmt != CKQ_FMT_Q8_0) return CKQ_EFORMAT;
+    if (fmt != CKQ_FMT_Q4_K && fmt != CKQ_FMT_Q5_K && fmt != CKQ_FMT_Q6_K && fmt != CKQ_FMT_Q8_0 && fmt != CKQ_FMT_Q5_0)
+        return CKQ_EFORMAT;
     return ckq_launch_gemv(fmt, NULL, W, x_q8, NULL, M, K, 1, M, 0, M, out, stream);
 }
 

@@ -286,6 +286,42 @@ static int launch_fmt(const GemvArgs &a, bool dump, int max_mt, hipStream_t s)
     return launch_mt<F, 64, 4>(a, dump, max_mt, s);   /* longer rows loop in passes of 256 positions */
 }
 
+/* Q5_0 block -> Q8_0 block: the scale is kept, the 32 values become int8
+ * q - 16.  One thread per block. */
+__global__ void __launch_bounds__(256) q5_0_to_q8_0_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, size_t nblocks)
+{
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= nblocks) return;
+    FmtQ50::Wt w;
+    FmtQ50::Off o;
+    o.blk = 0;
+    FmtQ50::load_w(w, src + i * 22, o);
+    FmtQ50::Dec d;
+    FmtQ50::decode(d, w, 0);
+    uint8_t *out = dst + i * 34;
+    *reinterpret_cast<uint16_t *>(out) = (uint16_t)w.d;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {             /* 34-byte blocks: 2-byte aligned stores */
+        reinterpret_cast<uint16_t *>(out + 2)[2 * k] = (uint16_t)((u32)d.q[k] & 0xffffu);
+        reinterpret_cast<uint16_t *>(out + 2)[2 * k + 1] = (uint16_t)((u32)d.q[k] >> 16);
+    }
+}
+
+static int launch_gemm_q50_via_q80(const void *A, const void *B, const float *bias, float *C,
+                                   int M, int N, int K, long ldc, hipStream_t s)
+{
+    const size_t nblocks = (size_t)N * (size_t)(K / 32);
+    std::lock_guard<std::recursive_mutex> lock(g_split_mu);   /* the scratch is shared by launches on this stream */
+    float *tmp = nullptr;
+    int rc = gemm_workspace(1, s, nblocks * 34, &tmp);
+    if (rc) return rc;
+    hipLaunchKernelGGL(q5_0_to_q8_0_kernel, dim3((unsigned)((nblocks + 255) / 256)), dim3(256), 0, s,
+                       (const uint8_t *)B, (uint8_t *)tmp, nblocks);
+    rc = (int)hipGetLastError();
+    if (rc) return rc;
+    return launch_gemm_q80_mfma(A, tmp, bias, C, M, N, K, ldc, s);
+}
+
 extern "C" int ckq_launch_gemv(int fmt, float *y, const void *W, const void *X, const float *bias,
                                int nrows, int K, int ntok, long ldy, int row0, int row1,
                                int32_t *subdots, void *stream)
@@ -328,6 +364,14 @@ extern "C" int ckq_launch_gemv(int fmt, float *y, const void *W, const void *X, 
             return launch_gemm_q80_mfma(X, W, bias, y, ntok, nrows, K, ldy, s);
         a.npos = K / 32; a.wrow = (long)(K / 32) * 34; a.xrow = (long)(K / 32) * 34; a.nsub_row = K / 32;
         return launch_fmt<FmtQ80>(a, dump, 8, s);
+    case CKQ_FMT_Q5_0:
+        if (K % 32) return CKQ_ESHAPE;
+        /* prefill: the blocks are rewritten as Q8_0 blocks (same scale, values
+         * q - 16: every dot product is unchanged) and go to the Q8_0 GEMM */
+        if (!dump && ntok > CKQ_GEMM_MIN_TOKENS && row0 == 0 && row1 == nrows)
+            return launch_gemm_q50_via_q80(X, W, bias, y, ntok, nrows, K, ldy, s);
+        a.npos = K / 32; a.wrow = (long)(K / 32) * 22; a.xrow = (long)(K / 32) * 34; a.nsub_row = K / 32;
+        return launch_fmt<FmtQ50>(a, dump, 8, s);
     case CKQ_KERNEL_Q80_F32:
         if (K % 32) return CKQ_ESHAPE;
         if (dump) return CKQ_EINVAL;

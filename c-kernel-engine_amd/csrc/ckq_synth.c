@@ -231,6 +231,29 @@ void ckq_synth_quantize_q8_0(const float *w, void *out, size_t n)
     }
 }
 
+/* Q5_0 weights: d = (value of largest magnitude) / -16 (fp16), q = min(31, trunc(w/d + 16.5)). */
+void ckq_synth_quantize_q5_0(const float *w, void *out, size_t n)
+{
+    ckq_block_q5_0 *b = (ckq_block_q5_0 *)out;
+    for (size_t i = 0; i < n / CKQ_QK8_0; ++i, w += CKQ_QK8_0) {
+        float amax = 0.0f, vmax = 0.0f;
+        for (int l = 0; l < 32; ++l) {
+            const float a = fabsf(w[l]);
+            if (a > amax) { amax = a; vmax = w[l]; }
+        }
+        const float d = vmax / -16.0f, id = d != 0.0f ? 1.0f / d : 0.0f;
+        uint32_t qh = 0;
+        b[i].d = ckq_synth_fp32_to_fp16(d);
+        for (int l = 0; l < 16; ++l) {
+            const int q0 = clampi((int)(w[l] * id + 16.5f), 0, 31), q1 = clampi((int)(w[16 + l] * id + 16.5f), 0, 31);
+            b[i].qs[l] = (uint8_t)((q0 & 15) | ((q1 & 15) << 4));
+            qh |= (uint32_t)(q0 >> 4) << l;
+            qh |= (uint32_t)(q1 >> 4) << (16 + l);
+        }
+        memcpy(b[i].qh, &qh, 4);
+    }
+}
+
 int ckq_synth_quantize(int fmt, const float *w, void *out, size_t n)
 {
     switch (fmt) {
@@ -238,6 +261,7 @@ int ckq_synth_quantize(int fmt, const float *w, void *out, size_t n)
     case CKQ_FMT_Q5_K: ckq_synth_quantize_q5_k(w, out, n); return 0;
     case CKQ_FMT_Q6_K: ckq_synth_quantize_q6_k(w, out, n); return 0;
     case CKQ_FMT_Q8_0: ckq_synth_quantize_q8_0(w, out, n); return 0;
+    case CKQ_FMT_Q5_0: ckq_synth_quantize_q5_0(w, out, n); return 0;
     default: return -1;
     }
 }
@@ -292,6 +316,9 @@ int ckq_synth_random_blocks(int fmt, void *out, size_t nblocks, uint64_t seed)
                 if (b->qs[j] == -128) b->qs[j] = -127;
             break;
         }
+        case CKQ_FMT_Q5_0:
+            ((ckq_block_q5_0 *)blk)->d = ckq_synth_fp32_to_fp16(d);
+            break;
         case CKQ_FMT_Q8_K: {
             ckq_block_q8_K *b = (ckq_block_q8_K *)blk;
             b->d = d;

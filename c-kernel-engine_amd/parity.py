@@ -22,7 +22,7 @@ def _p(a):
 
 
 def act_format(wfmt):
-    return "q8_0" if wfmt == "q8_0" else "q8_k"
+    return "q8_0" if wfmt in ("q8_0", "q5_0") else "q8_k"
 
 
 # ---- host-pointer (drop-in) path ------------------------------------------------
@@ -37,9 +37,10 @@ def quantize(x, fmt="q8_k", rows=1):
     return out
 
 
-_GEMV = {"q4_k": "gemv_q4_k_q8_k", "q5_k": "gemv_q5_k_q8_k", "q6_k": "gemv_q6_k_q8_k", "q8_0": "gemv_q8_0_q8_0"}
+_GEMV = {"q4_k": "gemv_q4_k_q8_k", "q5_k": "gemv_q5_k_q8_k", "q6_k": "gemv_q6_k_q8_k", "q8_0": "gemv_q8_0_q8_0",
+         "q5_0": "gemv_q5_0_q8_0"}
 _GEMM_NT = {"q4_k": "gemm_nt_q4_k_q8_k", "q5_k": "gemm_nt_q5_k_q8_k", "q6_k": "gemm_nt_q6_k_q8_k",
-            "q8_0": "gemm_nt_q8_0_q8_0"}
+            "q8_0": "gemm_nt_q8_0_q8_0", "q5_0": "gemm_nt_q5_0_q8_0"}
 
 
 def gemv(fmt, W, x_q8, M, K, name=None):

@@ -134,17 +134,26 @@ void embedding_forward_q8_0(const int32_t *token_ids, int token_count, int vocab
 void rmsnorm_q8_k_fused(const float *input, const float *gamma, void *vy, int tokens, int d_model,
                         int aligned_embed_dim, float eps);
 
+/* Q5_0 weights (fp16 d, 32 five-bit values q - 16 per 22-byte block: the
+ * format GGUF files use for rows too short for K-quants) against Q8_0
+ * activations.  Token counts above 16 rewrite the blocks as Q8_0 blocks on the
+ * device (same scale, values q - 16: every dot product is unchanged) and run
+ * the Q8_0 matrix-core GEMM.  Replaces src/kernels/gemm_kernels_q5_0.c:1602-1620
+ * (vec_dot), :1637-1657 (gemv), :1659-1700 (_parallel_simd), :1725-1753 (gemm_nt).
+ * The fp32-activation forms gemv_q5_0 / gemm_nt_q5_0 are not built. */
+void vec_dot_q5_0_q8_0(int n, float *s, const void *vx, const void *vy);
+void gemv_q5_0_q8_0(float *y, const void *W, const void *x_q8, int M, int K);
+void gemv_q5_0_q8_0_parallel_simd(float *y, const void *W, const void *x_q8, int M, int K, int ith, int nth);
+void gemm_nt_q5_0_q8_0(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K);
+
 /* Fused prefill MLP around the quantized GEMMs: x (seq_len rows of
  * aligned_embed_dim floats) is quantized to Q8_0, multiplied with W1 = [gate
  * rows; up rows] (2 * aligned_intermediate_dim rows, bias B1 of the same length
  * or NULL), SiLU(gate) * up is quantized to Q8_K and multiplied with W2
  * (aligned_embed_dim rows, bias B2 or NULL) into output (seq_len rows of
  * aligned_embed_dim floats).  w1_dt / w2_dt are the reference's CKDataType
- * values (include/ckernel_dtype.h:27-50): W1 CKQ_CK_DT_Q8_0, W2 CKQ_CK_DT_Q4_K
- * or CKQ_CK_DT_Q6_K.  The reference also accepts Q5_0 for W1; that format is
- * not built here and the request fails like any other the library cannot
- * serve: the process aborts, or with CKQ_ABORT_ON_ERROR=0 the call returns
- * without touching output and ckq_last_error() reports CKQ_EFORMAT.  Other
+ * values (include/ckernel_dtype.h:27-50): W1 CKQ_CK_DT_Q8_0 or CKQ_CK_DT_Q5_0, W2
+ * CKQ_CK_DT_Q4_K or CKQ_CK_DT_Q6_K, as in the reference; other types and other
  * argument errors return without touching output, as the reference does.  `scratch` must be non-NULL as in
  * the reference but is not used: intermediates stay in device memory.  Any mix
  * of host and device pointers; synchronous.  The SiLU uses an exponential

@@ -35,6 +35,16 @@ typedef struct {
     int8_t   qs[CKQ_QK8_0];
 } ckq_block_q8_0;
 
+/* Q5_0: 32 x 5-bit with one fp16 scale, value = d * (q - 16).  Element l < 16
+ * is the low nibble of qs[l] with bit l of qh (little-endian 32-bit) as fifth
+ * bit; element 16 + l the high nibble with bit 16 + l.  22 bytes, 2-byte
+ * aligned (reference: include/ckernel_quant.h:60-75). */
+typedef struct {
+    ckq_half d;
+    uint8_t  qh[4];
+    uint8_t  qs[CKQ_QK8_0 / 2];
+} ckq_block_q5_0;
+
 /* Q4_K: 256 x 4-bit. fp16 d, fp16 dmin, 8 six-bit scales + 8 six-bit mins
  * packed in 12 bytes, 128 nibble bytes. 144 bytes (9 x 16 B).
  * For j in {0,64,128,192}: qs[j/2 + l] low nibble = element j+l,
@@ -75,6 +85,7 @@ typedef struct {
 } ckq_block_q8_K;
 
 #define CKQ_BLOCK_Q8_0_SIZE 34
+#define CKQ_BLOCK_Q5_0_SIZE 22
 #define CKQ_BLOCK_Q4_K_SIZE 144
 #define CKQ_BLOCK_Q5_K_SIZE 176
 #define CKQ_BLOCK_Q6_K_SIZE 210
@@ -86,6 +97,7 @@ typedef struct {
 #define CKQ_STATIC_ASSERT(c, m) _Static_assert(c, m)
 #endif
 CKQ_STATIC_ASSERT(sizeof(ckq_block_q8_0) == CKQ_BLOCK_Q8_0_SIZE, "q8_0 size");
+CKQ_STATIC_ASSERT(sizeof(ckq_block_q5_0) == CKQ_BLOCK_Q5_0_SIZE, "q5_0 size");
 CKQ_STATIC_ASSERT(sizeof(ckq_block_q4_K) == CKQ_BLOCK_Q4_K_SIZE, "q4_K size");
 CKQ_STATIC_ASSERT(sizeof(ckq_block_q5_K) == CKQ_BLOCK_Q5_K_SIZE, "q5_K size");
 CKQ_STATIC_ASSERT(sizeof(ckq_block_q6_K) == CKQ_BLOCK_Q6_K_SIZE, "q6_K size");
@@ -101,12 +113,13 @@ typedef enum {
     CKQ_FMT_Q5_K = 1,
     CKQ_FMT_Q6_K = 2,
     CKQ_FMT_Q8_0 = 3,
-    CKQ_FMT_Q8_K = 4
+    CKQ_FMT_Q8_K = 4,
+    CKQ_FMT_Q5_0 = 5
 } ckq_format;
 
 static inline int ckq_block_elems(int fmt)
 {
-    return fmt == CKQ_FMT_Q8_0 ? CKQ_QK8_0 : CKQ_QK_K;
+    return (fmt == CKQ_FMT_Q8_0 || fmt == CKQ_FMT_Q5_0) ? CKQ_QK8_0 : CKQ_QK_K;
 }
 
 static inline size_t ckq_block_bytes(int fmt)
@@ -117,6 +130,7 @@ static inline size_t ckq_block_bytes(int fmt)
     case CKQ_FMT_Q6_K: return CKQ_BLOCK_Q6_K_SIZE;
     case CKQ_FMT_Q8_0: return CKQ_BLOCK_Q8_0_SIZE;
     case CKQ_FMT_Q8_K: return CKQ_BLOCK_Q8_K_SIZE;
+    case CKQ_FMT_Q5_0: return CKQ_BLOCK_Q5_0_SIZE;
     default: return 0;
     }
 }

@@ -1012,6 +1012,74 @@ void orc_gemm_nt_q8_0(const float *A, const void *B, const float *bias, float *C
 
 
 /* ------------------------------------------------------------------------ */
+/* Q5_0 x Q8_0                                                               */
+/* ------------------------------------------------------------------------ */
+
+/* value index l of a Q5_0 block, already minus 16 (gemm_kernels_q5_0.c:917-927) */
+static int q5_0_value(const ckq_block_q5_0 *b, int l)
+{
+    uint32_t qh;
+    memcpy(&qh, b->qh, 4);
+    const int nib = l < 16 ? (b->qs[l] & 0x0F) : (b->qs[l - 16] >> 4);
+    return (nib | (int)(((qh >> l) & 1u) << 4)) - 16;
+}
+
+static int32_t q5_0_block_dot(const ckq_block_q5_0 *w, const ckq_block_q8_0 *x)
+{
+    int32_t s = 0;
+    for (int l = 0; l < 32; ++l) s += (int32_t)q5_0_value(w, l) * (int32_t)x->qs[l];
+    return s;
+}
+
+void orc_subdots_q5_0_q8_0(const void *w_row, const void *x_q8, int K, int32_t *out)
+{
+    const ckq_block_q5_0 *w = (const ckq_block_q5_0 *)w_row;
+    const ckq_block_q8_0 *x = (const ckq_block_q8_0 *)x_q8;
+    for (int i = 0; i < K / CKQ_QK8_0; ++i) out[i] = q5_0_block_dot(&w[i], &x[i]);
+}
+
+void orc_vec_dot_q5_0_q8_0(int n, float *s, const void *vx, const void *vy)
+{
+    const ckq_block_q5_0 *w = (const ckq_block_q5_0 *)vx;
+    const ckq_block_q8_0 *x = (const ckq_block_q8_0 *)vy;
+    /* the reference's x86 builds enable FMA, which fuses this multiply-add
+     * (the golden test pins that choice bit for bit) */
+    float sumf = 0.0f;
+    for (int i = 0; i < n / CKQ_QK8_0; ++i)
+        sumf = fmaf(orc_fp16_to_fp32(w[i].d) * orc_fp16_to_fp32(x[i].d), (float)q5_0_block_dot(&w[i], &x[i]), sumf);
+    *s = sumf;
+}
+
+void orc_gemv_q5_0_q8_0(float *y, const void *W, const void *x_q8, int M, int K)
+{
+    if (!y || !W || !x_q8 || M <= 0 || K <= 0) return;
+    const size_t rb = (size_t)(K / CKQ_QK8_0) * sizeof(ckq_block_q5_0);
+    for (int r = 0; r < M; ++r) orc_vec_dot_q5_0_q8_0(K, &y[r], (const uint8_t *)W + (size_t)r * rb, x_q8);
+}
+
+void orc_gemm_nt_q5_0_q8_0(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K)
+{
+    if (!A_q8 || !B || !C || M <= 0 || N <= 0 || K <= 0) return;
+    const size_t wb = (size_t)(K / CKQ_QK8_0) * sizeof(ckq_block_q5_0), xb = (size_t)(K / CKQ_QK8_0) * sizeof(ckq_block_q8_0);
+    for (int m = 0; m < M; ++m)
+        for (int n = 0; n < N; ++n) {
+            float *out = &C[(size_t)m * N + n];
+            orc_vec_dot_q5_0_q8_0(K, out, (const uint8_t *)B + (size_t)n * wb, (const uint8_t *)A_q8 + (size_t)m * xb);
+            if (bias) *out += bias[n];
+        }
+}
+
+void orc_q5_0_to_q8_0(const void *src, void *dst, size_t nblocks)
+{
+    const ckq_block_q5_0 *s = (const ckq_block_q5_0 *)src;
+    ckq_block_q8_0 *d = (ckq_block_q8_0 *)dst;
+    for (size_t i = 0; i < nblocks; ++i) {
+        d[i].d = s[i].d;
+        for (int l = 0; l < 32; ++l) d[i].qs[l] = (int8_t)q5_0_value(&s[i], l);
+    }
+}
+
+/* ------------------------------------------------------------------------ */
 /* Fused prefill MLP                                                         */
 /* ------------------------------------------------------------------------ */
 
@@ -1043,14 +1111,14 @@ void orc_fused_mlp_swiglu_prefill_w1w2_quant(const float *x, const void *W1, con
                                              int intermediate_dim, int aligned_intermediate_dim,
                                              float *gate_up_out, void *h_q8k_out)
 {
-    enum { DT_Q4_K = 7, DT_Q6_K = 8, DT_Q8_0 = 9 };
+    enum { DT_Q4_K = 7, DT_Q6_K = 8, DT_Q8_0 = 9, DT_Q5_0 = 11 };
     if (!x || !W1 || !W2 || !output) return;
     if (seq_len <= 0 || embed_dim <= 0 || aligned_embed_dim <= 0 || intermediate_dim <= 0 ||
         aligned_intermediate_dim <= 0)
         return;
     if (aligned_embed_dim < embed_dim || aligned_intermediate_dim < intermediate_dim) return;
     if ((aligned_embed_dim % 32) != 0 || (aligned_intermediate_dim % 256) != 0) return;
-    if (w1_dt != DT_Q8_0 || (w2_dt != DT_Q4_K && w2_dt != DT_Q6_K)) return;
+    if ((w1_dt != DT_Q8_0 && w1_dt != DT_Q5_0) || (w2_dt != DT_Q4_K && w2_dt != DT_Q6_K)) return;
 
     const int E = aligned_embed_dim, I = aligned_intermediate_dim;
     const size_t q8_row = (size_t)(E / 32) * sizeof(ckq_block_q8_0);
@@ -1061,9 +1129,15 @@ void orc_fused_mlp_swiglu_prefill_w1w2_quant(const float *x, const void *W1, con
     uint8_t *hq = (uint8_t *)malloc((size_t)seq_len * q8k_row);
     if (xq && gate && up && hq) {
         for (int t = 0; t < seq_len; ++t) orc_quantize_row_q8_0(x + (size_t)t * E, xq + (size_t)t * q8_row, E);
-        const uint8_t *w_gate = (const uint8_t *)W1, *w_up = w_gate + (size_t)I * q8_row;
-        orc_gemm_nt_q8_0_q8_0(xq, w_gate, B1, gate, seq_len, I, E);
-        orc_gemm_nt_q8_0_q8_0(xq, w_up, B1 ? B1 + I : NULL, up, seq_len, I, E);
+        const size_t w1_row = w1_dt == DT_Q8_0 ? q8_row : (size_t)(E / 32) * sizeof(ckq_block_q5_0);
+        const uint8_t *w_gate = (const uint8_t *)W1, *w_up = w_gate + (size_t)I * w1_row;
+        if (w1_dt == DT_Q8_0) {
+            orc_gemm_nt_q8_0_q8_0(xq, w_gate, B1, gate, seq_len, I, E);
+            orc_gemm_nt_q8_0_q8_0(xq, w_up, B1 ? B1 + I : NULL, up, seq_len, I, E);
+        } else {
+            orc_gemm_nt_q5_0_q8_0(xq, w_gate, B1, gate, seq_len, I, E);
+            orc_gemm_nt_q5_0_q8_0(xq, w_up, B1 ? B1 + I : NULL, up, seq_len, I, E);
+        }
         orc_swiglu_q8_k(gate, up, hq, seq_len, I, I);
         if (gate_up_out)
             for (int t = 0; t < seq_len; ++t) {

@@ -88,11 +88,23 @@ void orc_gemm_q6_k(float *Y, const void *W, const float *X, int M, int N, int K)
 void orc_gemm_nt_q6_k(const float *A, const void *B, const float *bias, float *C, int M, int N, int K);            /* gemm_kernels_q6k.c:212-240 */
 void orc_gemm_nt_q8_0(const float *A, const void *B, const float *bias, float *C, int M, int N, int K);            /* gemm_kernels_q8_0.c:683-696 */
 
+/* ---- Q5_0 weights x Q8_0 activations ---------------------------------------
+ * per 32-block: sumi = sum (q5 - 16) * q8, sumf += (fp16(dw) * fp16(dx)) * sumi
+ * (gemm_kernels_q5_0.c:901-939; the SIMD dispatches sum the same terms in
+ * other orders).                                                            */
+void orc_subdots_q5_0_q8_0(const void *w_row, const void *x_q8, int K, int32_t *out);
+void orc_vec_dot_q5_0_q8_0(int n, float *s, const void *vx, const void *vy);                                       /* gemm_kernels_q5_0.c:1602-1620 */
+void orc_gemv_q5_0_q8_0(float *y, const void *W, const void *x_q8, int M, int K);                                  /* :1637-1657 */
+void orc_gemm_nt_q5_0_q8_0(const void *A_q8, const void *B, const float *bias, float *C, int M, int N, int K);     /* :1725-1753 */
+/* Q5_0 block -> the Q8_0 block with the same scale and the values q5 - 16:
+ * every dot product of the two is identical.                                */
+void orc_q5_0_to_q8_0(const void *src, void *dst, size_t nblocks);
+
 /* ---- fused prefill MLP ----------------------------------------------------
  * fused/prefill_fused_gemm.c:964-1060: Q8_0(x) x W1 (gate rows then up rows),
  * SiLU(gate)*up with the C library's expf, Q8_K of that, x W2.  w1_dt / w2_dt
- * are the reference's CKDataType values (Q8_0 = 9; Q4_K = 7, Q6_K = 8); other
- * types return without writing.  gate_up_out (seq_len x 2*aligned_intermediate
+ * are the reference's CKDataType values (W1: Q8_0 = 9 or Q5_0 = 11; W2: Q4_K = 7
+ * or Q6_K = 8); other types return without writing.  gate_up_out (seq_len x 2*aligned_intermediate
  * floats: gate, already multiplied, then up) and h_q8k_out receive the
  * intermediates when non-NULL.                                              */
 void orc_fused_mlp_swiglu_prefill_w1w2_quant(const float *x, const void *W1, const float *B1, int w1_dt,

@@ -12,9 +12,9 @@ ORACLE_DIR = os.path.join(ROOT, "oracle")
 CSRC = os.path.join(ROOT, "c-kernel-engine_amd", "csrc")
 GOLDEN = os.path.join(ROOT, "tests", "golden", "quant_path_golden.npz")
 
-FMT = {"q4_k": 0, "q5_k": 1, "q6_k": 2, "q8_0": 3, "q8_k": 4}
-BLK = {"q4_k": 144, "q5_k": 176, "q6_k": 210, "q8_0": 34, "q8_k": 292}
-ELEMS = {"q4_k": 256, "q5_k": 256, "q6_k": 256, "q8_0": 32, "q8_k": 256}
+FMT = {"q4_k": 0, "q5_k": 1, "q6_k": 2, "q8_0": 3, "q8_k": 4, "q5_0": 5}
+BLK = {"q4_k": 144, "q5_k": 176, "q6_k": 210, "q8_0": 34, "q8_k": 292, "q5_0": 22}
+ELEMS = {"q4_k": 256, "q5_k": 256, "q6_k": 256, "q8_0": 32, "q8_k": 256, "q5_0": 32}
 
 vp = ctypes.c_void_p
 
@@ -31,7 +31,7 @@ def row_bytes(fmt, k):
 
 
 def act_fmt(wfmt):
-    return "q8_0" if wfmt == "q8_0" else "q8_k"
+    return "q8_0" if wfmt in ("q8_0", "q5_0") else "q8_k"
 
 
 _cache = {}
@@ -108,11 +108,12 @@ def oracle_quantize(x, fmt="q8_k", rows=1):
 
 
 ORC_GEMV = {"q4_k": "orc_gemv_q4_k_q8_k", "q5_k": "orc_gemv_q5_k_q8_k",
-            "q6_k": "orc_gemv_q6_k_q8_k", "q8_0": "orc_gemv_q8_0_q8_0"}
+            "q6_k": "orc_gemv_q6_k_q8_k", "q8_0": "orc_gemv_q8_0_q8_0", "q5_0": "orc_gemv_q5_0_q8_0"}
 ORC_GEMM_NT = {"q4_k": "orc_gemm_nt_q4_k_q8_k", "q5_k": "orc_gemm_nt_q5_k_q8_k",
-               "q6_k": "orc_gemm_nt_q6_k_q8_k", "q8_0": "orc_gemm_nt_q8_0_q8_0"}
+               "q6_k": "orc_gemm_nt_q6_k_q8_k", "q8_0": "orc_gemm_nt_q8_0_q8_0", "q5_0": "orc_gemm_nt_q5_0_q8_0"}
 ORC_SUBDOTS = {"q4_k": ("orc_subdots_q4_k_q8_k", 8), "q5_k": ("orc_subdots_q5_k_q8_k", 8),
-               "q6_k": ("orc_subdots_q6_k_q8_k", 16), "q8_0": ("orc_subdots_q8_0_q8_0", 1)}
+               "q6_k": ("orc_subdots_q6_k_q8_k", 16), "q8_0": ("orc_subdots_q8_0_q8_0", 1),
+               "q5_0": ("orc_subdots_q5_0_q8_0", 1)}
 
 
 def oracle_gemv(fmt, W, xq, M, K, name=None):
@@ -137,11 +138,11 @@ def oracle_gemm_nt_f32act(fmt, A_f32, B, bias, M, N, K):
 CK_DT = {"q4_k": 7, "q6_k": 8, "q8_0": 9, "q8_k": 10, "q5_0": 11}   # the reference's CKDataType values
 
 
-def oracle_fused_mlp(x, W1, B1, W2, B2, w2_fmt, seq, embed, aembed, inter, ainter, want_intermediates=False):
+def oracle_fused_mlp(x, W1, B1, W2, B2, w2_fmt, seq, embed, aembed, inter, ainter, want_intermediates=False, w1_fmt="q8_0"):
     out = np.zeros(seq * aembed, dtype=np.float32)
     gu = np.zeros(seq * 2 * ainter, dtype=np.float32) if want_intermediates else None
     hq = np.zeros(seq * row_bytes("q8_k", ainter), dtype=np.uint8) if want_intermediates else None
-    oracle().orc_fused_mlp_swiglu_prefill_w1w2_quant(ptr(x), ptr(W1), ptr(B1), CK_DT["q8_0"], ptr(W2), ptr(B2),
+    oracle().orc_fused_mlp_swiglu_prefill_w1w2_quant(ptr(x), ptr(W1), ptr(B1), CK_DT[w1_fmt], ptr(W2), ptr(B2),
                                                      CK_DT[w2_fmt], ptr(out), seq, embed, aembed, inter, ainter,
                                                      ptr(gu), ptr(hq))
     out = out.reshape(seq, aembed)
@@ -228,6 +229,17 @@ def np_decode_q8_0(w):
     return dict(d=_f16(b[:, 0:2]).reshape(-1), q=b[:, 2:34].view(np.int8).astype(np.int32))
 
 
+def np_decode_q5_0(w):
+    """From the format definition: element l < 16 = low nibble of qs[l] | bit l of
+    qh << 4, element 16 + l = high nibble | bit 16 + l << 4; value = q - 16."""
+    b = w.reshape(-1, 22)
+    qh = np.ascontiguousarray(b[:, 2:6]).view(np.uint32).reshape(-1).astype(np.int64)
+    qs = b[:, 6:22].astype(np.int32)
+    bits = ((qh[:, None] >> np.arange(32)[None, :]) & 1).astype(np.int32)
+    q = np.concatenate([qs & 15, qs >> 4], axis=1) | (bits << 4)
+    return dict(d=_f16(b[:, 0:2]).reshape(-1), q=q - 16)
+
+
 def np_decode_q8_k(x):
     b = x.reshape(-1, 292)
     return dict(d=np.ascontiguousarray(b[:, 0:4]).view(np.float32).reshape(-1),
@@ -247,8 +259,8 @@ def np_dequant(fmt, w):
         b = np_decode_q6_k(w)
         q = b["q"].reshape(-1, 16, 16).astype(np.float64)
         return (b["d"][:, None, None].astype(np.float64) * b["sc"][:, :, None] * q).reshape(-1)
-    if fmt == "q8_0":
-        b = np_decode_q8_0(w)
+    if fmt in ("q8_0", "q5_0"):
+        b = np_decode_q8_0(w) if fmt == "q8_0" else np_decode_q5_0(w)
         return (b["d"][:, None].astype(np.float64) * b["q"]).reshape(-1)
     if fmt == "q8_k":
         b = np_decode_q8_k(w)
@@ -258,8 +270,8 @@ def np_dequant(fmt, w):
 
 def np_subdots(fmt, W, xq, M, K):
     """Brute-force integer sub-block dots, [M, nsub]."""
-    if fmt == "q8_0":
-        wq = np_decode_q8_0(W)["q"].reshape(M, K // 32, 32)
+    if fmt in ("q8_0", "q5_0"):
+        wq = (np_decode_q8_0(W) if fmt == "q8_0" else np_decode_q5_0(W))["q"].reshape(M, K // 32, 32)
         xv = np_decode_q8_0(xq)["q"].reshape(K // 32, 32)
         return (wq * xv[None]).sum(axis=2).astype(np.int32)
     xv = np_decode_q8_k(xq)["q"].reshape(K // 256, 256)

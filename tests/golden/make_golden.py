@@ -25,9 +25,9 @@ REFDIR = os.path.join(ROOT, "oracle", "_ref")
 SYNTH = os.path.join(ROOT, "c-kernel-engine_amd", "csrc", "libckq_synth.so")
 OUT = os.path.join(ROOT, "tests", "golden", "quant_path_golden.npz")
 
-FMT = {"q4_k": 0, "q5_k": 1, "q6_k": 2, "q8_0": 3, "q8_k": 4}
-BLK = {"q4_k": 144, "q5_k": 176, "q6_k": 210, "q8_0": 34, "q8_k": 292}
-ELEMS = {"q4_k": 256, "q5_k": 256, "q6_k": 256, "q8_0": 32, "q8_k": 256}
+FMT = {"q4_k": 0, "q5_k": 1, "q6_k": 2, "q8_0": 3, "q8_k": 4, "q5_0": 5}
+BLK = {"q4_k": 144, "q5_k": 176, "q6_k": 210, "q8_0": 34, "q8_k": 292, "q5_0": 22}
+ELEMS = {"q4_k": 256, "q5_k": 256, "q6_k": 256, "q8_0": 32, "q8_k": 256, "q5_0": 32}
 
 c_f32p = ctypes.POINTER(ctypes.c_float)
 vp = ctypes.c_void_p
@@ -230,6 +230,24 @@ def main():
                 run(libs["avx2"], "vec_dot_q8_0_q8_0", K, ptr(s), ptr(w), ptr(act))
                 G["s_q8_0_%s_vecdot" % kind] = s
 
+    # ---- Q5_0 weights x Q8_0 activations (the fallback format of rows K-quants cannot hold) ----
+    for kind in ("rand", "enc"):
+        w = random_blocks(S, "q5_0", ROWS * (K // 32), 450) if kind == "rand" else synth_weights(S, "q5_0", ROWS, K, 550)
+        G["w_q5_0_" + kind] = w
+        for tag, L in libs.items():
+            y = np.zeros(ROWS, np.float32)
+            run(L, "gemv_q5_0_q8_0", ptr(y), ptr(w), ptr(xq80), ROWS, K)
+            G["y_q5_0_%s_%s" % (kind, tag)] = y
+            c = np.zeros(TOK * ROWS, np.float32)
+            run(L, "gemm_nt_q5_0_q8_0", ptr(xq80), ptr(w), ptr(bias), ptr(c), TOK, ROWS, K)
+            G["c_q5_0_%s_%s" % (kind, tag)] = c
+        sv = np.zeros(1, np.float32)
+        run(libs["avx2"], "vec_dot_q5_0_q8_0", K, ptr(sv), ptr(w), ptr(xq80))
+        G["s_q5_0_%s_vecdot" % kind] = sv
+        sv = np.zeros(1, np.float32)
+        run(libs["avx2"], "vec_dot_q5_0_q8_0_ref", K, ptr(sv), ptr(w), ptr(xq80))
+        G["s_q5_0_%s_vecdot_ref" % kind] = sv
+
     # ---- fused producer rmsnorm -> Q8_K (both builds must agree: integer output) ----
     TF, DF, AF = 3, 768, 800                       # row stride larger than d_model
     xr = normal(S, TF * AF, 0.0, 1.5, 601)
@@ -288,6 +306,18 @@ def main():
                                                   ptr(o), SEQ, ED2, AED2, ID2, AID2, ptr(scr))
             G["mlp_out_%s_%s" % (fmt, tag)] = o
         G["mlp_scratch_size"] = np.array([len(scr)], np.int64)
+    # the same with the gate/up matrix in Q5_0
+    w1q5 = synth_weights(S, "q5_0", 2 * AID2, AED2, 812)
+    w1v = w1q5.reshape(-1, 22)
+    d16 = w1v[:, 0:2].copy().view(np.float16).astype(np.float32) * 12.0
+    w1v[:, 0:2] = d16.astype(np.float16).view(np.uint8)
+    G["mlp_w1_q5_0"] = w1q5
+    for tag, L in libs.items():
+        scr = np.zeros(L.fused_mlp_swiglu_prefill_w1w2_quant_scratch_size(AED2, AID2), np.uint8)
+        o = np.zeros(SEQ * AED2, np.float32)
+        L.fused_mlp_swiglu_prefill_w1w2_quant(ptr(xm), ptr(w1q5), ptr(b1), 11, ptr(G["mlp_w2_q4_k"]), ptr(b2), DT["q4_k"],
+                                              ptr(o), SEQ, ED2, AED2, ID2, AID2, ptr(scr))
+        G["mlp_out_q5_0w1_q4_k_%s" % tag] = o
 
     np.savez_compressed(OUT, **G)
     print("wrote %s: %d arrays, %.1f KiB" % (OUT, len(G), os.path.getsize(OUT) / 1024.0))

@@ -707,22 +707,6 @@ def test_fused_mlp_argument_errors_leave_output_untouched():
     P.fused_mlp_swiglu_prefill_w1w2_quant(x, w1, None, "q8_0", w2, None, "q4_k", SEQ, ED, AED, ID, AID, output=out,
                                           scratch=False)
     assert np.all(out == 7.0)
-    # Q5_0 for W1 is a format this library does not build: reported, never computed silently wrong
-    import os
-    old = os.environ.get("CKQ_ABORT_ON_ERROR")
-    os.environ["CKQ_ABORT_ON_ERROR"] = "0"
-    try:
-        out = mk()
-        P.fused_mlp_swiglu_prefill_w1w2_quant(x, w1, None, "q5_0", w2, None, "q4_k", SEQ, ED, AED, ID, AID, output=out)
-        assert np.all(out == 7.0)
-        assert ckq.lib().ckq_last_error() == -3
-        ckq.lib().ckq_clear_error()
-        assert ckq.lib().ckq_last_error() == 0
-    finally:
-        if old is None:
-            del os.environ["CKQ_ABORT_ON_ERROR"]
-        else:
-            os.environ["CKQ_ABORT_ON_ERROR"] = old
     assert int(ckq.lib().fused_mlp_swiglu_prefill_w1w2_quant_scratch_size(AED, AID)) == int(G["mlp_scratch_size"][0])
 
 
@@ -953,3 +937,70 @@ def test_gemm_mfma_random_shapes(fmt):
         c = c_d.cpu().numpy().reshape(M, ldc)
         assert T.norm_err(c[:, :N], ref) <= TOL, (fmt, M, N, K, ldc)
         assert np.all(c[:, N:] == 3.0), (fmt, M, N, K, ldc)         # nothing written beyond a row's N outputs
+
+
+# ---- Q5_0 weights x Q8_0 activations ------------------------------------------------------------
+
+def test_q5_0_subblock_dots_and_gemv_k_sweep():
+    rows = 41
+    for K in (32, 128, 512, 896, 1024, 2048, 4096, 8192, 10240):
+        for kind in ("rand", "enc"):
+            W, _, xq = make_case("q5_0", rows, K, kind, 60 + K)
+            say("q5_0", kind, "rows", rows, "K", K)
+            W_d, xq_d = P.to_device(W), P.to_device(xq)
+            got = P.dev_subblock_dots("q5_0", W_d, xq_d, rows, K).cpu().numpy()
+            assert np.array_equal(got, T.oracle_subdots("q5_0", W, xq, rows, K)), K
+            y = P.dev_gemm_nt("q5_0", xq_d, W_d, None, 1, rows, K).cpu().numpy().reshape(-1)
+            assert T.norm_err(y, T.oracle_gemv("q5_0", W, xq, rows, K)) <= TOL, (K, kind)
+
+
+@pytest.mark.parametrize("kind", ["rand", "enc"])
+def test_q5_0_golden_fixture(kind):
+    G = T.golden()
+    M, K, TOK = (int(v) for v in G["shape"])
+    W, xq = G["w_q5_0_" + kind], G["act_q80"]
+    say("q5_0 golden", kind)
+    y = P.gemv("q5_0", W, xq, M, K)
+    c = P.gemm_nt("q5_0", xq, W, G["bias"], TOK, M, K)
+    for build in ("avx2", "avx512"):
+        assert T.norm_err(y, G["y_q5_0_%s_%s" % (kind, build)]) <= TOL
+        assert T.norm_err(c, G["c_q5_0_%s_%s" % (kind, build)].reshape(TOK, M)) <= TOL
+    s = np.zeros(1, np.float32)
+    ckq.lib().vec_dot_q5_0_q8_0(K, T.ptr(s), T.ptr(W), T.ptr(xq))
+    assert abs(float(s[0]) - float(G["s_q5_0_%s_vecdot" % kind][0])) <= TOL * np.abs(y).max()
+    yp = np.zeros(M, np.float32)
+    for ith in range(5):
+        ckq.lib().gemv_q5_0_q8_0_parallel_simd(T.ptr(yp), T.ptr(W), T.ptr(xq), M, K, ith, 5)
+    assert np.array_equal(yp, y)
+
+
+def test_q5_0_row_and_token_counts():
+    """Token tiles up to 16 tokens; above that the blocks are rewritten as Q8_0
+    blocks and the Q8_0 matrix-core GEMM runs: the same bits as that GEMM on
+    weights converted by the oracle."""
+    K = 896
+    for rows in (1, 3, 17, 64, 65, 257):
+        W, _, xq = make_case("q5_0", rows, K, "rand", 11 * rows)
+        say("q5_0 rows", rows)
+        assert T.norm_err(P.gemv("q5_0", W, xq, rows, K), T.oracle_gemv("q5_0", W, xq, rows, K)) <= TOL, rows
+    N = 77
+    bias = T.normal(N, 0.0, 0.5, seed=8)
+    for M in (1, 2, 5, 8, 9, 16, 17, 33, 130, 512):
+        W, _, xq = make_case("q5_0", N, K, "enc", 310 + M, tokens=M)
+        say("q5_0 gemm_nt tokens", M)
+        ref = T.oracle_gemm_nt("q5_0", xq, W, bias, M, N, K)
+        c = P.gemm_nt("q5_0", xq, W, bias, M, N, K)
+        assert T.norm_err(c, ref) <= TOL, M
+        if M > 16:
+            w8 = np.zeros(len(W) // 22 * 34, np.uint8)
+            T.oracle().orc_q5_0_to_q8_0(T.ptr(W), T.ptr(w8), ctypes.c_size_t(len(W) // 22))
+            assert np.array_equal(P.gemm_nt("q8_0", xq, w8, bias, M, N, K), c), M
+
+
+def test_fused_mlp_q5_0_gate_up_golden_case():
+    G = T.golden()
+    SEQ, ED, AED, ID, AID = (int(v) for v in G["mlp_shape"])
+    say("fused mlp q5_0 gate/up golden")
+    got = P.fused_mlp_swiglu_prefill_w1w2_quant(G["mlp_x"], G["mlp_w1_q5_0"], G["mlp_b1"], "q5_0", G["mlp_w2_q4_k"],
+                                                G["mlp_b2"], "q4_k", SEQ, ED, AED, ID, AID)
+    assert T.norm_err(got, G["mlp_out_q5_0w1_q4_k_avx2"].reshape(SEQ, AED)) <= TOL

@@ -366,6 +366,52 @@ def test_embedding_forward_bit_exact_vs_reference(fmt, add_pos):
     assert np.all(o[NTOK:] == 0.0)
 
 
+# ---- Q5_0 weights x Q8_0 activations ------------------------------------------------------------
+
+@pytest.mark.parametrize("kind", ["rand", "enc"])
+def test_q5_0_q8_0_vs_reference(kind):
+    """gemv / gemm_nt / vec_dot of both reference builds within the summation-order
+    tolerance; the scalar _ref routine (the order restated here) bit for bit; the
+    integer block dots against a NumPy decoder written from the format definition;
+    and the Q5_0 -> Q8_0 block conversion, under which every dot is unchanged."""
+    G = T.golden()
+    O = T.oracle()
+    ROWS, K, TOK = (int(v) for v in G["shape"])
+    W, xq, bias = G["w_q5_0_" + kind], G["act_q80"], G["bias"]
+    y = T.oracle_gemv("q5_0", W, xq, ROWS, K)
+    c = T.oracle_gemm_nt("q5_0", xq, W, bias, TOK, ROWS, K)
+    for tag in ("avx2", "avx512"):
+        assert T.norm_err(y, G["y_q5_0_%s_%s" % (kind, tag)]) <= 2e-6
+        assert T.norm_err(c, G["c_q5_0_%s_%s" % (kind, tag)].reshape(TOK, ROWS)) <= 2e-6
+    s = np.zeros(1, np.float32)
+    O.orc_vec_dot_q5_0_q8_0(K, ptr(s), ptr(W), ptr(xq))
+    assert s.view(np.uint32)[0] == G["s_q5_0_%s_vecdot_ref" % kind].view(np.uint32)[0]
+    assert abs(float(s[0]) - float(G["s_q5_0_%s_vecdot" % kind][0])) <= 2e-6 * np.abs(y).max()
+    # integers, from the format definition
+    x0 = xq[:T.row_bytes("q8_0", K)].copy()
+    sub = T.oracle_subdots("q5_0", W, x0, ROWS, K)
+    assert np.array_equal(sub, T.np_subdots("q5_0", W, x0, ROWS, K))
+    # closed form of the row sums in float64
+    wv = T.np_dequant("q5_0", W).reshape(ROWS, K)
+    xv = T.np_dequant("q8_0", xq).reshape(TOK, K)
+    assert np.allclose(y, wv @ xv[0], rtol=0, atol=2e-6 * np.abs(y).max())
+    # conversion to Q8_0 blocks keeps every value and scale
+    w8 = np.zeros(len(W) // 22 * 34, np.uint8)
+    O.orc_q5_0_to_q8_0(ptr(W), ptr(w8), ctypes.c_size_t(len(W) // 22))
+    assert np.array_equal(T.np_dequant("q8_0", w8), T.np_dequant("q5_0", W))
+    assert np.array_equal(T.oracle_subdots("q8_0", w8, x0, ROWS, K), sub)
+    assert T.norm_err(T.oracle_gemv("q8_0", w8, xq, ROWS, K), y) <= 2e-6
+
+
+def test_fused_mlp_q5_0_gate_up_vs_reference():
+    G = T.golden()
+    SEQ, ED, AED, ID, AID = (int(v) for v in G["mlp_shape"])
+    out = T.oracle_fused_mlp(G["mlp_x"], G["mlp_w1_q5_0"], G["mlp_b1"], G["mlp_w2_q4_k"], G["mlp_b2"], "q4_k",
+                             SEQ, ED, AED, ID, AID, w1_fmt="q5_0")
+    for tag in ("avx2", "avx512"):
+        assert T.norm_err(out, G["mlp_out_q5_0w1_q4_k_%s" % tag].reshape(SEQ, AED)) <= 2e-6, tag
+
+
 # ---- fused prefill MLP ----------------------------------------------------------------------
 
 @pytest.mark.parametrize("fmt", ["q4_k", "q6_k"])
