@@ -47,7 +47,7 @@ __device__ __forceinline__ void k4_scale_pair(u32 u0, u32 u1, u32 u2, int g, u32
 /* ------------------------------------------------------------------------- */
 struct FmtQ4K {
     static constexpr int POS_PER_BLOCK = 4, WBLOCK = 144, XBLOCK = 292, NSUB = 2;
-    static constexpr int OCC1 = 8;            /* waves per SIMD the one-token kernel is held to */
+    static constexpr int OCC1 = 8, OCC2 = 6;   /* waves per SIMD the one-token kernel is held to: one row, two rows per wave */
     static constexpr bool TOKEN_TILES = true; /* tiles of 2, 4 and 8 tokens exist */
     struct Wt  { u32 hdr[4]; u32 qs[8]; };
     struct Act { int q[16]; float d; int b_lo, b_hi; };
@@ -127,7 +127,7 @@ struct FmtQ4K {
 /* ------------------------------------------------------------------------- */
 struct FmtQ5K {
     static constexpr int POS_PER_BLOCK = 4, WBLOCK = 176, XBLOCK = 292, NSUB = 2;
-    static constexpr int OCC1 = 8;            /* waves per SIMD the one-token kernel is held to */
+    static constexpr int OCC1 = 8, OCC2 = 5;            /* waves per SIMD the one-token kernel is held to */
     static constexpr bool TOKEN_TILES = true; /* tiles of 2, 4 and 8 tokens exist */
     struct Wt  { u32 hdr[4]; u32 qh[8]; u32 qs[8]; };
     typedef FmtQ4K::Act Act;
@@ -189,7 +189,7 @@ struct FmtQ5K {
 /* ------------------------------------------------------------------------- */
 struct FmtQ6K {
     static constexpr int POS_PER_BLOCK = 4, WBLOCK = 210, XBLOCK = 292, NSUB = 4;
-    static constexpr int OCC1 = 8;            /* waves per SIMD the one-token kernel is held to */
+    static constexpr int OCC1 = 8, OCC2 = 6;   /* waves per SIMD the one-token kernel is held to: one row, two rows per wave */
     static constexpr bool TOKEN_TILES = true; /* tiles of 2, 4 and 8 tokens exist */
     struct Wt  { u32 ql0[4], ql1[4], qh[4]; u32 sc[2]; u32 d; };
     struct Act { int q[16]; float d; int a32[4]; };      /* a32[r] = 32 * sum of the run's 16 quants */
@@ -282,7 +282,7 @@ struct FmtQ6K {
 /* ------------------------------------------------------------------------- */
 struct FmtQ80 {
     static constexpr int POS_PER_BLOCK = 1, WBLOCK = 34, XBLOCK = 34, NSUB = 1;
-    static constexpr int OCC1 = 8;            /* waves per SIMD the one-token kernel is held to */
+    static constexpr int OCC1 = 8, OCC2 = 6;   /* waves per SIMD the one-token kernel is held to: one row, two rows per wave */
     static constexpr bool TOKEN_TILES = true; /* tiles of 2, 4 and 8 tokens exist */
     struct Wt  { u32 q[8]; u32 d; };
     struct Act { int q[8]; float d; };
@@ -389,7 +389,7 @@ struct FmtQ50 : FmtQ80 {
 /* Q8_0 weights against fp32 activations (no activation quantization). */
 struct FmtQ80F32 {
     static constexpr int POS_PER_BLOCK = 1, WBLOCK = 34, XBLOCK = 128, NSUB = 1;
-    static constexpr int OCC1 = 4;            /* 64 activation floats per lane: 128 registers */
+    static constexpr int OCC1 = 4, OCC2 = 1;            /* 64 activation floats per lane: 128 registers */
     static constexpr bool TOKEN_TILES = false;
     typedef FmtQ80::Wt Wt;
     typedef FmtQ80::Dec Dec;
@@ -444,7 +444,7 @@ struct FmtQ80F32 {
  * sum (d*sc*q - dmin*m) * x (reference: gemm_kernels_q4k.c:53-101). */
 struct FmtQ4KF32 {
     static constexpr int POS_PER_BLOCK = 4, WBLOCK = 144, XBLOCK = 1024, NSUB = 1;
-    static constexpr int OCC1 = 4;            /* 64 activation floats per lane: 128 registers */
+    static constexpr int OCC1 = 4, OCC2 = 1;            /* 64 activation floats per lane: 128 registers */
     static constexpr bool TOKEN_TILES = false;
     typedef FmtQ4K::Wt Wt;
     typedef FmtQ4K::Dec Dec;
@@ -504,7 +504,7 @@ struct FmtQ4KF32 {
  * (reference: gemm_kernels_q6k.c:39-76). */
 struct FmtQ6KF32 {
     static constexpr int POS_PER_BLOCK = 4, WBLOCK = 210, XBLOCK = 1024, NSUB = 1;
-    static constexpr int OCC1 = 4;            /* 64 activation floats per lane: 128 registers */
+    static constexpr int OCC1 = 4, OCC2 = 1;            /* 64 activation floats per lane: 128 registers */
     static constexpr bool TOKEN_TILES = false;
     typedef FmtQ6K::Wt Wt;
     typedef FmtQ6K::Dec Dec;

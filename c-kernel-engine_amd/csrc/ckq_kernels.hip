@@ -62,7 +62,7 @@ __device__ __forceinline__ int wave_in_block() { return __builtin_amdgcn_readfir
  * stores.
  */
 template <class F, int LPR, int PPL, int MT, int RPI, bool DUMP, int WPB, bool LDSX>
-__global__ void __launch_bounds__(64 * WPB) __attribute__((amdgpu_waves_per_eu(MT == 1 && !DUMP && PPL == 1 && RPI == 1 ? F::OCC1 : MT >= 4 && PPL == 1 ? 4 : 1)))
+__global__ void __launch_bounds__(64 * WPB) __attribute__((amdgpu_waves_per_eu(MT == 1 && !DUMP && PPL == 1 && RPI == 1 ? F::OCC1 : MT == 1 && !DUMP && PPL == 1 && RPI == 2 && LPR == 64 ? F::OCC2 : MT >= 4 && PPL == 1 ? 4 : 1)))
 gemv_kernel(GemvArgs a)
 {
     constexpr int SLOTS = 64 / LPR;
