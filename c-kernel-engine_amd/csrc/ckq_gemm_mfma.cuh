@@ -62,12 +62,17 @@ struct GemmArgs {
     float *part;
 };
 
-/* Where a block of a (possibly K-split) GEMM writes, and whether it adds the bias. */
+/* What one block of a GEMM launch does: which tile id, which K-steps, where it
+ * writes and whether it adds the bias. */
 struct GemmOut { float *C; long ldc; const float *bias; };
-__device__ __forceinline__ GemmOut gemm_out(const GemmArgs &a)
+struct GemmWork { int id, k0, k1; GemmOut out; };
+__device__ __forceinline__ GemmWork gemm_work(const GemmArgs &a, int k_steps)
 {
-    if (a.splits <= 1) return {a.C, a.ldc, a.bias};
-    return {a.part + (size_t)blockIdx.y * (size_t)a.M * (size_t)a.N, (long)a.N, nullptr};
+    const int id = blockIdx.x;
+    if (a.splits <= 1) return {id, 0, k_steps, {a.C, a.ldc, a.bias}};
+    const int k0 = (int)blockIdx.y * a.k_per;
+    return {id, k0, min(k_steps, k0 + a.k_per),
+            {a.part + (size_t)blockIdx.y * (size_t)a.M * (size_t)a.N, (long)a.N, nullptr}};
 }
 
 /* C = bias + partial 0 + partial 1 + ... in that order: the result does not
@@ -102,6 +107,7 @@ static int gemm_choose_splits(int tiles, int k_steps)
  * caller holds g_split_mu from here until the reduction is enqueued, so two
  * host threads launching on one stream cannot interleave their kernel pairs. */
 #include <mutex>
+constexpr int GEMM_TILE_ROWS = 128;    /* weight rows per tile, all four kernels */
 static std::recursive_mutex g_split_mu;
 /* kind 0: partial tiles of a K split; kind 1: weights rewritten for another kernel */
 static int gemm_workspace(int kind, hipStream_t s, size_t bytes, float **out)
@@ -166,7 +172,7 @@ __device__ __forceinline__ int mul_bytes(u32 v, u32 s16x2)
 __device__ __forceinline__ u32 bf16_bits(float f) { return __builtin_bit_cast(u32, f) >> 16; }
 
 constexpr int GEMM_BM = 64;     /* tokens per tile */
-constexpr int GEMM_BN = 128;    /* weight rows per tile */
+constexpr int GEMM_BN = GEMM_TILE_ROWS;    /* weight rows per tile */
 
 /* LDS image of one 256-block for a tile of 128 weight rows x 64 tokens. */
 struct GemmStage {
@@ -310,14 +316,14 @@ __global__ void __launch_bounds__(256 * KG, KG == 2 ? 1 : WPE) gemm_q4k_mfma_ker
     const int col = lane & 31, half = lane >> 5;
     GemmStage *const stage = stage_all[grp];
 
-    const int id = blockIdx.x, xcd = id & 7, seq = id >> 3;
+    const GemmWork work = gemm_work(a, a.nb);
+    const int id = work.id, xcd = id & 7, seq = id >> 3;
     const int tt = seq % a.ntt;
     const int nt = (seq / a.ntt) * 8 + xcd;
     if (nt >= a.nnt) return;
     const int t0 = tt * BM, n0 = nt * GEMM_BN;
     const u32 wstride = (u32)a.nb * 144u, xstride = (u32)a.nb * 292u;
-    const int b0 = a.splits > 1 ? (int)blockIdx.y * a.k_per : 0;
-    const int b1 = a.splits > 1 ? min(a.nb, b0 + a.k_per) : a.nb, last = b1 - 1;
+    const int b0 = work.k0, b1 = work.k1, last = b1 - 1;
     const uint8_t *wbase = a.B + (size_t)n0 * wstride;       /* uniform */
     const uint8_t *xbase = a.A + (size_t)t0 * xstride;       /* uniform */
 
@@ -427,7 +433,7 @@ __global__ void __launch_bounds__(256 * KG, KG == 2 ? 1 : WPE) gemm_q4k_mfma_ker
             for (int r = 0; r < 16; ++r) acc[ts][r] += red[(ts * 16 + r) * 256 + tid];
     }
 
-    const GemmOut o = gemm_out(a);
+    const GemmOut o = work.out;
     const int n = n0 + wave * 32 + col;
     if (n < a.N) {
         const float bias = o.bias ? o.bias[n] : 0.0f;

@@ -180,14 +180,14 @@ __global__ void __launch_bounds__(256, 1) gemm_q5k_mfma_kernel(GemmArgs a)
     const int col = lane & 31, half = lane >> 5;
 
     /* token tiles fastest inside an XCD, so each XCD's L2 sees a weight tile once */
-    const int id = blockIdx.x, xcd = id & 7, seq = id >> 3;
+    const GemmWork work = gemm_work(a, a.nb);
+    const int id = work.id, xcd = id & 7, seq = id >> 3;
     const int tt = seq % a.ntt;
     const int nt = (seq / a.ntt) * 8 + xcd;
     if (nt >= a.nnt) return;
     const int t0 = tt * BM, n0 = nt * GEMM5_BN;
     const u32 wstride = (u32)a.nb * 176u, xstride = (u32)a.nb * 292u;
-    const int b0 = a.splits > 1 ? (int)blockIdx.y * a.k_per : 0;
-    const int b1 = a.splits > 1 ? min(a.nb, b0 + a.k_per) : a.nb, last = b1 - 1;
+    const int b0 = work.k0, b1 = work.k1, last = b1 - 1;
     const uint8_t *wbase = a.B + (size_t)n0 * wstride;       /* uniform */
     const uint8_t *xbase = a.A + (size_t)t0 * xstride;       /* uniform */
 
@@ -272,7 +272,7 @@ __global__ void __launch_bounds__(256, 1) gemm_q5k_mfma_kernel(GemmArgs a)
         pf = pf + 1 == NST ? 0 : pf + 1;
     }
 
-    const GemmOut o = gemm_out(a);
+    const GemmOut o = work.out;
     const int n = n0 + wave * 32 + col;
     if (n < a.N) {
         const float bias = o.bias ? o.bias[n] : 0.0f;

@@ -61,16 +61,15 @@ __global__ void __launch_bounds__(256, 2) gemm_q80_mfma_kernel(GemmArgs a)
     const int col = lane & 31, half = lane >> 5;
 
     /* token tiles fastest inside an XCD, so each XCD's L2 sees a weight tile once */
-    const int id = blockIdx.x, xcd = id & 7, seq = id >> 3;
+    const GemmWork work = gemm_work(a, (a.nb + KB - 1) / KB);
+    const int id = work.id, xcd = id & 7, seq = id >> 3;
     const int tt = seq % a.ntt;
     const int nt = (seq / a.ntt) * 8 + xcd;
     if (nt >= a.nnt) return;
     const int t0 = tt * BM, n0 = nt * BN;
     const int nblk = a.nb;                                  /* 32-blocks per row */
     const u32 stride = (u32)nblk * 34u;                     /* bytes per weight row and per activation row */
-    const int niter_all = (nblk + KB - 1) / KB;
-    const int it0 = a.splits > 1 ? (int)blockIdx.y * a.k_per : 0;
-    const int niter = a.splits > 1 ? min(niter_all, it0 + a.k_per) : niter_all;   /* this block runs iterations [it0, niter) */
+    const int it0 = work.k0, niter = work.k1;               /* this block runs iterations [it0, niter) */
     const uint8_t *wbase = a.B + (size_t)n0 * stride;       /* uniform */
     const uint8_t *xbase = a.A + (size_t)t0 * stride;       /* uniform */
 
@@ -212,7 +211,7 @@ __global__ void __launch_bounds__(256, 2) gemm_q80_mfma_kernel(GemmArgs a)
     }
 
     /* lane: token t0 + col + 32 ts, rows n0 + 32 wave + 8 q + 4 half + (0..3) */
-    const GemmOut o = gemm_out(a);
+    const GemmOut o = work.out;
     const bool vec_ok = (o.ldc % 4 == 0) && (((uintptr_t)o.C) % 16 == 0) && (n0 + BN <= a.N);
 #pragma unroll
     for (int ts = 0; ts < 2; ++ts) {

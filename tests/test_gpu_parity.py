@@ -503,20 +503,51 @@ def test_gemm_mfma_full_prefill_shape():
     M, N, K = 512, 11008, 4096
     W = T.synth_weights("q4_k", N, K, seed=5150)
     xf = T.normal(M * K, 0.0, 1.0, seed=5151)
+    bias = T.normal(N, 0.0, 0.5, seed=5152)
     say("gemm mfma full prefill shape")
     xq_d = P.dev_quantize(P.to_device(xf), "q8_k", rows=M)
     xq = xq_d.cpu().numpy()
-    Wd = P.to_device(W)
-    c = P.dev_gemm_nt("q4_k", xq_d, Wd, None, M, N, K).cpu().numpy()
+    Wd, bd = P.to_device(W), P.to_device(bias)
+    c = P.dev_gemm_nt("q4_k", xq_d, Wd, bd, M, N, K).cpu().numpy()
     rb = T.row_bytes("q4_k", K)
-    rows = np.array([0, 1, 31, 32, 127, 128, 5000, 5503, 5504, 11006, 11007])
+    rows = np.array([0, 1, 31, 32, 127, 128, 5000, 5503, 5504, 8191, 8192, 9000, 11006, 11007])
     Wsub = np.ascontiguousarray(W.reshape(N, rb)[rows]).reshape(-1)
-    ref = T.oracle_gemm_nt("q4_k", xq, Wsub, None, M, len(rows), K)
+    ref = T.oracle_gemm_nt("q4_k", xq, Wsub, np.ascontiguousarray(bias[rows]), M, len(rows), K)
     assert T.norm_err(c[:, rows], ref) <= TOL
     ab = T.row_bytes("q8_k", K)
     for t in (0, 63, 64, 300, 511):
-        y = P.dev_gemm_nt("q4_k", P.to_device(xq[t * ab:(t + 1) * ab].copy()), Wd, None, 1, N, K).cpu().numpy().reshape(-1)
+        y = P.dev_gemm_nt("q4_k", P.to_device(xq[t * ab:(t + 1) * ab].copy()), Wd, bd, 1, N, K).cpu().numpy().reshape(-1)
         assert T.norm_err(c[t], y) <= 2e-6, t
+    assert np.array_equal(P.dev_gemm_nt("q4_k", xq_d, Wd, bd, M, N, K).cpu().numpy(), c)
+
+
+@pytest.mark.parametrize("fmt", ["q4_k", "q6_k"])
+def test_gemm_mfma_more_tiles_than_block_slots(fmt):
+    """A ragged grid larger than the chip holds at once (549 tiles of 64 tokens
+    x 128 rows for Q4_K, nine K-blocks), with a bias: blocks of a second round
+    start while others still run.  Oracle on weight rows spread over the row
+    tiles for every token, whole rows against the GEMV kernel for a few tokens,
+    same bits on a second run."""
+    M, N, K = 520, 7700, 2304
+    W = T.synth_weights(fmt, N, K, seed=5350)
+    xf = T.normal(M * K, 0.0, 1.0, seed=5351)
+    bias = T.normal(N, 0.0, 0.5, seed=5352)
+    say("gemm mfma more tiles than slots", fmt)
+    af = P.act_format(fmt)
+    xq_d = P.dev_quantize(P.to_device(xf), af, rows=M)
+    xq = xq_d.cpu().numpy()
+    Wd, bd = P.to_device(W), P.to_device(bias)
+    c = P.dev_gemm_nt(fmt, xq_d, Wd, bd, M, N, K).cpu().numpy()
+    rb = T.row_bytes(fmt, K)
+    rows = np.array([0, 127, 128, 3583, 3584, 7039, 7040, 7167, 7168, 7169, 7423, 7424, 7679, 7680, 7698, 7699])
+    Wsub = np.ascontiguousarray(W.reshape(N, rb)[rows]).reshape(-1)
+    ref = T.oracle_gemm_nt(fmt, xq, Wsub, np.ascontiguousarray(bias[rows]), M, len(rows), K)
+    assert T.norm_err(c[:, rows], ref) <= TOL
+    ab = T.row_bytes(af, K)
+    for t in (0, 63, 64, 300, 511, 512, 519):
+        y = P.dev_gemm_nt(fmt, P.to_device(xq[t * ab:(t + 1) * ab].copy()), Wd, bd, 1, N, K).cpu().numpy().reshape(-1)
+        assert T.norm_err(c[t], y) <= 2e-6, t
+    assert np.array_equal(P.dev_gemm_nt(fmt, xq_d, Wd, bd, M, N, K).cpu().numpy(), c)
 
 
 # ---- prefill GEMM on the matrix cores, Q6_K (token counts above 16) --------------------------
