@@ -24,6 +24,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <strings.h>
 
 #include "ckernel_quant_hip.h"
 #include "ckq_launch.h"
@@ -320,7 +321,7 @@ int ckq_weights_register_manifest(const void *base, const char *manifest_path)
     if (!base || !manifest_path) return CKQ_EINVAL;
     FILE *mf = fopen(manifest_path, "r");
     if (!mf) return CKQ_EINVAL;
-    static const char *const quant[] = {"q4_k", "q4k", "q5_k", "q5k", "q6_k", "q6k", "q8_0"};
+    static const char *const quant[] = {"q4_k", "q4k", "q5_k", "q5k", "q6_k", "q6k", "q8_0", "q80", "q5_0", "q50"};
     char line[4096];
     int n = 0, rc = 0, inited = 0;
     while (rc == 0 && fgets(line, sizeof line, mf)) {
@@ -338,7 +339,7 @@ int ckq_weights_register_manifest(const void *base, const char *manifest_path)
         }
         if (nf < 5) { rc = CKQ_EINVAL; break; }        /* malformed line */
         int is_quant = 0;
-        for (size_t i = 0; i < sizeof quant / sizeof quant[0]; ++i) is_quant |= strcmp(f[1], quant[i]) == 0;
+        for (size_t i = 0; i < sizeof quant / sizeof quant[0]; ++i) is_quant |= strcasecmp(f[1], quant[i]) == 0;
         if (!is_quant) continue;
         const unsigned long long size = strtoull(f[3], NULL, 0), off = strtoull(f[4], NULL, 0);
         if (size == 0) continue;

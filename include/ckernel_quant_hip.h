@@ -290,7 +290,8 @@ int ckq_synchronize(void);
  * reference's loader reads (one tensor per line,
  * name|dtype|file_offset|size|runtime_offset; version/v7/src/
  * ckernel_model_load_v7.c:17-35, 330-377) and registers every q4_k / q5_k /
- * q6_k / q8_0 tensor at base + runtime_offset, base being the arena
+ * q6_k / q8_0 / q5_0 tensor (names compared without case, with or without the
+ * underscore) at base + runtime_offset, base being the arena
  * ck_load_weights filled.  Returns the number of tensors registered or a
  * negative CKQ_E* code (unreadable file, malformed line).
  * resident = number of resident regions, total size through *bytes. */

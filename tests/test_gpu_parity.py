@@ -861,7 +861,7 @@ def test_weights_register_manifest_and_ranges(tmp_path):
     m = tmp_path / "weights_manifest.map"
     m.write_text("# name|dtype|file_offset|size|runtime_offset\n"
                  "model.norm.weight|fp32|8|4096|0\n"
-                 "model.layers.0.wq|q4_k|4104|%d|%d\n"
+                 "model.layers.0.wq|Q4_K|4104|%d|%d\n"
                  "model.layers.0.wdown|q6k|0x%x|%d|%d\n" % (len(wa), oa, 4104 + len(wa), len(wb), ob))
     say("ckq_weights_register_manifest")
     assert L.ckq_weights_register_manifest(T.ptr(arena), str(m).encode()) == 2
