@@ -129,6 +129,7 @@ _SIGS = {
     "ckq_weights_clear": (None, []),
     "ckq_weights_set_cache": (None, [_i]),
     "ckq_set_parallel_whole": (None, [_i]),
+    "ckq_set_gemm_policy": (None, [_i]),
     "ckq_last_error": (_i, []),
     "ckq_clear_error": (None, []),
     "ckq_error_string": (_c.c_char_p, [_i]),

@@ -119,6 +119,9 @@ static int init_locked(void)
     if (c && strcmp(c, "0") == 0) g_cache_on = 0;
     const char *p = getenv("CKQ_PARALLEL_MODE");
     if (p && strcmp(p, "whole") == 0) g_parallel_whole = 1;
+    const char *gp = getenv("CKQ_GEMM_POLICY");
+    if (gp && strcmp(gp, "matrix") == 0) ckq_launch_set_gemm_policy(CKQ_GEMM_MATRIX);
+    if (gp && strcmp(gp, "stream") == 0) ckq_launch_set_gemm_policy(CKQ_GEMM_STREAM);
     g_inited = 1;
     return 0;
 }
@@ -402,6 +405,8 @@ void ckq_weights_set_cache(int enabled)
     g_cache_on = enabled != 0;
     pthread_mutex_unlock(&g_mu);
 }
+
+void ckq_set_gemm_policy(int policy) { ckq_launch_set_gemm_policy(policy); }
 
 void ckq_set_parallel_whole(int enabled)
 {

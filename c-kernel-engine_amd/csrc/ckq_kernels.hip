@@ -28,10 +28,32 @@ __device__ __forceinline__ int wave_in_block();
 /* GEMV                                                                       */
 /* ========================================================================= */
 
-/* Token counts above this use the MFMA GEMMs; at or below it the
- * weight-streaming dot4 kernel with 8-token tiles reads the weights once or
- * twice and is faster. */
-#define CKQ_GEMM_MIN_TOKENS 16
+/* Which kernel serves a matmul of `ntok` tokens.  The weight-streaming dot4
+ * kernel takes up to eight tokens per pass over the weights; the matrix-core
+ * GEMMs read the weights once for any token count but have a floor of 13-19 us
+ * (their K loop waits on global->LDS copies of ~1.5 us latency with only two or
+ * three stages to cover it).  Measured crossover: one pass always streams;
+ * beyond that the streaming kernel stays ahead while (passes x weight bytes,
+ * at least 3 MB each) fits the budget - 20 MB, 40 MB for the Q5_K GEMM whose
+ * floor is higher.  Examples at 9-16 tokens: Q4_K 4096x4096 (9.4 MB) streams
+ * (12 us against 14), 11008x4096 (25 MB) goes to the matrix cores (19 us
+ * against 25-28), the Q8_0 LM head 151936x896 likewise (67 us against 89-102);
+ * Q8_0 4864x896 streams up to 32 tokens. */
+constexpr int CKQ_STREAM_TOKENS = 8;
+#include <atomic>
+static std::atomic<int> g_gemm_policy{0};      /* 0 automatic, 1 matrix cores above one pass, 2 always stream */
+
+extern "C" void ckq_launch_set_gemm_policy(int policy) { g_gemm_policy.store(policy < 0 || policy > 2 ? 0 : policy); }
+
+static bool gemm_on_matrix_cores(int ntok, size_t weight_bytes, size_t budget_mb)
+{
+    const int policy = g_gemm_policy.load(std::memory_order_relaxed);
+    if (ntok <= CKQ_STREAM_TOKENS || policy == 2) return false;
+    if (policy == 1) return true;
+    const size_t passes = (size_t)(ntok + CKQ_STREAM_TOKENS - 1) / CKQ_STREAM_TOKENS;
+    const size_t per = weight_bytes > ((size_t)3 << 20) ? weight_bytes : ((size_t)3 << 20);
+    return passes * per > (budget_mb << 20);
+}
 
 struct GemvArgs {
     float         *y;
@@ -339,28 +361,25 @@ extern "C" int ckq_launch_gemv(int fmt, float *y, const void *W, const void *X, 
     switch (fmt) {
     case CKQ_FMT_Q4_K:
         if (K % 256) return CKQ_ESHAPE;
-        /* prefill-sized token counts go to the matrix cores */
-        if (!dump && ntok > CKQ_GEMM_MIN_TOKENS && row0 == 0 && row1 == nrows)
+        if (!dump && row0 == 0 && row1 == nrows && gemm_on_matrix_cores(ntok, (size_t)nrows * (K / 256) * 144, 20))
             return launch_gemm_q4k_mfma(X, W, bias, y, ntok, nrows, K, ldy, s);
         a.npos = K / 64; a.wrow = (long)(K / 256) * 144; a.xrow = (long)(K / 256) * 292; a.nsub_row = K / 32;
         return launch_fmt<FmtQ4K>(a, dump, 8, s);
     case CKQ_FMT_Q5_K:
         if (K % 256) return CKQ_ESHAPE;
-        /* the min term and the 16-bit scale products make this kernel's fixed
-         * cost per block higher: the token tiles stay ahead up to 64 tokens */
-        if (!dump && ntok > 4 * CKQ_GEMM_MIN_TOKENS && row0 == 0 && row1 == nrows)
+        if (!dump && row0 == 0 && row1 == nrows && gemm_on_matrix_cores(ntok, (size_t)nrows * (K / 256) * 176, 40))
             return launch_gemm_q5k_mfma(X, W, bias, y, ntok, nrows, K, ldy, s);
         a.npos = K / 64; a.wrow = (long)(K / 256) * 176; a.xrow = (long)(K / 256) * 292; a.nsub_row = K / 32;
         return launch_fmt<FmtQ5K>(a, dump, 8, s);
     case CKQ_FMT_Q6_K:
         if (K % 256) return CKQ_ESHAPE;
-        if (!dump && ntok > CKQ_GEMM_MIN_TOKENS && row0 == 0 && row1 == nrows)
+        if (!dump && row0 == 0 && row1 == nrows && gemm_on_matrix_cores(ntok, (size_t)nrows * (K / 256) * 210, 20))
             return launch_gemm_q6k_mfma(X, W, bias, y, ntok, nrows, K, ldy, s);
         a.npos = K / 64; a.wrow = (long)(K / 256) * 210; a.xrow = (long)(K / 256) * 292; a.nsub_row = K / 16;
         return launch_fmt<FmtQ6K>(a, dump, 8, s);
     case CKQ_FMT_Q8_0:
         if (K % 32) return CKQ_ESHAPE;
-        if (!dump && ntok > CKQ_GEMM_MIN_TOKENS && row0 == 0 && row1 == nrows)
+        if (!dump && row0 == 0 && row1 == nrows && gemm_on_matrix_cores(ntok, (size_t)nrows * (K / 32) * 34, 20))
             return launch_gemm_q80_mfma(X, W, bias, y, ntok, nrows, K, ldy, s);
         a.npos = K / 32; a.wrow = (long)(K / 32) * 34; a.xrow = (long)(K / 32) * 34; a.nsub_row = K / 32;
         return launch_fmt<FmtQ80>(a, dump, 8, s);
@@ -368,7 +387,7 @@ extern "C" int ckq_launch_gemv(int fmt, float *y, const void *W, const void *X, 
         if (K % 32) return CKQ_ESHAPE;
         /* prefill: the blocks are rewritten as Q8_0 blocks (same scale, values
          * q - 16: every dot product is unchanged) and go to the Q8_0 GEMM */
-        if (!dump && ntok > CKQ_GEMM_MIN_TOKENS && row0 == 0 && row1 == nrows)
+        if (!dump && row0 == 0 && row1 == nrows && gemm_on_matrix_cores(ntok, (size_t)nrows * (K / 32) * 22, 20))
             return launch_gemm_q50_via_q80(X, W, bias, y, ntok, nrows, K, ldy, s);
         a.npos = K / 32; a.wrow = (long)(K / 32) * 22; a.xrow = (long)(K / 32) * 34; a.nsub_row = K / 32;
         return launch_fmt<FmtQ50>(a, dump, 8, s);

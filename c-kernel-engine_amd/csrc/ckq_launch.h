@@ -38,6 +38,10 @@ int ckq_launch_gemv(int fmt, float *y, const void *W, const void *X, const float
                     int nrows, int K, int ntok, long ldy, int row0, int row1,
                     int32_t *subdots, void *stream);
 
+/* Kernel choice for more than eight tokens: 0 = by token count and weight size
+ * (default), 1 = always the matrix-core GEMM, 2 = always the streaming kernel. */
+void ckq_launch_set_gemm_policy(int policy);
+
 /* fp32 [rows x k] -> Q8_K / Q8_0 blocks, row-major. */
 int ckq_launch_quantize_q8_k(const float *x, void *y, int rows, int k, void *stream);
 int ckq_launch_quantize_q8_0(const float *x, void *y, int rows, int k, void *stream);

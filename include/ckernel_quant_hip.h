@@ -136,9 +136,10 @@ void rmsnorm_q8_k_fused(const float *input, const float *gamma, void *vy, int to
 
 /* Q5_0 weights (fp16 d, 32 five-bit values q - 16 per 22-byte block: the
  * format GGUF files use for rows too short for K-quants) against Q8_0
- * activations.  Token counts above 16 rewrite the blocks as Q8_0 blocks on the
- * device (same scale, values q - 16: every dot product is unchanged) and run
- * the Q8_0 matrix-core GEMM.  Replaces src/kernels/gemm_kernels_q5_0.c:1602-1620
+ * activations.  When the launch picks the matrix cores (more than eight tokens
+ * and enough weight bytes, see ckq_set_gemm_policy) the blocks are rewritten as
+ * Q8_0 blocks on the device (same scale, values q - 16: every dot product is
+ * unchanged) and the Q8_0 matrix-core GEMM runs.  Replaces src/kernels/gemm_kernels_q5_0.c:1602-1620
  * (vec_dot), :1637-1657 (gemv), :1659-1700 (_parallel_simd), :1725-1753 (gemm_nt).
  * The fp32-activation forms gemv_q5_0 / gemm_nt_q5_0 are not built. */
 void vec_dot_q5_0_q8_0(int n, float *s, const void *vx, const void *vy);
@@ -304,6 +305,15 @@ void ckq_weights_set_cache(int enabled);
 /* Thread-split entry points: 0 (default) = every call computes its own row
  * range; 1 = the ith==0 call computes all rows and the others return. */
 void ckq_set_parallel_whole(int enabled);
+/* Which kernel serves a matmul of more than eight tokens (up to eight always
+ * take the weight-streaming kernel, one pass over the weights).  AUTO, the
+ * default, picks by token count and weight size: the streaming kernel while
+ * its passes over the weights are cheaper than the matrix-core GEMM's fixed
+ * cost, the matrix cores beyond.  MATRIX and STREAM force one of them (tests,
+ * tuning); CKQ_GEMM_POLICY=matrix|stream sets it from the environment.  Both
+ * kernels meet the same tolerance; their fp32 summation orders differ. */
+enum { CKQ_GEMM_AUTO = 0, CKQ_GEMM_MATRIX = 1, CKQ_GEMM_STREAM = 2 };
+void ckq_set_gemm_policy(int policy);
 /* Last error of the calling process (0 = none), its text, and a reset for
  * callers that run with CKQ_ABORT_ON_ERROR=0 and handle errors themselves. */
 int         ckq_last_error(void);

@@ -37,6 +37,20 @@ def _lib():
     L.ckq_weights_clear()
 
 
+MATRIX_CORE_TESTS = ("mfma", "split_k", "q5_0_row_and_token")
+
+
+@pytest.fixture(autouse=True)
+def _gemm_policy(request, _lib):
+    """Tests aimed at the matrix-core GEMMs force them for every token count
+    above eight (the automatic choice would send their small shapes to the
+    streaming kernel); everything else runs with the automatic choice."""
+    forced = any(k in request.node.name for k in MATRIX_CORE_TESTS)
+    _lib.ckq_set_gemm_policy(1 if forced else 0)
+    yield
+    _lib.ckq_set_gemm_policy(0)
+
+
 def make_case(fmt, rows, K, kind, seed, tokens=1):
     if kind == "rand":
         W = T.random_blocks(fmt, rows * (K // T.ELEMS[fmt]), seed)
@@ -1006,9 +1020,9 @@ def test_q5_0_golden_fixture(kind):
 
 
 def test_q5_0_row_and_token_counts():
-    """Token tiles up to 16 tokens; above that the blocks are rewritten as Q8_0
-    blocks and the Q8_0 matrix-core GEMM runs: the same bits as that GEMM on
-    weights converted by the oracle."""
+    """Token tiles up to eight tokens; above that (forced here, this matrix is
+    small) the blocks are rewritten as Q8_0 blocks and the Q8_0 matrix-core GEMM
+    runs: the same bits as that GEMM on weights converted by the oracle."""
     K = 896
     for rows in (1, 3, 17, 64, 65, 257):
         W, _, xq = make_case("q5_0", rows, K, "rand", 11 * rows)
@@ -1022,7 +1036,7 @@ def test_q5_0_row_and_token_counts():
         ref = T.oracle_gemm_nt("q5_0", xq, W, bias, M, N, K)
         c = P.gemm_nt("q5_0", xq, W, bias, M, N, K)
         assert T.norm_err(c, ref) <= TOL, M
-        if M > 16:
+        if M > 8:
             w8 = np.zeros(len(W) // 22 * 34, np.uint8)
             T.oracle().orc_q5_0_to_q8_0(T.ptr(W), T.ptr(w8), ctypes.c_size_t(len(W) // 22))
             assert np.array_equal(P.gemm_nt("q8_0", xq, w8, bias, M, N, K), c), M
@@ -1035,3 +1049,36 @@ def test_fused_mlp_q5_0_gate_up_golden_case():
     got = P.fused_mlp_swiglu_prefill_w1w2_quant(G["mlp_x"], G["mlp_w1_q5_0"], G["mlp_b1"], "q5_0", G["mlp_w2_q4_k"],
                                                 G["mlp_b2"], "q4_k", SEQ, ED, AED, ID, AID)
     assert T.norm_err(got, G["mlp_out_q5_0w1_q4_k_avx2"].reshape(SEQ, AED)) <= TOL
+
+
+# ---- automatic choice between the streaming kernel and the matrix cores --------------------------
+
+@pytest.mark.parametrize("fmt,N,K,expect", [
+    ("q4_k", 4096, 4096, {8: "stream", 9: "stream", 16: "stream", 17: "matrix"}),      # 9.4 MB: two passes stream
+    ("q4_k", 11008, 4096, {8: "stream", 9: "matrix"}),                                  # 25 MB
+    ("q6_k", 1024, 4096, {16: "stream", 40: "stream", 49: "matrix"}),                   # 3.4 MB
+    ("q8_0", 4864, 896, {32: "stream", 33: "matrix"}),                                  # 4.4 MB
+    ("q5_k", 4864, 1024, {64: "stream", 96: "stream", 100: "matrix"}),                  # 3.3 MB, 40 MB budget
+    ("q5_0", 896, 896, {48: "stream", 57: "matrix"}),                                   # below the 3 MB floor
+])
+def test_gemm_automatic_kernel_choice(fmt, N, K, expect):
+    """With the default policy the library picks the kernel by token count and
+    weight size.  Each result matches the oracle on a sample of rows, and equals
+    bit for bit what the kernel it should have picked gives when forced."""
+    L = ckq.lib()
+    W = T.random_blocks(fmt, N * (K // T.ELEMS[fmt]), 4242)
+    Wd = P.to_device(W)
+    rb = T.row_bytes(fmt, K)
+    rows = np.array([0, 1, N // 2, N - 1])
+    Wsub = np.ascontiguousarray(W.reshape(N, rb)[rows]).reshape(-1)
+    for M, which in expect.items():
+        say("automatic kernel choice", fmt, N, K, M, which)
+        xq = T.oracle_quantize(T.normal(M * K, 0.0, 1.0, 500 + M), T.act_fmt(fmt), rows=M)
+        xd = P.to_device(xq)
+        L.ckq_set_gemm_policy(0)
+        auto = P.dev_gemm_nt(fmt, xd, Wd, None, M, N, K).cpu().numpy()
+        assert T.norm_err(auto[:, rows], T.oracle_gemm_nt(fmt, xq, Wsub, None, M, len(rows), K)) <= TOL, M
+        L.ckq_set_gemm_policy(1 if which == "matrix" else 2)
+        forced = P.dev_gemm_nt(fmt, xd, Wd, None, M, N, K).cpu().numpy()
+        L.ckq_set_gemm_policy(0)
+        assert np.array_equal(auto, forced), (M, which)
