@@ -365,9 +365,12 @@ def main():
 
         # a 7B decoder layer's projection set at M=1: Q,K,V,O (4096x4096 Q4_K), gate, up
         # (11008x4096 Q4_K), down (4096x11008 Q6_K), one C call per layer, weights of
-        # successive steps distinct (4 rotated layers = 502 MB)
+        # successive steps distinct (4 rotated layers = 502 MB).  The sequence call issues
+        # independent same-shape entries as one launch; to keep the dependencies of a real
+        # layer, O reads its activations from V's output buffer, gate/up from O's and down
+        # from up's (the bytes are not meaningful activations; the timing does not care),
+        # so the launches are Q+K+V | O | gate+up | down.
         x4k = P.dev_quantize(P.to_device(T.normal(4096, seed=31)), "q8_k")
-        x11k = P.dev_quantize(P.to_device(T.normal(11008, seed=32)), "q8_k")
         layers, keep, lbytes = [], [], 0
         for li in range(4):
             ops = []
@@ -375,15 +378,17 @@ def main():
                 Wj = torch.from_numpy(T.synth_weights(fmt, r, k, seed=1000 + j)).cuda()
                 if li:
                     Wj = torch.roll(Wj.view(r, -1), shifts=li * 13 + j, dims=0).contiguous().reshape(-1)
-                o = torch.empty(r, dtype=torch.float32, device="cuda")
+                o = torch.zeros(r, dtype=torch.float32, device="cuda")
                 keep += [Wj, o]
-                ops.append((fmt, x11k if k == 11008 else x4k, Wj, None, o, 1, r, k))
+                src = x4k if j < 3 else ops[2][4] if j == 3 else ops[3][4] if j < 6 else ops[5][4]
+                ops.append((fmt, src, Wj, None, o, 1, r, k))
                 if li == 0:
                     lbytes += gemv_bytes(fmt, r, k)
             layers.append(ops)
         s = H.time_sequence(layers, max(40, a.steps // 10), 8)
         extras["layer_7b_projection_set_M1"] = {"us": round(s * 1e6, 2), "gbs": round(lbytes / s / 1e9, 1), "bytes": lbytes,
-                                                "frac_hbm": round(lbytes / s / 1e9 / HBM_PEAK_GBS, 4), "launches": 7}
+                                                "frac_hbm": round(lbytes / s / 1e9 / HBM_PEAK_GBS, 4), "launches": 4,
+                                                "note": "Q+K+V and gate+up each as one grouped launch"}
         del layers, keep
         torch.cuda.empty_cache()
 

@@ -55,6 +55,8 @@ static bool gemm_on_matrix_cores(int ntok, size_t weight_bytes, size_t budget_mb
     return passes * per > (budget_mb << 20);
 }
 
+constexpr int CKQ_GROUP_MAX = 4;   /* independent matmuls of one shape in one launch */
+
 struct GemvArgs {
     float         *y;
     const uint8_t *W;
@@ -63,6 +65,15 @@ struct GemvArgs {
     int32_t       *sub;
     int  nrows, npos, ntok, row0, row1, nsub_row;
     long wrow, xrow, ldy;
+};
+
+/* Problems 1..3 of a grouped launch (blockIdx.z = g > 0); problem 0 is in GemvArgs. */
+struct GemvGroup {
+    float         *y[CKQ_GROUP_MAX - 1];
+    const uint8_t *W[CKQ_GROUP_MAX - 1];
+    const uint8_t *X[CKQ_GROUP_MAX - 1];
+    const float   *bias[CKQ_GROUP_MAX - 1];
+    int n;                                  /* problems in the launch, 1 = not grouped */
 };
 
 /* Wave index as a scalar: lets the compiler keep row indices, row base
@@ -83,12 +94,26 @@ __device__ __forceinline__ int wave_in_block() { return __builtin_amdgcn_readfir
  * summed over the LPR lanes with a fixed DPP tree; the last lane of the group
  * stores.
  */
-template <class F, int LPR, int PPL, int MT, int RPI, bool DUMP, int WPB, bool LDSX>
+template <class F, int LPR, int PPL, int MT, int RPI, bool DUMP, int WPB, bool LDSX, bool GRP = false>
 __global__ void __launch_bounds__(64 * WPB) __attribute__((amdgpu_waves_per_eu(MT == 1 && !DUMP && PPL == 1 && RPI == 1 ? F::OCC1 : MT == 1 && !DUMP && PPL == 1 && RPI == 2 && LPR == 64 ? F::OCC2 : MT >= 4 && PPL == 1 ? 4 : 1)))
-gemv_kernel(GemvArgs a)
+gemv_kernel(const uint8_t *W, const uint8_t *X, long wrow, long xrow, int row0, int row1, int npos, int ntok,
+            float *y, const float *bias, long ldy, int32_t *sub, int nsub_row, int nrows, GemvGroup grp)
 {
+    /* The arguments are scalars, those the first loads need in front: the
+     * first fourteen registers' worth arrive preloaded with the wave (build
+     * flag -amdgpu-kernarg-preload-count) instead of through a scalar load
+     * that every wave waits for before it can issue its first weight load. */
+    const GemvArgs a = {y, W, X, bias, sub, nrows, npos, ntok, row0, row1, nsub_row, wrow, xrow, ldy};
     constexpr int SLOTS = 64 / LPR;
     extern __shared__ __attribute__((aligned(16))) uint8_t xs[];   /* LDSX: the MT activation rows */
+    /* grouped launch: blockIdx.z picks the problem (a separate instantiation: the extra
+     * argument loads lengthen the start of every wave, which a bandwidth-bound launch
+     * of a few microseconds feels) */
+    const int g = GRP ? (int)blockIdx.z : 0;
+    float *const         gy    = g == 0 ? a.y    : grp.y[g - 1];
+    const uint8_t *const gW    = g == 0 ? a.W    : grp.W[g - 1];
+    const uint8_t *const gX    = g == 0 ? a.X    : grp.X[g - 1];
+    const float *const   gbias = g == 0 ? a.bias : grp.bias[g - 1];
     const int lane = threadIdx.x & 63, wave = wave_in_block();
     const int slot = lane / LPR, l = lane % LPR;
     const int wave_row = a.row0 + (blockIdx.x * WPB + wave) * (SLOTS * RPI);   /* uniform */
@@ -97,14 +122,14 @@ gemv_kernel(GemvArgs a)
     const int wrow_c = min(wave_row, a.row1 - 1);
     const int rbase = wave_row + slot * RPI;
     const int t0 = blockIdx.y * MT;
-    const uint8_t *wbase = a.W + (size_t)wrow_c * a.wrow;                      /* uniform */
+    const uint8_t *wbase = gW + (size_t)wrow_c * a.wrow;                      /* uniform */
 
     /* Every wave of the block reads the same activation rows: they are staged
      * once in LDS instead of once per wave through the vector cache.  Their
      * loads go out first, all at once (one round trip, they hit in L2), the
      * weight loads follow, and only then are the staged values written. */
     constexpr int XNT = 64 * WPB, XU = MT == 1 ? 2 : 4;
-    const uint8_t *xsrc = a.X + (size_t)t0 * a.xrow;
+    const uint8_t *xsrc = gX + (size_t)t0 * a.xrow;
     const int xbytes = (int)((long)min(MT, a.ntok - t0) * a.xrow), xn = xbytes / F::XS_SRC;   /* staging units */
     const u32 xcap = (u32)((long)MT * a.xrow / F::XS_SRC);                                     /* units of a full tile */
     u32 xv[XU][F::XS_REGS];
@@ -182,7 +207,7 @@ gemv_kernel(GemvArgs a)
                         F::load_act_lds(at, xs, tl, pos, (u32)a.xrow, a.npos, xcap);
                     } else {
                         const int tok = min(t0 + t, a.ntok - 1);                   /* uniform */
-                        F::load_act(at, a.X + (size_t)tok * a.xrow, pos);
+                        F::load_act(at, gX + (size_t)tok * a.xrow, pos);
                     }
 #pragma unroll
                     for (int r = 0; r < RPI; ++r) {
@@ -203,7 +228,7 @@ gemv_kernel(GemvArgs a)
                     F::load_act_lds(act[t][p], xs, tl, pos, (u32)a.xrow, a.npos, xcap);
                 } else {
                     const int tok = min(t0 + t, a.ntok - 1);                   /* uniform */
-                    F::load_act(act[t][p], a.X + (size_t)tok * a.xrow, pos);
+                    F::load_act(act[t][p], gX + (size_t)tok * a.xrow, pos);
                 }
             }
         }
@@ -239,18 +264,34 @@ gemv_kernel(GemvArgs a)
             const float s = group_sum<LPR>(acc[r][t]);
             const int row = rbase + r, tok = t0 + t;
             if (!DUMP && l == LPR - 1 && row < a.row1 && tok < a.ntok)
-                a.y[(size_t)tok * a.ldy + row] = a.bias ? s + a.bias[row] : s;
+                gy[(size_t)tok * a.ldy + row] = gbias ? s + gbias[row] : s;
         }
 }
+
+/* The group of the launch in flight on this thread (set by ckq_launch_gemv_group
+ * around its dispatch; every other launch sees n = 1). */
+static thread_local GemvGroup t_group = {{}, {}, {}, {}, 1};
 
 template <class F, int LPR, int PPL, int MT, int RPI, bool DUMP, int WPB, bool LDSX>
 static int launch_one(const GemvArgs &a, hipStream_t s)
 {
     constexpr int rows_per_block = WPB * (64 / LPR) * RPI;
     const int nr = a.row1 - a.row0;
-    dim3 grid((nr + rows_per_block - 1) / rows_per_block, (a.ntok + MT - 1) / MT);
+    dim3 grid((nr + rows_per_block - 1) / rows_per_block, (a.ntok + MT - 1) / MT, 1);
     const size_t lds = LDSX ? F::xs_lds_bytes((size_t)MT * (size_t)a.xrow) : 0;
-    hipLaunchKernelGGL((gemv_kernel<F, LPR, PPL, MT, RPI, DUMP, WPB, LDSX>), grid, dim3(64 * WPB), lds, s, a);
+    if (t_group.n > 1) {
+        if constexpr (MT == 1 && !DUMP && LDSX) {        /* grouped launches are single-token */
+            grid.z = (unsigned)t_group.n;
+            hipLaunchKernelGGL((gemv_kernel<F, LPR, PPL, MT, RPI, DUMP, WPB, LDSX, true>), grid, dim3(64 * WPB), lds, s,
+                               a.W, a.X, a.wrow, a.xrow, a.row0, a.row1, a.npos, a.ntok, a.y, a.bias, a.ldy, a.sub,
+                               a.nsub_row, a.nrows, t_group);
+            return (int)hipGetLastError();
+        }
+        return CKQ_EINVAL;
+    }
+    hipLaunchKernelGGL((gemv_kernel<F, LPR, PPL, MT, RPI, DUMP, WPB, LDSX>), grid, dim3(64 * WPB), lds, s,
+                       a.W, a.X, a.wrow, a.xrow, a.row0, a.row1, a.npos, a.ntok, a.y, a.bias, a.ldy, a.sub,
+                       a.nsub_row, a.nrows, t_group);
     return (int)hipGetLastError();
 }
 
@@ -344,6 +385,8 @@ static int launch_gemm_q50_via_q80(const void *A, const void *B, const float *bi
     return launch_gemm_q80_mfma(A, tmp, bias, C, M, N, K, ldc, s);
 }
 
+static int launch_gemv_args(int fmt, GemvArgs &a, int K, void *stream);
+
 extern "C" int ckq_launch_gemv(int fmt, float *y, const void *W, const void *X, const float *bias,
                                int nrows, int K, int ntok, long ldy, int row0, int row1,
                                int32_t *subdots, void *stream)
@@ -353,11 +396,46 @@ extern "C" int ckq_launch_gemv(int fmt, float *y, const void *W, const void *X, 
     if (row1 > nrows) row1 = nrows;
     if (row0 >= row1) return 0;
     if (subdots && ntok != 1) return CKQ_EINVAL;
-    GemvArgs a;
+    GemvArgs a = {};
     a.y = y; a.W = (const uint8_t *)W; a.X = (const uint8_t *)X; a.bias = bias; a.sub = subdots;
     a.nrows = nrows; a.ntok = ntok; a.row0 = row0; a.row1 = row1; a.ldy = ldy;
+    return launch_gemv_args(fmt, a, K, stream);
+}
+
+/* `n` (2..CKQ_GROUP_MAX) independent matmuls of one format and shape - the
+ * Q/K/V or the gate/up projections of a token - as one launch of the streaming
+ * kernel: the launches' fixed start-up cost is paid once and the chip holds n
+ * times the loads in flight.  One token (decode); K up to 8192 elements. */
+extern "C" int ckq_launch_gemv_group(int fmt, int n, float *const *y, const void *const *W, const void *const *X,
+                                     const float *const *bias, int nrows, int K, int ntok, long ldy, void *stream)
+{
+    if (n < 1 || n > CKQ_GROUP_MAX || !y || !W || !X || nrows <= 0 || K <= 0 || ntok != 1) return CKQ_EINVAL;
+    /* the activation row is staged in LDS in every grouped kernel */
+    if ((size_t)K * 4 > 32768) return CKQ_ESHAPE;
+    for (int i = 0; i < n; ++i)
+        if (!y[i] || !W[i] || !X[i]) return CKQ_EINVAL;
+    GemvArgs a = {};
+    a.y = y[0]; a.W = (const uint8_t *)W[0]; a.X = (const uint8_t *)X[0]; a.bias = bias ? bias[0] : nullptr; a.sub = nullptr;
+    a.nrows = nrows; a.ntok = ntok; a.row0 = 0; a.row1 = nrows; a.ldy = ldy;
+    for (int i = 1; i < n; ++i) {
+        t_group.y[i - 1] = y[i]; t_group.W[i - 1] = (const uint8_t *)W[i]; t_group.X[i - 1] = (const uint8_t *)X[i];
+        t_group.bias[i - 1] = bias ? bias[i] : nullptr;
+    }
+    t_group.n = n;
+    const int rc = launch_gemv_args(fmt, a, K, stream);
+    t_group.n = 1;
+    return rc;
+}
+
+static int launch_gemv_args(int fmt, GemvArgs &a, int K, void *stream)
+{
+    float *const y = a.y;
+    const void *const W = a.W, *const X = a.X;
+    const float *const bias = a.bias;
+    const int nrows = a.nrows, ntok = a.ntok, row0 = a.row0, row1 = a.row1;
+    const long ldy = a.ldy;
     hipStream_t s = (hipStream_t)stream;
-    const bool dump = subdots != nullptr;
+    const bool dump = a.sub != nullptr;
     switch (fmt) {
     case CKQ_FMT_Q4_K:
         if (K % 256) return CKQ_ESHAPE;

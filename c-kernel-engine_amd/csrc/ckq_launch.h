@@ -38,6 +38,12 @@ int ckq_launch_gemv(int fmt, float *y, const void *W, const void *X, const float
                     int nrows, int K, int ntok, long ldy, int row0, int row1,
                     int32_t *subdots, void *stream);
 
+/* n (at most 4) independent single-token matmuls of one format and shape
+ * (K <= 8192) in one launch of the streaming kernel; pointer arrays are host
+ * arrays of device pointers, bias may be NULL or hold NULL entries. */
+int ckq_launch_gemv_group(int fmt, int n, float *const *y, const void *const *W, const void *const *X,
+                          const float *const *bias, int nrows, int K, int ntok, long ldy, void *stream);
+
 /* Kernel choice for more than eight tokens: 0 = by token count and weight size
  * (default), 1 = always the matrix-core GEMM, 2 = always the streaming kernel. */
 void ckq_launch_set_gemm_policy(int policy);

@@ -1082,3 +1082,63 @@ def test_gemm_automatic_kernel_choice(fmt, N, K, expect):
         forced = P.dev_gemm_nt(fmt, xd, Wd, None, M, N, K).cpu().numpy()
         L.ckq_set_gemm_policy(0)
         assert np.array_equal(auto, forced), (M, which)
+
+
+# ---- sequences: independent entries of one shape share a launch ----------------------------------
+
+@pytest.mark.parametrize("fmt,N,K", [("q4_k", 384, 1024), ("q6_k", 200, 512), ("q8_0", 130, 896), ("q5_k", 96, 768)])
+def test_matmul_sequence_groups_independent_entries(fmt, N, K):
+    """Q/K/V-like entries (one input, separate weights and outputs) and a pair
+    with separate inputs go out as grouped launches; every output has the bits
+    of the same matmul launched alone, with and without biases, for one and
+    several tokens, and the oracle's values."""
+    import torch
+    for M in (1, 3, 8):
+        Ws = [T.random_blocks(fmt, N * (K // T.ELEMS[fmt]), 700 + i) for i in range(6)]
+        xs = [T.oracle_quantize(T.normal(M * K, 0.0, 1.0, 800 + i), T.act_fmt(fmt), rows=M) for i in range(2)]
+        bias = [T.normal(N, 0.0, 0.5, seed=900 + i) if i % 2 else None for i in range(6)]
+        Wd = [P.to_device(w) for w in Ws]
+        xd = [P.to_device(x) for x in xs]
+        bd = [None if b is None else P.to_device(b) for b in bias]
+        inp = [0, 0, 0, 1, 0, 1]                       # entries 0-2 share an input; 3-5 alternate
+        outs = [torch.full((M * N,), 7.0, dtype=torch.float32, device="cuda") for _ in range(6)]
+        say("sequence grouping", fmt, M)
+        P.dev_matmul_sequence([(fmt, xd[inp[i]], Wd[i], bd[i], outs[i], M, N, K) for i in range(6)])
+        for i in range(6):
+            alone = P.dev_gemm_nt(fmt, xd[inp[i]], Wd[i], bd[i], M, N, K).cpu().numpy()
+            got = outs[i].cpu().numpy().reshape(M, N)
+            assert np.array_equal(got, alone), (M, i)
+            assert T.norm_err(got, T.oracle_gemm_nt(fmt, xs[inp[i]], Ws[i], bias[i], M, N, K)) <= TOL, (M, i)
+
+
+def test_matmul_sequence_keeps_order_where_entries_depend():
+    """Entries that write what a later entry reads, or write the same output,
+    stay separate launches in list order: the bytes equal those of the same
+    entries issued one call at a time."""
+    import torch
+    fmt, N, K, M = "q4_k", 1168, 1024, 1
+    W1 = P.to_device(T.random_blocks(fmt, N * (K // 256), 31))
+    W2 = P.to_device(T.random_blocks(fmt, N * (K // 256), 32))
+    x = P.to_device(T.oracle_quantize(T.normal(K, 0.0, 1.0, 33), "q8_k"))
+    say("sequence with dependent entries")
+
+    def run(seq_call):
+        a = torch.zeros(N, dtype=torch.float32, device="cuda")
+        b = torch.zeros(N, dtype=torch.float32, device="cuda")
+        ops = [(fmt, x, W1, None, a, M, N, K),
+               (fmt, a, W2, None, b, M, N, K),      # reads the first 1168 bytes of `a` as a Q8_K row
+               (fmt, x, W2, None, b, M, N, K),      # same output as the entry before: the last one wins
+               (fmt, x, W1, None, a, M, N, K)]      # and `a` again
+        if seq_call:
+            P.dev_matmul_sequence(ops)
+        else:
+            for o in ops:
+                P.dev_matmul_sequence([o])
+        torch.cuda.synchronize()
+        return a.cpu().numpy().view(np.uint32), b.cpu().numpy().view(np.uint32)
+
+    a1, b1 = run(True)
+    a2, b2 = run(False)
+    assert np.array_equal(a1, a2) and np.array_equal(b1, b2)
+    ref = P.dev_gemm_nt(fmt, x, W2, None, M, N, K).cpu().numpy().reshape(-1).view(np.uint32)
+    assert np.array_equal(b1, ref)
