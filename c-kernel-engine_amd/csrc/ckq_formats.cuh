@@ -350,6 +350,74 @@ struct FmtQ80 {
     static constexpr int SUBS_PER_BLOCK = 1;
 };
 
+/* Q8_0 rows of an even number of blocks, taken two blocks (68 bytes) per
+ * position.  A 34-byte block starts 2 bytes off a dword boundary in every
+ * second block, and 16-byte loads at such addresses run 14 % below the aligned
+ * rate; a pair starts on a dword boundary (row pitch 34 * even), so its 17
+ * dwords are loaded aligned and the first block's quants, which sit 2 bytes in,
+ * are realigned in registers with v_alignbyte (the second block's quants start
+ * at byte 36 and need nothing).  Same integer dots; a lane adds its two blocks'
+ * fp32 terms before the cross-lane sum. */
+struct FmtQ80P : FmtQ80 {
+    static constexpr int NSUB = 2;
+    static constexpr int OCC1 = 6, OCC2 = 4;   /* 17 weight + 18 activation registers per position */
+    struct Wt  { u32 v[17]; };
+    struct Act { int q[16]; float d[2]; };
+    struct Dec { int q[16]; float d[2]; };
+    static __device__ __forceinline__ Off w_off(int pos)
+    {
+        Off o;
+        o.blk = (u32)pos * 68u;
+        return o;
+    }
+    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, const Off &o)
+    {
+        const uint8_t *p = row + o.blk;
+        ld16<4>(w.v, p);
+        ld16<4>(w.v + 4, p + 16);
+        ld16<4>(w.v + 8, p + 32);
+        ld16<4>(w.v + 12, p + 48);
+        w.v[16] = ld4<4>(p + 64);
+    }
+    static __device__ __forceinline__ void load_act(Act &a, const uint8_t *x, int pos)
+    {
+        const uint8_t *blk = x + (u32)pos * 68u;
+        a.d[0] = h2f(ld2(blk));
+        ld16<2>(a.q, blk + 2);
+        ld16<2>(a.q + 4, blk + 18);
+        a.d[1] = h2f(ld2(blk + 34));
+        ld16<2>(a.q + 8, blk + 36);
+        ld16<2>(a.q + 12, blk + 52);
+    }
+    /* the staged image is FmtQ80's (per 34-byte block); a position reads two consecutive blocks */
+    static __device__ __forceinline__ void load_act_lds(Act &a, const uint8_t *xs, int tl, int pos, u32, int npos, u32 total)
+    {
+        const u32 j = 2u * ((u32)tl * (u32)npos + (u32)pos);
+        const u32 *q = reinterpret_cast<const u32 *>(xs + 32u * j);
+        for (int i = 0; i < 16; ++i) a.q[i] = (int)q[i];
+        const float *d = reinterpret_cast<const float *>(xs + 32u * total + 4u * j);
+        a.d[0] = d[0];
+        a.d[1] = d[1];
+    }
+    static __device__ __forceinline__ void decode(Dec &d, const Wt &w, int)
+    {
+        d.d[0] = h2f(w.v[0] & 0xffffu);
+        for (int i = 0; i < 8; ++i) d.q[i] = (int)__builtin_amdgcn_alignbyte(w.v[i + 1], w.v[i], 2);
+        d.d[1] = h2f(w.v[8] >> 16);
+        for (int i = 0; i < 8; ++i) d.q[8 + i] = (int)w.v[9 + i];
+    }
+    static __device__ __forceinline__ float dot(const Dec &d, const Act &a, int *sub)
+    {
+        int s0 = 0, s1 = 0;
+        for (int i = 0; i < 8; ++i) s0 = dot4(d.q[i], a.q[i], s0);
+        for (int i = 0; i < 8; ++i) s1 = dot4(d.q[8 + i], a.q[8 + i], s1);
+        sub[0] = s0;
+        sub[1] = s1;
+        return (float)s0 * (d.d[0] * a.d[0]) + (float)s1 * (d.d[1] * a.d[1]);
+    }
+    static __device__ __forceinline__ int sub_index(int pos, int r) { return 2 * pos + r; }
+};
+
 /* Q5_0 weights against Q8_0 activations: 22-byte blocks (fp16 d, 32 fifth bits,
  * 16 nibble bytes), values q - 16 in [-16, 15]; everything on the activation
  * side is FmtQ80's.  Reference: gemm_kernels_q5_0.c:901-939. */

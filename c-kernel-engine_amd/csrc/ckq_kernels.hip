@@ -427,6 +427,13 @@ extern "C" int ckq_launch_gemv_group(int fmt, int n, float *const *y, const void
     return rc;
 }
 
+static bool weights_dword_aligned(const GemvArgs &a)
+{
+    uintptr_t bits = reinterpret_cast<uintptr_t>(a.W);
+    for (int i = 0; i + 1 < t_group.n; ++i) bits |= reinterpret_cast<uintptr_t>(t_group.W[i]);
+    return (bits & 3) == 0;
+}
+
 static int launch_gemv_args(int fmt, GemvArgs &a, int K, void *stream)
 {
     float *const y = a.y;
@@ -459,7 +466,13 @@ static int launch_gemv_args(int fmt, GemvArgs &a, int K, void *stream)
         if (K % 32) return CKQ_ESHAPE;
         if (!dump && row0 == 0 && row1 == nrows && gemm_on_matrix_cores(ntok, (size_t)nrows * (K / 32) * 34, 20))
             return launch_gemm_q80_mfma(X, W, bias, y, ntok, nrows, K, ldy, s);
-        a.npos = K / 32; a.wrow = (long)(K / 32) * 34; a.xrow = (long)(K / 32) * 34; a.nsub_row = K / 32;
+        a.wrow = (long)(K / 32) * 34; a.xrow = (long)(K / 32) * 34; a.nsub_row = K / 32;
+        /* rows of an even number of blocks at dword-aligned addresses: two blocks per position, aligned loads */
+        if (K % 64 == 0 && weights_dword_aligned(a)) {
+            a.npos = K / 64;
+            return launch_fmt<FmtQ80P>(a, dump, 8, s);
+        }
+        a.npos = K / 32;
         return launch_fmt<FmtQ80>(a, dump, 8, s);
     case CKQ_FMT_Q5_0:
         if (K % 32) return CKQ_ESHAPE;
