@@ -27,7 +27,7 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 # HBM bytes per headline launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by the
 # same counters on the plain copy kernel (2.000 and 1.000); measurement recorded in
 # profiles/gemv_q4_k_11008x4096_hbm_traffic_pmc.txt
-TRAFFIC_BYTES_PER_LAUNCH = 25531392
+TRAFFIC_BYTES_PER_LAUNCH = 25528524
 INT8_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA, published
 MALL_BYTES = 256 << 20
 
