@@ -45,6 +45,24 @@ static std::atomic<int> g_gemm_policy{0};      /* 0 automatic, 1 matrix cores ab
 
 extern "C" void ckq_launch_set_gemm_policy(int policy) { g_gemm_policy.store(policy < 0 || policy > 2 ? 0 : policy); }
 
+/* Q8_0 has its own estimate, fitted to the same kind of measurements after its
+ * streaming kernel went to aligned loads (us, weight bytes in MB): streaming
+ * 4.8 + passes * MB / 5.0 (MB / 3.6 for rows it must read with 2-byte-aligned
+ * loads), matrix cores max(14, 9 + MB / 2.5).  LM head 151936x896 (145 MB):
+ * 9-16 tokens stream (63-66 us against 67-69), 17 and more go to the matrix
+ * cores (89 against 69); 4864x896 (4.6 MB) streams up to 72 tokens (64 tokens:
+ * 11.8 us against 15.3). */
+static bool gemm_q80_on_matrix_cores(int ntok, size_t weight_bytes, bool aligned_rows)
+{
+    const int policy = g_gemm_policy.load(std::memory_order_relaxed);
+    if (ntok <= CKQ_STREAM_TOKENS || policy == 2) return false;
+    if (policy == 1) return true;
+    const float passes = (float)((ntok + CKQ_STREAM_TOKENS - 1) / CKQ_STREAM_TOKENS), mb = (float)weight_bytes * 1e-6f;
+    const float t_stream = 4.8f + passes * mb / (aligned_rows ? 5.0f : 3.6f);
+    const float t_matrix = fmaxf(14.0f, 9.0f + mb / 2.5f);
+    return t_stream > t_matrix;
+}
+
 static bool gemm_on_matrix_cores(int ntok, size_t weight_bytes, size_t budget_mb)
 {
     const int policy = g_gemm_policy.load(std::memory_order_relaxed);
@@ -385,6 +403,13 @@ static int launch_gemm_q50_via_q80(const void *A, const void *B, const float *bi
     return launch_gemm_q80_mfma(A, tmp, bias, C, M, N, K, ldc, s);
 }
 
+static bool weights_dword_aligned(const GemvArgs &a)
+{
+    uintptr_t bits = reinterpret_cast<uintptr_t>(a.W);
+    for (int i = 0; i + 1 < t_group.n; ++i) bits |= reinterpret_cast<uintptr_t>(t_group.W[i]);
+    return (bits & 3) == 0;
+}
+
 static int launch_gemv_args(int fmt, GemvArgs &a, int K, void *stream);
 
 extern "C" int ckq_launch_gemv(int fmt, float *y, const void *W, const void *X, const float *bias,
@@ -427,13 +452,6 @@ extern "C" int ckq_launch_gemv_group(int fmt, int n, float *const *y, const void
     return rc;
 }
 
-static bool weights_dword_aligned(const GemvArgs &a)
-{
-    uintptr_t bits = reinterpret_cast<uintptr_t>(a.W);
-    for (int i = 0; i + 1 < t_group.n; ++i) bits |= reinterpret_cast<uintptr_t>(t_group.W[i]);
-    return (bits & 3) == 0;
-}
-
 static int launch_gemv_args(int fmt, GemvArgs &a, int K, void *stream)
 {
     float *const y = a.y;
@@ -464,7 +482,8 @@ static int launch_gemv_args(int fmt, GemvArgs &a, int K, void *stream)
         return launch_fmt<FmtQ6K>(a, dump, 8, s);
     case CKQ_FMT_Q8_0:
         if (K % 32) return CKQ_ESHAPE;
-        if (!dump && row0 == 0 && row1 == nrows && gemm_on_matrix_cores(ntok, (size_t)nrows * (K / 32) * 34, 20))
+        if (!dump && row0 == 0 && row1 == nrows &&
+            gemm_q80_on_matrix_cores(ntok, (size_t)nrows * (K / 32) * 34, K % 64 == 0 && weights_dword_aligned(a)))
             return launch_gemm_q80_mfma(X, W, bias, y, ntok, nrows, K, ldy, s);
         a.wrow = (long)(K / 32) * 34; a.xrow = (long)(K / 32) * 34; a.nsub_row = K / 32;
         /* rows of an even number of blocks at dword-aligned addresses: two blocks per position, aligned loads */

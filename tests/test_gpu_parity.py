@@ -1057,7 +1057,8 @@ def test_fused_mlp_q5_0_gate_up_golden_case():
     ("q4_k", 4096, 4096, {8: "stream", 9: "stream", 16: "stream", 17: "matrix"}),      # 9.4 MB: two passes stream
     ("q4_k", 11008, 4096, {8: "stream", 9: "matrix"}),                                  # 25 MB
     ("q6_k", 1024, 4096, {16: "stream", 40: "stream", 49: "matrix"}),                   # 3.4 MB
-    ("q8_0", 4864, 896, {32: "stream", 33: "matrix"}),                                  # 4.4 MB
+    ("q8_0", 4864, 896, {64: "stream", 72: "stream", 73: "matrix"}),                    # 4.6 MB, aligned-load streaming
+    ("q8_0", 32000, 4096, {16: "stream", 17: "matrix"}),                                # 139 MB: two passes still stream
     ("q5_k", 4864, 1024, {64: "stream", 96: "stream", 100: "matrix"}),                  # 3.3 MB, 40 MB budget
     ("q5_0", 896, 896, {48: "stream", 57: "matrix"}),                                   # below the 3 MB floor
 ])
