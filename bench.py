@@ -2,8 +2,8 @@
 """Benchmark of the quantized dequant-dot hot path on one MI355X.
 
 A step is one pass of the hot path over one batch of synthetic input: one
-Q4_K x Q8_K GEMV, N=11008 output rows, K=4096, M=1 token (the shape
-BASELINE.json's metric is quoted on), device-resident inputs, launched
+Q4_K x Q8_K GEMV, N=11008 output rows, K=4096, M=1 token (a 7B model's
+gate/up projection at decode), device-resident inputs, launched
 back-to-back on one stream.  Consecutive steps read different copies of the
 weight matrix, enough of them to exceed the 256 MB Infinity Cache, so the
 figure is an HBM figure; the cache-resident rate is reported beside it.
@@ -208,8 +208,8 @@ def main():
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings")
     a = ap.parse_args()
     if a.gpus != 1:
-        sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported (every box here has one GPU, "
-                 "see DESIGN.md for how the path would shard)" % a.gpus)
+        sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported (the path shards by output "
+                 "rows, one all-gather per matmul; nothing here uses a second GPU)" % a.gpus)
 
     H = Harness()
     torch, P, T = H.torch, H.P, H.T
