@@ -400,13 +400,16 @@ def main():
         small = {}
         for Mb in (1, 2, 4, 8):
             xa = P.dev_quantize(P.to_device(T.normal(Mb * 1024, seed=41)), "q8_k", rows=Mb)
-            xb = P.dev_quantize(P.to_device(T.normal(Mb * 4864, seed=42)), "q8_k", rows=Mb)
             xh = P.dev_quantize(P.to_device(T.normal(Mb * 896, seed=43)), "q8_0", rows=Mb)
             layers, nbytes = [], 0
             for hi, head in enumerate(heads):
                 ops = []
-                for (r, k), Wj in zip(proj, Wp):
-                    ops.append(("q5_k", xb if k == 4864 else xa, Wj, None, torch.empty(Mb * r, dtype=torch.float32, device="cuda"), Mb, r, k))
+                for j, ((r, k), Wj) in enumerate(zip(proj, Wp)):
+                    # dependencies of a real layer, as in the 7B list: O reads Q's output buffer,
+                    # gate/up read O's, down reads up's; Q, K, V (one input, K and V narrower) and
+                    # gate, up are independent and share a launch at one token
+                    src = xa if j < 3 else ops[0][4] if j == 3 else ops[3][4] if j < 6 else ops[5][4]
+                    ops.append(("q5_k", src, Wj, None, torch.zeros(Mb * r, dtype=torch.float32, device="cuda"), Mb, r, k))
                     if hi == 0:
                         nbytes += gemv_bytes("q5_k", r, k, Mb)
                 ops.append(("q8_0", xh, head, None, torch.empty(Mb * 151936, dtype=torch.float32, device="cuda"), Mb, 151936, 896))

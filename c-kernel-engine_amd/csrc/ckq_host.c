@@ -1046,19 +1046,23 @@ static int ranges_overlap(const void *a, size_t na, const void *b, size_t nb)
     return a0 < b0 + nb && b0 < a0 + na;
 }
 
-/* Entries i and j of a sequence can share a launch when they have one format
- * and shape and neither writes what the other reads or writes. */
+/* Entries i and j of a sequence can share a launch when they have one format,
+ * input width and token count (their row counts may differ: K and V are
+ * narrower than Q under grouped-query attention) and neither writes what the
+ * other reads or writes. */
 static int ops_independent(const ckq_matmul_op *p, const ckq_matmul_op *q)
 {
-    if (p->fmt != q->fmt || p->M != q->M || p->N != q->N || p->K != q->K || p->ldc != q->ldc) return 0;
-    const size_t cb = ((size_t)(p->M - 1) * (size_t)p->ldc + (size_t)p->N) * sizeof(float);
+    if (p->fmt != q->fmt || p->M != q->M || p->K != q->K || q->N <= 0 || q->ldc < q->N || !q->A_q8 || !q->B || !q->C)
+        return 0;
+    const size_t pc = ((size_t)(p->M - 1) * (size_t)p->ldc + (size_t)p->N) * sizeof(float);
+    const size_t qc = ((size_t)(q->M - 1) * (size_t)q->ldc + (size_t)q->N) * sizeof(float);
     const size_t ab = (size_t)p->M * act_row_bytes(p->fmt, p->K);
-    const size_t wb = (size_t)p->N * weight_row_bytes(p->fmt, p->K);
-    if (ranges_overlap(p->C, cb, q->C, cb)) return 0;
-    if (ranges_overlap(p->C, cb, q->A_q8, ab) || ranges_overlap(q->C, cb, p->A_q8, ab)) return 0;
-    if (ranges_overlap(p->C, cb, q->B, wb) || ranges_overlap(q->C, cb, p->B, wb)) return 0;
-    if (p->bias && ranges_overlap(q->C, cb, p->bias, (size_t)p->N * sizeof(float))) return 0;
-    if (q->bias && ranges_overlap(p->C, cb, q->bias, (size_t)q->N * sizeof(float))) return 0;
+    const size_t pw = (size_t)p->N * weight_row_bytes(p->fmt, p->K), qw = (size_t)q->N * weight_row_bytes(q->fmt, q->K);
+    if (ranges_overlap(p->C, pc, q->C, qc)) return 0;
+    if (ranges_overlap(p->C, pc, q->A_q8, ab) || ranges_overlap(q->C, qc, p->A_q8, ab)) return 0;
+    if (ranges_overlap(p->C, pc, q->B, qw) || ranges_overlap(q->C, qc, p->B, pw)) return 0;
+    if (p->bias && ranges_overlap(q->C, qc, p->bias, (size_t)p->N * sizeof(float))) return 0;
+    if (q->bias && ranges_overlap(p->C, pc, q->bias, (size_t)q->N * sizeof(float))) return 0;
     return 1;
 }
 
@@ -1072,8 +1076,9 @@ int ckq_matmul_sequence_dev(const ckq_matmul_op *ops, int nops, int repeat, void
             /* consecutive entries of one shape that do not depend on each other
              * (Q/K/V, gate/up) go out as one launch */
             int n = 1;
-            const int groupable = o->A_q8 && o->B && o->C && o->M == 1 && o->N > 0 && o->K > 0 && o->K <= 8192 &&
-                                  o->ldc >= o->N && !is_f32act(o->fmt) && o->K % fmt_block_elems(o->fmt) == 0;
+            const int groupable = o->A_q8 && o->B && o->C && o->M >= 1 && o->M <= 8 && o->N > 0 && o->K > 0 &&
+                                  (long)o->K * o->M <= 49152 && o->ldc >= o->N && !is_f32act(o->fmt) &&
+                                  o->K % fmt_block_elems(o->fmt) == 0;
             while (groupable && n < GROUP_MAX && i + n < nops) {
                 int ok = 1;
                 for (int j = 0; j < n && ok; ++j) ok = ops_independent(&ops[i + j], &ops[i + n]);
@@ -1085,8 +1090,13 @@ int ckq_matmul_sequence_dev(const ckq_matmul_op *ops, int nops, int repeat, void
                 float *y[GROUP_MAX];
                 const void *W[GROUP_MAX], *X[GROUP_MAX];
                 const float *b[GROUP_MAX];
-                for (int j = 0; j < n; ++j) { y[j] = ops[i + j].C; W[j] = ops[i + j].B; X[j] = ops[i + j].A_q8; b[j] = ops[i + j].bias; }
-                rc = ckq_launch_gemv_group(o->fmt, n, y, W, X, b, o->N, o->K, o->M, o->ldc, stream);
+                int rows[GROUP_MAX];
+                long ld[GROUP_MAX];
+                for (int j = 0; j < n; ++j) {
+                    y[j] = ops[i + j].C; W[j] = ops[i + j].B; X[j] = ops[i + j].A_q8; b[j] = ops[i + j].bias;
+                    rows[j] = ops[i + j].N; ld[j] = ops[i + j].ldc;
+                }
+                rc = ckq_launch_gemv_group(o->fmt, n, y, W, X, b, rows, ld, o->K, o->M, stream);
             } else {
                 rc = ckq_gemm_nt_dev(o->fmt, o->A_q8, o->B, o->bias, o->C, o->M, o->N, o->K, o->ldc, stream);
             }

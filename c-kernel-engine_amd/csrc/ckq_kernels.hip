@@ -91,6 +91,8 @@ struct GemvGroup {
     const uint8_t *W[CKQ_GROUP_MAX - 1];
     const uint8_t *X[CKQ_GROUP_MAX - 1];
     const float   *bias[CKQ_GROUP_MAX - 1];
+    int nrows[CKQ_GROUP_MAX - 1];           /* rows of each further problem (the grid covers the largest) */
+    int ldy[CKQ_GROUP_MAX - 1];             /* and its output row stride */
     int n;                                  /* problems in the launch, 1 = not grouped */
 };
 
@@ -121,13 +123,15 @@ gemv_kernel(const uint8_t *W, const uint8_t *X, long wrow, long xrow, int row0, 
      * first fourteen registers' worth arrive preloaded with the wave (build
      * flag -amdgpu-kernarg-preload-count) instead of through a scalar load
      * that every wave waits for before it can issue its first weight load. */
-    const GemvArgs a = {y, W, X, bias, sub, nrows, npos, ntok, row0, row1, nsub_row, wrow, xrow, ldy};
+    const int g = GRP ? (int)blockIdx.z : 0;
+    const int row1g = GRP && g ? grp.nrows[g - 1] : row1;    /* problems of a group may differ in their row count */
+    const long ldyg = GRP && g ? (long)grp.ldy[g - 1] : ldy;
+    const GemvArgs a = {y, W, X, bias, sub, nrows, npos, ntok, row0, row1g, nsub_row, wrow, xrow, ldyg};
     constexpr int SLOTS = 64 / LPR;
     extern __shared__ __attribute__((aligned(16))) uint8_t xs[];   /* LDSX: the MT activation rows */
     /* grouped launch: blockIdx.z picks the problem (a separate instantiation: the extra
      * argument loads lengthen the start of every wave, which a bandwidth-bound launch
      * of a few microseconds feels) */
-    const int g = GRP ? (int)blockIdx.z : 0;
     float *const         gy    = g == 0 ? a.y    : grp.y[g - 1];
     const uint8_t *const gW    = g == 0 ? a.W    : grp.W[g - 1];
     const uint8_t *const gX    = g == 0 ? a.X    : grp.X[g - 1];
@@ -288,17 +292,20 @@ gemv_kernel(const uint8_t *W, const uint8_t *X, long wrow, long xrow, int row0, 
 
 /* The group of the launch in flight on this thread (set by ckq_launch_gemv_group
  * around its dispatch; every other launch sees n = 1). */
-static thread_local GemvGroup t_group = {{}, {}, {}, {}, 1};
+static thread_local GemvGroup t_group = {{}, {}, {}, {}, {}, {}, 1};
+
+/* Rows the grid has to cover: the computed range, or the largest problem of a group. */
+static int launch_rows(const GemvArgs &a) { return t_group.n > 1 ? a.nrows : a.row1 - a.row0; }
 
 template <class F, int LPR, int PPL, int MT, int RPI, bool DUMP, int WPB, bool LDSX>
 static int launch_one(const GemvArgs &a, hipStream_t s)
 {
     constexpr int rows_per_block = WPB * (64 / LPR) * RPI;
-    const int nr = a.row1 - a.row0;
+    const int nr = launch_rows(a);
     dim3 grid((nr + rows_per_block - 1) / rows_per_block, (a.ntok + MT - 1) / MT, 1);
     const size_t lds = LDSX ? F::xs_lds_bytes((size_t)MT * (size_t)a.xrow) : 0;
     if (t_group.n > 1) {
-        if constexpr (MT == 1 && !DUMP && LDSX) {        /* grouped launches are single-token */
+        if constexpr (!DUMP && LDSX) {                   /* grouped launches stage their activations in LDS */
             grid.z = (unsigned)t_group.n;
             hipLaunchKernelGGL((gemv_kernel<F, LPR, PPL, MT, RPI, DUMP, WPB, LDSX, true>), grid, dim3(64 * WPB), lds, s,
                                a.W, a.X, a.wrow, a.xrow, a.row0, a.row1, a.npos, a.ntok, a.y, a.bias, a.ldy, a.sub,
@@ -336,14 +343,14 @@ static int launch_mt(const GemvArgs &a, bool dump, int max_mt, hipStream_t s)
         /* 256-thread blocks; a second row per slot once the matrix needs more
          * than two rounds of resident waves anyway (halves the activation
          * staging per weight byte) */
-        const long waves = ((long)(a.row1 - a.row0) * LPR + 63) / 64;
+        const long waves = ((long)launch_rows(a) * LPR + 63) / 64;
         if (PPL == 1 && waves > 16384) return launch_tile<F, LPR, PPL, 1, 2, 4>(a, s);
         /* rows longer than one pass: each staged activation row is shared
          * between eight weight rows, as 512-thread blocks (a whole number of
          * blocks per CU on the usual projection shapes) or, for the largest
          * matrices, two rows per slot */
-        if (PPL > 1 && a.row1 - a.row0 >= 8192) return launch_tile<F, LPR, PPL, 1, 2, 4>(a, s);
-        if (PPL > 1 && a.row1 - a.row0 >= 2048) return launch_tile<F, LPR, PPL, 1, 1, 8>(a, s);
+        if (PPL > 1 && launch_rows(a) >= 8192) return launch_tile<F, LPR, PPL, 1, 2, 4>(a, s);
+        if (PPL > 1 && launch_rows(a) >= 2048) return launch_tile<F, LPR, PPL, 1, 1, 8>(a, s);
         return launch_tile<F, LPR, PPL, 1, 1, 4>(a, s);
     }
     if constexpr (F::TOKEN_TILES) {
@@ -427,24 +434,38 @@ extern "C" int ckq_launch_gemv(int fmt, float *y, const void *W, const void *X, 
     return launch_gemv_args(fmt, a, K, stream);
 }
 
-/* `n` (2..CKQ_GROUP_MAX) independent matmuls of one format and shape - the
- * Q/K/V or the gate/up projections of a token - as one launch of the streaming
+/* `n` (2..CKQ_GROUP_MAX) independent matmuls of one format and input width,
+ * each with its own number of rows - the Q/K/V (grouped-query attention makes
+ * K and V narrower than Q) or the gate/up projections of a token - as one
+ * launch of the streaming
  * kernel: the launches' fixed start-up cost is paid once and the chip holds n
- * times the loads in flight.  One token (decode); K up to 8192 elements. */
+ * times the loads in flight.  Up to eight tokens, K * tokens <= 49152. */
 extern "C" int ckq_launch_gemv_group(int fmt, int n, float *const *y, const void *const *W, const void *const *X,
-                                     const float *const *bias, int nrows, int K, int ntok, long ldy, void *stream)
+                                     const float *const *bias, const int *rows, const long *ldys, int K, int ntok,
+                                     void *stream)
 {
-    if (n < 1 || n > CKQ_GROUP_MAX || !y || !W || !X || nrows <= 0 || K <= 0 || ntok != 1) return CKQ_EINVAL;
-    /* the activation row is staged in LDS in every grouped kernel */
-    if ((size_t)K * 4 > 32768) return CKQ_ESHAPE;
+    if (n < 1 || n > CKQ_GROUP_MAX || !y || !W || !X || !rows || !ldys || K <= 0 || ntok < 1 || ntok > CKQ_STREAM_TOKENS)
+        return CKQ_EINVAL;
+    int nrows = 0;                                  /* the grid and the launch shape follow the largest problem */
+    for (int i = 0; i < n; ++i) {
+        if (rows[i] <= 0) return CKQ_EINVAL;
+        if (rows[i] > nrows) nrows = rows[i];
+    }
+    for (int i = 0; i < n; ++i)
+        if (ldys[i] < rows[i] || ldys[i] > 0x7fffffff) return CKQ_EINVAL;
+    const long ldy = ldys[0];
+    /* the activation tile is staged in LDS in every grouped kernel: K * ntok is bounded */
+    if ((size_t)K * (size_t)ntok > 49152) return CKQ_ESHAPE;
     for (int i = 0; i < n; ++i)
         if (!y[i] || !W[i] || !X[i]) return CKQ_EINVAL;
     GemvArgs a = {};
     a.y = y[0]; a.W = (const uint8_t *)W[0]; a.X = (const uint8_t *)X[0]; a.bias = bias ? bias[0] : nullptr; a.sub = nullptr;
-    a.nrows = nrows; a.ntok = ntok; a.row0 = 0; a.row1 = nrows; a.ldy = ldy;
+    a.nrows = nrows; a.ntok = ntok; a.row0 = 0; a.row1 = rows[0]; a.ldy = ldy;
     for (int i = 1; i < n; ++i) {
         t_group.y[i - 1] = y[i]; t_group.W[i - 1] = (const uint8_t *)W[i]; t_group.X[i - 1] = (const uint8_t *)X[i];
         t_group.bias[i - 1] = bias ? bias[i] : nullptr;
+        t_group.nrows[i - 1] = rows[i];
+        t_group.ldy[i - 1] = (int)ldys[i];
     }
     t_group.n = n;
     const int rc = launch_gemv_args(fmt, a, K, stream);

@@ -38,11 +38,14 @@ int ckq_launch_gemv(int fmt, float *y, const void *W, const void *X, const float
                     int nrows, int K, int ntok, long ldy, int row0, int row1,
                     int32_t *subdots, void *stream);
 
-/* n (at most 4) independent single-token matmuls of one format and shape
- * (K <= 8192) in one launch of the streaming kernel; pointer arrays are host
- * arrays of device pointers, bias may be NULL or hold NULL entries. */
+/* n (at most 4) independent matmuls of one format, input width and token count
+ * (at most eight tokens, K * tokens <= 49152), problem i with rows[i] weight
+ * rows and output row stride ldys[i], in one launch of the streaming kernel;
+ * the arrays are host arrays (of device pointers), bias may be NULL or hold
+ * NULL entries. */
 int ckq_launch_gemv_group(int fmt, int n, float *const *y, const void *const *W, const void *const *X,
-                          const float *const *bias, int nrows, int K, int ntok, long ldy, void *stream);
+                          const float *const *bias, const int *rows, const long *ldys, int K, int ntok,
+                          void *stream);
 
 /* Kernel choice for more than eight tokens: 0 = by token count and weight size
  * (default), 1 = always the matrix-core GEMM, 2 = always the streaming kernel. */

@@ -245,9 +245,10 @@ int ckq_gemm_nt_f32act_dev(int fmt, const float *A, const void *B, const float *
 /* A list of matmuls enqueued back-to-back, the whole list `repeat` times: the
  * per-token projection set of a decoder layer (Q/K/V/O, gate/up, down) is one
  * such list.  Entry i computes C[m*ldc + n] as ckq_gemm_nt_dev does, with the
- * same bits.  Up to four consecutive single-token entries of one format and
- * shape (K <= 8192), none of which writes memory another reads or writes
- * (Q/K/V, gate/up of a decode step), are issued as ONE launch. */
+ * same bits.  Up to four consecutive entries of one format, input width and
+ * token count (at most eight tokens, K * tokens <= 49152; their row counts may
+ * differ), none of which writes memory another reads or writes (Q/K/V,
+ * gate/up of a decode step), are issued as ONE launch. */
 typedef struct {
     int          fmt;    /* ckq_format weight tag */
     int          M;      /* tokens */

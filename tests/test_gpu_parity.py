@@ -1089,27 +1089,29 @@ def test_gemm_automatic_kernel_choice(fmt, N, K, expect):
 
 @pytest.mark.parametrize("fmt,N,K", [("q4_k", 384, 1024), ("q6_k", 200, 512), ("q8_0", 130, 896), ("q5_k", 96, 768)])
 def test_matmul_sequence_groups_independent_entries(fmt, N, K):
-    """Q/K/V-like entries (one input, separate weights and outputs) and a pair
-    with separate inputs go out as grouped launches; every output has the bits
-    of the same matmul launched alone, with and without biases, for one and
-    several tokens, and the oracle's values."""
+    """Q/K/V-like entries (one input, separate weights and outputs, K and V
+    narrower than Q) and a pair with separate inputs go out as grouped launches
+    at one token; every output has the bits of the same matmul launched alone,
+    with and without biases, for one and several tokens, and the oracle's
+    values."""
     import torch
+    Ns = [N, N // 4 + 1, N // 4 + 1, N, N + 5, 2 * N]
     for M in (1, 3, 8):
-        Ws = [T.random_blocks(fmt, N * (K // T.ELEMS[fmt]), 700 + i) for i in range(6)]
+        Ws = [T.random_blocks(fmt, Ns[i] * (K // T.ELEMS[fmt]), 700 + i) for i in range(6)]
         xs = [T.oracle_quantize(T.normal(M * K, 0.0, 1.0, 800 + i), T.act_fmt(fmt), rows=M) for i in range(2)]
-        bias = [T.normal(N, 0.0, 0.5, seed=900 + i) if i % 2 else None for i in range(6)]
+        bias = [T.normal(Ns[i], 0.0, 0.5, seed=900 + i) if i % 2 else None for i in range(6)]
         Wd = [P.to_device(w) for w in Ws]
         xd = [P.to_device(x) for x in xs]
         bd = [None if b is None else P.to_device(b) for b in bias]
         inp = [0, 0, 0, 1, 0, 1]                       # entries 0-2 share an input; 3-5 alternate
-        outs = [torch.full((M * N,), 7.0, dtype=torch.float32, device="cuda") for _ in range(6)]
+        outs = [torch.full((M * Ns[i],), 7.0, dtype=torch.float32, device="cuda") for i in range(6)]
         say("sequence grouping", fmt, M)
-        P.dev_matmul_sequence([(fmt, xd[inp[i]], Wd[i], bd[i], outs[i], M, N, K) for i in range(6)])
+        P.dev_matmul_sequence([(fmt, xd[inp[i]], Wd[i], bd[i], outs[i], M, Ns[i], K) for i in range(6)])
         for i in range(6):
-            alone = P.dev_gemm_nt(fmt, xd[inp[i]], Wd[i], bd[i], M, N, K).cpu().numpy()
-            got = outs[i].cpu().numpy().reshape(M, N)
+            alone = P.dev_gemm_nt(fmt, xd[inp[i]], Wd[i], bd[i], M, Ns[i], K).cpu().numpy()
+            got = outs[i].cpu().numpy().reshape(M, Ns[i])
             assert np.array_equal(got, alone), (M, i)
-            assert T.norm_err(got, T.oracle_gemm_nt(fmt, xs[inp[i]], Ws[i], bias[i], M, N, K)) <= TOL, (M, i)
+            assert T.norm_err(got, T.oracle_gemm_nt(fmt, xs[inp[i]], Ws[i], bias[i], M, Ns[i], K)) <= TOL, (M, i)
 
 
 def test_matmul_sequence_keeps_order_where_entries_depend():
