@@ -39,6 +39,7 @@ typedef struct {
     uint64_t    fp;
     void       *dev;
     int         pinned;   /* registered by the caller: serves any sub-range, content is not re-checked */
+    uint64_t    last_use; /* value of g_use_clock at the last hit (eviction order of unpinned entries) */
 } weight_entry;
 
 typedef struct {
@@ -50,13 +51,14 @@ enum { BUF_X = 0, BUF_Y, BUF_BIAS, BUF_Q, BUF_GU, BUF_H, BUF_COUNT };
 
 static pthread_mutex_t g_mu = PTHREAD_MUTEX_INITIALIZER;
 static int          g_inited = 0;
-static int          g_err = 0;
+static int          g_err = 0;            /* accessed with __atomic builtins: any thread may fail */
 static int          g_cache_on = 1;
 static int          g_parallel_whole = 0;
 static hipStream_t  g_stream = NULL;
 static dev_buf      g_buf[BUF_COUNT];
 static weight_entry *g_w = NULL;
 static size_t       g_nw = 0, g_capw = 0;
+static size_t       g_cache_max_bytes = (size_t)64 << 30;   /* bound on unpinned resident weights */
 
 /* ------------------------------------------------------------------------ */
 /* Errors                                                                    */
@@ -73,13 +75,13 @@ const char *ckq_error_string(int code)
     }
 }
 
-int ckq_last_error(void) { return g_err; }
-void ckq_clear_error(void) { g_err = 0; }
+int ckq_last_error(void) { return __atomic_load_n(&g_err, __ATOMIC_RELAXED); }
+void ckq_clear_error(void) { __atomic_store_n(&g_err, 0, __ATOMIC_RELAXED); }
 
 static int fail(int code, const char *what)
 {
     if (code == 0) return 0;
-    g_err = code;
+    __atomic_store_n(&g_err, code, __ATOMIC_RELAXED);
     fprintf(stderr, "libckernel_quant_hip: %s failed: %s (%d)\n", what, ckq_error_string(code), code);
     const char *e = getenv("CKQ_ABORT_ON_ERROR");
     if (!e || strcmp(e, "0") != 0) {
@@ -94,6 +96,11 @@ static int fail(int code, const char *what)
         hipError_t e_ = (expr);                         \
         if (e_ != hipSuccess) return fail((int)e_, #expr); \
     } while (0)
+
+/* An error path leaves its do-block after copies from the caller's buffers
+ * may have been enqueued: wait for them, so that with CKQ_ABORT_ON_ERROR=0 the
+ * call does not return while the device still reads the caller's memory. */
+static void drain_after_error(void);
 
 /* ------------------------------------------------------------------------ */
 /* Init, buffers, pointer classification                                     */
@@ -117,6 +124,8 @@ static int init_locked(void)
     HIP_TRY(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
     const char *c = getenv("CKQ_WEIGHT_CACHE");
     if (c && strcmp(c, "0") == 0) g_cache_on = 0;
+    const char *mb = getenv("CKQ_WEIGHT_CACHE_MB");
+    if (mb && atoll(mb) > 0) g_cache_max_bytes = (size_t)atoll(mb) << 20;
     const char *p = getenv("CKQ_PARALLEL_MODE");
     if (p && strcmp(p, "whole") == 0) g_parallel_whole = 1;
     const char *gp = getenv("CKQ_GEMM_POLICY");
@@ -124,6 +133,14 @@ static int init_locked(void)
     if (gp && strcmp(gp, "stream") == 0) ckq_launch_set_gemm_policy(CKQ_GEMM_STREAM);
     g_inited = 1;
     return 0;
+}
+
+static void drain_after_error(void)
+{
+    if (g_inited && g_stream) {
+        (void)hipStreamSynchronize(g_stream);
+        (void)hipGetLastError();
+    }
 }
 
 int ckq_init(void)
@@ -212,6 +229,39 @@ static uint64_t fingerprint(const void *p, size_t bytes)
     return h;
 }
 
+/* The table of unpinned entries is bounded: beyond CACHE_MAX_ENTRIES entries
+ * or g_cache_max_bytes bytes (CKQ_WEIGHT_CACHE_MB, default 64 GiB) the least
+ * recently used unpinned entry is dropped.  Registered regions are never
+ * evicted. */
+enum { CACHE_MAX_ENTRIES = 4096 };
+static uint64_t g_use_clock = 0;
+
+static size_t cache_unpinned_bytes(void)
+{
+    size_t b = 0;
+    for (size_t i = 0; i < g_nw; ++i)
+        if (!g_w[i].pinned) b += g_w[i].bytes;
+    return b;
+}
+
+static void drop_entry(size_t i);
+
+/* Make room for a new unpinned entry of `bytes`. */
+static void cache_evict_for(size_t bytes)
+{
+    for (;;) {
+        size_t n_unpinned = 0, lru = (size_t)-1;
+        for (size_t i = 0; i < g_nw; ++i) {
+            if (g_w[i].pinned) continue;
+            ++n_unpinned;
+            if (lru == (size_t)-1 || g_w[i].last_use < g_w[lru].last_use) lru = i;
+        }
+        if (lru == (size_t)-1) return;
+        if (n_unpinned < CACHE_MAX_ENTRIES && cache_unpinned_bytes() + bytes <= g_cache_max_bytes) return;
+        drop_entry(lru);
+    }
+}
+
 static int weights_lookup(const void *W, size_t bytes, const void **out)
 {
     if (is_device_ptr(W)) {
@@ -229,17 +279,20 @@ static int weights_lookup(const void *W, size_t bytes, const void **out)
     const uint64_t fp = fingerprint(W, bytes);
     for (size_t i = 0; i < g_nw; ++i) {
         if (g_w[i].host == W && g_w[i].bytes == bytes) {
+            g_w[i].last_use = ++g_use_clock;
             if (g_w[i].fp == fp) {
                 *out = g_w[i].dev;
                 return 0;
             }
-            /* same address, new content: refresh in place */
+            /* same address, new content: refresh in place; the old fingerprint
+             * stays if the copy cannot be enqueued */
             HIP_TRY(hipMemcpyAsync(g_w[i].dev, W, bytes, hipMemcpyHostToDevice, g_stream));
             g_w[i].fp = fp;
             *out = g_w[i].dev;
             return 0;
         }
     }
+    cache_evict_for(bytes);
     if (g_nw == g_capw) {
         size_t nc = g_capw ? g_capw * 2 : 64;
         weight_entry *nw = (weight_entry *)realloc(g_w, nc * sizeof(*nw));
@@ -249,44 +302,68 @@ static int weights_lookup(const void *W, size_t bytes, const void **out)
     }
     void *d = NULL;
     HIP_TRY(hipMalloc(&d, bytes));
-    HIP_TRY(hipMemcpyAsync(d, W, bytes, hipMemcpyHostToDevice, g_stream));
+    hipError_t e = hipMemcpyAsync(d, W, bytes, hipMemcpyHostToDevice, g_stream);
+    if (e != hipSuccess) {                       /* no entry for a failed upload */
+        (void)hipFree(d);
+        return fail((int)e, "upload weights");
+    }
     g_w[g_nw].host = W;
     g_w[g_nw].bytes = bytes;
     g_w[g_nw].fp = fp;
     g_w[g_nw].dev = d;
     g_w[g_nw].pinned = 0;
+    g_w[g_nw].last_use = ++g_use_clock;
     g_nw++;
     *out = d;
     return 0;
 }
 
-/* Uncached weights share no staging buffer with activations: they get their
- * own grow-only device buffer. */
-static dev_buf g_wtmp;
-static int weights_uncached(const void *W, size_t bytes, const void **out)
+/* Uncached weights share no staging buffer with activations: every weight
+ * operand of a call gets its own grow-only device buffer (`slot`), so a call
+ * with two weight matrices (the fused MLP) keeps both alive until its kernels
+ * have been enqueued. */
+enum { WTMP_SLOTS = 2 };
+static dev_buf g_wtmp[WTMP_SLOTS];
+static int weights_uncached(int slot, const void *W, size_t bytes, const void **out)
 {
-    if (g_wtmp.cap < bytes) {
-        if (g_wtmp.dev) {
+    dev_buf *b = &g_wtmp[slot];
+    if (b->cap < bytes) {
+        if (b->dev) {
             HIP_TRY(hipStreamSynchronize(g_stream));
-            HIP_TRY(hipFree(g_wtmp.dev));
-            g_wtmp.dev = NULL;
-            g_wtmp.cap = 0;
+            HIP_TRY(hipFree(b->dev));
+            b->dev = NULL;
+            b->cap = 0;
         }
-        HIP_TRY(hipMalloc(&g_wtmp.dev, bytes));
-        g_wtmp.cap = bytes;
+        HIP_TRY(hipMalloc(&b->dev, bytes));
+        b->cap = bytes;
     }
-    HIP_TRY(hipMemcpyAsync(g_wtmp.dev, W, bytes, hipMemcpyHostToDevice, g_stream));
-    *out = g_wtmp.dev;
+    HIP_TRY(hipMemcpyAsync(b->dev, W, bytes, hipMemcpyHostToDevice, g_stream));
+    *out = b->dev;
     return 0;
 }
 
-static int weights_resolve(const void *W, size_t bytes, const void **out)
+enum { CACHE_MIN_BYTES = 64 * 1024 };
+static int in_registered_region(const void *W, size_t bytes)
+{
+    for (size_t i = 0; i < g_nw; ++i) {
+        const uint8_t *h = (const uint8_t *)g_w[i].host, *w = (const uint8_t *)W;
+        if (g_w[i].pinned && w >= h && w + bytes <= h + g_w[i].bytes) return 1;
+    }
+    return 0;
+}
+
+/* Device view of weight operand number `slot` (0 or 1) of the current call. */
+static int weights_resolve(int slot, const void *W, size_t bytes, const void **out)
 {
     if (is_device_ptr(W)) {
         *out = W;
         return 0;
     }
-    if (!g_cache_on) return weights_uncached(W, bytes, out);
+    if (!g_cache_on) return weights_uncached(slot, W, bytes, out);
+    /* Operands under 64 KiB (a single row handed to a vec_dot, a parity
+     * harness's scratch matrix) are cheaper to copy than to track: a per-row
+     * loop over a large matrix would otherwise leave one allocation per row. */
+    if (bytes < CACHE_MIN_BYTES && !in_registered_region(W, bytes)) return weights_uncached(slot, W, bytes, out);
     return weights_lookup(W, bytes, out);
 }
 
@@ -452,10 +529,11 @@ static size_t act_row_bytes(int fmt, int K)
 static void matmul_locked(int fmt, const void *A, const void *B, const float *bias, float *C,
                           int ntok, int nrows, int K, long ldc, int row0, int row1)
 {
+    int done = 0;
     do {
         if (init_locked()) break;
         const void *dB, *dA, *dbias = NULL;
-        if (weights_resolve(B, (size_t)nrows * weight_row_bytes(fmt, K), &dB)) break;
+        if (weights_resolve(0, B, (size_t)nrows * weight_row_bytes(fmt, K), &dB)) break;
         if (stage_in(BUF_X, A, (size_t)ntok * act_row_bytes(fmt, K), &dA)) break;
         if (bias && stage_in(BUF_BIAS, bias, (size_t)nrows * sizeof(float), &dbias)) break;
         const int c_on_dev = is_device_ptr(C);
@@ -484,7 +562,9 @@ static void matmul_locked(int fmt, const void *A, const void *B, const float *bi
         }
         hipError_t e = hipStreamSynchronize(g_stream);
         if (e != hipSuccess) fail((int)e, "hipStreamSynchronize");
+        done = 1;
     } while (0);
+    if (!done) drain_after_error();
 }
 
 static void host_matmul(int fmt, const void *A, const void *B, const float *bias, float *C,
@@ -533,6 +613,7 @@ static void host_quantize(int q8k, const float *x, void *y, int rows, int k)
     const size_t in_bytes = (size_t)rows * k * 4;
     const size_t out_bytes = (size_t)rows * ckq_row_bytes(q8k ? CKQ_FMT_Q8_K : CKQ_FMT_Q8_0, k);
     pthread_mutex_lock(&g_mu);
+    int done = 0;
     do {
         if (init_locked()) break;
         const void *dx;
@@ -549,7 +630,9 @@ static void host_quantize(int q8k, const float *x, void *y, int rows, int k)
         }
         hipError_t e = hipStreamSynchronize(g_stream);
         if (e != hipSuccess) fail((int)e, "hipStreamSynchronize");
+        done = 1;
     } while (0);
+    if (!done) drain_after_error();
     pthread_mutex_unlock(&g_mu);
 }
 
@@ -562,6 +645,7 @@ static void host_matmul_f32act(int fmt, const float *A, const void *B, const flo
     if (K % (q8k ? 256 : 32)) return;
     pthread_mutex_lock(&g_mu);
     void *dq = NULL;
+    int done = 0;
     do {
         if (init_locked()) break;
         const void *dA;
@@ -573,7 +657,9 @@ static void host_matmul_f32act(int fmt, const float *A, const void *B, const flo
         /* dq is a device pointer, so the second stage uses it in place; work
          * on one stream runs in order. */
         matmul_locked(fmt, dq, B, bias, C, ntok, nrows, K, ldc, 0, nrows);
+        done = 1;
     } while (0);
+    if (!done) drain_after_error();
     pthread_mutex_unlock(&g_mu);
 }
 
@@ -703,10 +789,11 @@ static void host_dequant_rows(int fmt, const void *table, size_t table_rows, con
     if (tokens < 0) tokens = 0;
     if (tokens > n_out_rows) tokens = n_out_rows;
     pthread_mutex_lock(&g_mu);
+    int done = 0;
     do {
         if (init_locked()) break;
         const void *dT, *dids = NULL, *dpos = NULL;
-        if (weights_resolve(table, table_rows * ckq_row_bytes(fmt, n_row), &dT)) break;
+        if (weights_resolve(0, table, table_rows * ckq_row_bytes(fmt, n_row), &dT)) break;
         if (ids && tokens > 0 && stage_in(BUF_X, ids, (size_t)tokens * sizeof(int32_t), &dids)) break;
         if (pos && tokens > 0 && stage_in(BUF_BIAS, pos, (size_t)tokens * n_row * sizeof(float), &dpos)) break;
         const size_t out_bytes = (size_t)n_out_rows * n_row * sizeof(float);
@@ -722,7 +809,9 @@ static void host_dequant_rows(int fmt, const void *table, size_t table_rows, con
         }
         hipError_t e = hipStreamSynchronize(g_stream);
         if (e != hipSuccess) fail((int)e, "hipStreamSynchronize");
+        done = 1;
     } while (0);
+    if (!done) drain_after_error();
     pthread_mutex_unlock(&g_mu);
 }
 
@@ -767,6 +856,7 @@ void rmsnorm_q8_k_fused(const float *input, const float *gamma, void *vy, int to
     const size_t in_bytes = ((size_t)(tokens - 1) * aligned_embed_dim + d_model) * 4;
     const size_t out_bytes = (size_t)tokens * ckq_row_bytes(CKQ_FMT_Q8_K, d_model);
     pthread_mutex_lock(&g_mu);
+    int done = 0;
     do {
         if (init_locked()) break;
         const void *dx, *dg;
@@ -784,18 +874,21 @@ void rmsnorm_q8_k_fused(const float *input, const float *gamma, void *vy, int to
         }
         hipError_t e = hipStreamSynchronize(g_stream);
         if (e != hipSuccess) fail((int)e, "hipStreamSynchronize");
+        done = 1;
     } while (0);
+    if (!done) drain_after_error();
     pthread_mutex_unlock(&g_mu);
 }
 
 /* Fused prefill MLP: Q8_0 quantization, one GEMM over the stacked gate and up
  * rows, SiLU(gate)*up quantized to Q8_K, the down GEMM.  The four kernels run
  * back to back on the library's stream; intermediates never leave the device. */
-void fused_mlp_swiglu_prefill_w1w2_quant(const float *x, const void *W1, const float *B1, int w1_dt,
-                                         const void *W2, const float *B2, int w2_dt, float *output,
+void fused_mlp_swiglu_prefill_w1w2_quant(const float *x, const void *W1, const float *B1, ckq_ck_dtype w1_dt_e,
+                                         const void *W2, const float *B2, ckq_ck_dtype w2_dt_e, float *output,
                                          int seq_len, int embed_dim, int aligned_embed_dim,
                                          int intermediate_dim, int aligned_intermediate_dim, void *scratch)
 {
+    const int w1_dt = (int)w1_dt_e, w2_dt = (int)w2_dt_e;
     if (!x || !W1 || !W2 || !output || !scratch) return;
     if (seq_len <= 0 || embed_dim <= 0 || aligned_embed_dim <= 0 || intermediate_dim <= 0 ||
         aligned_intermediate_dim <= 0)
@@ -809,13 +902,14 @@ void fused_mlp_swiglu_prefill_w1w2_quant(const float *x, const void *W1, const f
     const int fmt2 = w2_dt == CKQ_CK_DT_Q4_K ? CKQ_FMT_Q4_K : CKQ_FMT_Q6_K;
     const size_t out_bytes = (size_t)seq_len * E * 4;
     pthread_mutex_lock(&g_mu);
+    int done = 0;
     do {
         if (init_locked()) break;
         const void *dx, *dW1, *dW2, *dB1 = NULL, *dB2 = NULL;
         void *dq, *dgu, *dh;
         if (stage_in(BUF_X, x, (size_t)seq_len * E * 4, &dx)) break;
-        if (weights_resolve(W1, (size_t)2 * I * weight_row_bytes(fmt1, E), &dW1)) break;
-        if (weights_resolve(W2, (size_t)E * weight_row_bytes(fmt2, I), &dW2)) break;
+        if (weights_resolve(0, W1, (size_t)2 * I * weight_row_bytes(fmt1, E), &dW1)) break;
+        if (weights_resolve(1, W2, (size_t)E * weight_row_bytes(fmt2, I), &dW2)) break;
         /* both biases share the bias staging buffer: B1 first, B2 behind it */
         if (B1 || B2) {
             const int b1_dev = B1 && is_device_ptr(B1), b2_dev = B2 && is_device_ptr(B2);
@@ -856,7 +950,9 @@ void fused_mlp_swiglu_prefill_w1w2_quant(const float *x, const void *W1, const f
         }
         hipError_t e = hipStreamSynchronize(g_stream);
         if (e != hipSuccess) fail((int)e, "hipStreamSynchronize");
+        done = 1;
     } while (0);
+    if (!done) drain_after_error();
     pthread_mutex_unlock(&g_mu);
 }
 
@@ -1077,8 +1173,7 @@ int ckq_matmul_sequence_dev(const ckq_matmul_op *ops, int nops, int repeat, void
              * (Q/K/V, gate/up) go out as one launch */
             int n = 1;
             const int groupable = o->A_q8 && o->B && o->C && o->M >= 1 && o->M <= 8 && o->N > 0 && o->K > 0 &&
-                                  (long)o->K * o->M <= 49152 && o->ldc >= o->N && !is_f32act(o->fmt) &&
-                                  o->K % fmt_block_elems(o->fmt) == 0;
+                                  o->ldc >= o->N && !is_f32act(o->fmt) && o->K % fmt_block_elems(o->fmt) == 0;
             while (groupable && n < GROUP_MAX && i + n < nops) {
                 int ok = 1;
                 for (int j = 0; j < n && ok; ++j) ok = ops_independent(&ops[i + j], &ops[i + n]);

@@ -297,27 +297,51 @@ static thread_local GemvGroup t_group = {{}, {}, {}, {}, {}, {}, 1};
 /* Rows the grid has to cover: the computed range, or the largest problem of a group. */
 static int launch_rows(const GemvArgs &a) { return t_group.n > 1 ? a.nrows : a.row1 - a.row0; }
 
+/* Token tiles a launch can carry in gridDim.y; longer token lists go out as
+ * several launches over consecutive token ranges. */
+constexpr int CKQ_GRID_Y_MAX = 65535;
+
+/* Token range [t, t + n) of a launch chunked over gridDim.y: chunk c of size
+ * `per` tokens.  Host arithmetic only (also used by the index test). */
+extern "C" void ckq_grid_chunk(long total, long per, long c, long *first, long *count)
+{
+    *first = c * per;
+    *count = total - *first < per ? total - *first : per;
+    if (*count < 0) *count = 0;
+}
+
 template <class F, int LPR, int PPL, int MT, int RPI, bool DUMP, int WPB, bool LDSX>
-static int launch_one(const GemvArgs &a, hipStream_t s)
+static int launch_one(const GemvArgs &a0, hipStream_t s)
 {
     constexpr int rows_per_block = WPB * (64 / LPR) * RPI;
-    const int nr = launch_rows(a);
-    dim3 grid((nr + rows_per_block - 1) / rows_per_block, (a.ntok + MT - 1) / MT, 1);
-    const size_t lds = LDSX ? F::xs_lds_bytes((size_t)MT * (size_t)a.xrow) : 0;
+    const int nr = launch_rows(a0);
+    const size_t lds = LDSX ? F::xs_lds_bytes((size_t)MT * (size_t)a0.xrow) : 0;
     if (t_group.n > 1) {
         if constexpr (!DUMP && LDSX) {                   /* grouped launches stage their activations in LDS */
-            grid.z = (unsigned)t_group.n;
+            dim3 grid((nr + rows_per_block - 1) / rows_per_block, (a0.ntok + MT - 1) / MT, (unsigned)t_group.n);
             hipLaunchKernelGGL((gemv_kernel<F, LPR, PPL, MT, RPI, DUMP, WPB, LDSX, true>), grid, dim3(64 * WPB), lds, s,
-                               a.W, a.X, a.wrow, a.xrow, a.row0, a.row1, a.npos, a.ntok, a.y, a.bias, a.ldy, a.sub,
-                               a.nsub_row, a.nrows, t_group);
+                               a0.W, a0.X, a0.wrow, a0.xrow, a0.row0, a0.row1, a0.npos, a0.ntok, a0.y, a0.bias, a0.ldy, a0.sub,
+                               a0.nsub_row, a0.nrows, t_group);
             return (int)hipGetLastError();
         }
         return CKQ_EINVAL;
     }
-    hipLaunchKernelGGL((gemv_kernel<F, LPR, PPL, MT, RPI, DUMP, WPB, LDSX>), grid, dim3(64 * WPB), lds, s,
-                       a.W, a.X, a.wrow, a.xrow, a.row0, a.row1, a.npos, a.ntok, a.y, a.bias, a.ldy, a.sub,
-                       a.nsub_row, a.nrows, t_group);
-    return (int)hipGetLastError();
+    const long per = (long)MT * CKQ_GRID_Y_MAX;
+    for (long c = 0; c * per < a0.ntok; ++c) {
+        long first, count;
+        ckq_grid_chunk(a0.ntok, per, c, &first, &count);
+        GemvArgs a = a0;
+        a.X = a0.X + (size_t)first * (size_t)a0.xrow;
+        a.y = a0.y ? a0.y + (size_t)first * (size_t)a0.ldy : nullptr;
+        a.ntok = (int)count;
+        dim3 grid((nr + rows_per_block - 1) / rows_per_block, (a.ntok + MT - 1) / MT, 1);
+        hipLaunchKernelGGL((gemv_kernel<F, LPR, PPL, MT, RPI, DUMP, WPB, LDSX>), grid, dim3(64 * WPB), lds, s,
+                           a.W, a.X, a.wrow, a.xrow, a.row0, a.row1, a.npos, a.ntok, a.y, a.bias, a.ldy, a.sub,
+                           a.nsub_row, a.nrows, t_group);
+        const int rc = (int)hipGetLastError();
+        if (rc) return rc;
+    }
+    return 0;
 }
 
 /* Activation rows are staged in LDS when the token tile fits in 64 KB. */
@@ -434,12 +458,29 @@ extern "C" int ckq_launch_gemv(int fmt, float *y, const void *W, const void *X, 
     return launch_gemv_args(fmt, a, K, stream);
 }
 
+/* LDS bytes of the staged token tile of a grouped launch against the 64 KB a
+ * block may use: MT rows of activations, MT = token count rounded up to the
+ * tile sizes launch_mt knows (1, 2, 4, 8); Q8_0 activations are re-laid out to
+ * 36 bytes per block. */
+static bool group_tile_fits_lds(int fmt, int K, int ntok)
+{
+    const size_t mt = ntok <= 1 ? 1 : ntok == 2 ? 2 : ntok <= 4 ? 4 : 8;
+    size_t bytes;
+    switch (fmt) {
+    case CKQ_FMT_Q4_K: case CKQ_FMT_Q5_K: case CKQ_FMT_Q6_K: bytes = FmtQ4K::xs_lds_bytes(mt * (size_t)(K / 256) * 292); break;
+    case CKQ_FMT_Q8_0: case CKQ_FMT_Q5_0:                     bytes = FmtQ80::xs_lds_bytes(mt * (size_t)(K / 32) * 34); break;
+    default: return false;
+    }
+    return bytes <= 65536;
+}
+
 /* `n` (2..CKQ_GROUP_MAX) independent matmuls of one format and input width,
  * each with its own number of rows - the Q/K/V (grouped-query attention makes
  * K and V narrower than Q) or the gate/up projections of a token - as one
  * launch of the streaming
  * kernel: the launches' fixed start-up cost is paid once and the chip holds n
- * times the loads in flight.  Up to eight tokens, K * tokens <= 49152. */
+ * times the loads in flight.  Up to eight tokens; a token tile too large for
+ * LDS is issued as separate launches. */
 extern "C" int ckq_launch_gemv_group(int fmt, int n, float *const *y, const void *const *W, const void *const *X,
                                      const float *const *bias, const int *rows, const long *ldys, int K, int ntok,
                                      void *stream)
@@ -454,10 +495,19 @@ extern "C" int ckq_launch_gemv_group(int fmt, int n, float *const *y, const void
     for (int i = 0; i < n; ++i)
         if (ldys[i] < rows[i] || ldys[i] > 0x7fffffff) return CKQ_EINVAL;
     const long ldy = ldys[0];
-    /* the activation tile is staged in LDS in every grouped kernel: K * ntok is bounded */
-    if ((size_t)K * (size_t)ntok > 49152) return CKQ_ESHAPE;
     for (int i = 0; i < n; ++i)
         if (!y[i] || !W[i] || !X[i]) return CKQ_EINVAL;
+    /* Every grouped kernel stages its token tile in LDS.  A tile that does not
+     * fit (the tile is the token count rounded up to 1, 2, 4 or 8 rows of
+     * activations) goes out as n separate launches, which stream it instead. */
+    if (n == 1 || !group_tile_fits_lds(fmt, K, ntok)) {
+        for (int i = 0; i < n; ++i) {
+            const int rc = ckq_launch_gemv(fmt, y[i], W[i], X[i], bias ? bias[i] : nullptr, rows[i], K, ntok, ldys[i], 0,
+                                           rows[i], nullptr, stream);
+            if (rc) return rc;
+        }
+        return 0;
+    }
     GemvArgs a = {};
     a.y = y[0]; a.W = (const uint8_t *)W[0]; a.X = (const uint8_t *)X[0]; a.bias = bias ? bias[0] : nullptr; a.sub = nullptr;
     a.nrows = nrows; a.ntok = ntok; a.row0 = 0; a.row1 = rows[0]; a.ldy = ldy;
@@ -841,10 +891,11 @@ __device__ __forceinline__ float4 dequant4(const uint8_t *row, u32 e)
 template <int FMT>
 __global__ void __launch_bounds__(256) dequant_rows_kernel(const uint8_t *__restrict__ table, const int32_t *__restrict__ ids,
                                                            int vocab, const float *__restrict__ pos, float *__restrict__ out,
-                                                           int n_valid, int n_row, long row_bytes, int tokens)
+                                                           int n_valid, int n_row, long row_bytes, int tokens, int col_blocks)
 {
-    const int t = blockIdx.y;
-    const u32 e = 4u * (blockIdx.x * 256u + threadIdx.x);
+    /* the output row rides in blockIdx.x with the column block (gridDim.y stops at 65 535 rows) */
+    const int t = (int)(blockIdx.x / (u32)col_blocks);
+    const u32 e = 4u * ((blockIdx.x % (u32)col_blocks) * 256u + threadIdx.x);
     if (e >= (u32)n_row) return;
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
     if (t < tokens) {
@@ -875,17 +926,19 @@ extern "C" int ckq_launch_dequant_rows(int fmt, const void *table, const int32_t
     if (tokens > n_out_rows) tokens = n_out_rows;
     if (n_valid > n_row) n_valid = n_row;
     const long rb = (long)ckq_row_bytes(fmt, n_row);
-    const dim3 grid((unsigned)((n_row / 4 + 255) / 256), (unsigned)n_out_rows), block(256);
+    const int col_blocks = (n_row / 4 + 255) / 256;
+    if ((long long)col_blocks * n_out_rows > 0x7fffffffll) return CKQ_ESHAPE;
+    const dim3 grid((unsigned)((long long)col_blocks * n_out_rows)), block(256);
     hipStream_t s = (hipStream_t)stream;
     switch (fmt) {
     case CKQ_FMT_Q4_K:
-        hipLaunchKernelGGL(dequant_rows_kernel<CKQ_FMT_Q4_K>, grid, block, 0, s, (const uint8_t *)table, ids, vocab, pos, out, n_valid, n_row, rb, tokens);
+        hipLaunchKernelGGL(dequant_rows_kernel<CKQ_FMT_Q4_K>, grid, block, 0, s, (const uint8_t *)table, ids, vocab, pos, out, n_valid, n_row, rb, tokens, col_blocks);
         break;
     case CKQ_FMT_Q6_K:
-        hipLaunchKernelGGL(dequant_rows_kernel<CKQ_FMT_Q6_K>, grid, block, 0, s, (const uint8_t *)table, ids, vocab, pos, out, n_valid, n_row, rb, tokens);
+        hipLaunchKernelGGL(dequant_rows_kernel<CKQ_FMT_Q6_K>, grid, block, 0, s, (const uint8_t *)table, ids, vocab, pos, out, n_valid, n_row, rb, tokens, col_blocks);
         break;
     default:
-        hipLaunchKernelGGL(dequant_rows_kernel<CKQ_FMT_Q8_0>, grid, block, 0, s, (const uint8_t *)table, ids, vocab, pos, out, n_valid, n_row, rb, tokens);
+        hipLaunchKernelGGL(dequant_rows_kernel<CKQ_FMT_Q8_0>, grid, block, 0, s, (const uint8_t *)table, ids, vocab, pos, out, n_valid, n_row, rb, tokens, col_blocks);
         break;
     }
     return (int)hipGetLastError();

@@ -39,7 +39,8 @@ int ckq_launch_gemv(int fmt, float *y, const void *W, const void *X, const float
                     int32_t *subdots, void *stream);
 
 /* n (at most 4) independent matmuls of one format, input width and token count
- * (at most eight tokens, K * tokens <= 49152), problem i with rows[i] weight
+ * (at most eight tokens; a token tile that does not fit in LDS is issued as
+ * separate launches), problem i with rows[i] weight
  * rows and output row stride ldys[i], in one launch of the streaming kernel;
  * the arrays are host arrays (of device pointers), bias may be NULL or hold
  * NULL entries. */
@@ -69,6 +70,11 @@ int ckq_launch_rmsnorm_q8_k_fused(const float *input, const float *gamma, void *
  * rows from `tokens` on are zero. */
 int ckq_launch_dequant_rows(int fmt, const void *table, const int32_t *ids, int vocab, const float *pos,
                             float *out, int n_valid, int n_row, int tokens, int n_out_rows, void *stream);
+
+/* Host arithmetic of launches chunked over gridDim.y (at most 65 535 token
+ * tiles per launch): chunk c of `per` tokens out of `total` covers
+ * [*first, *first + *count).  Exported for the index test. */
+void ckq_grid_chunk(long total, long per, long c, long *first, long *count);
 
 /* Plain device copy kernel (calibration of the memory counters / roofline). */
 int ckq_launch_copy(void *dst, const void *src, size_t bytes, void *stream);

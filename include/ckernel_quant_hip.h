@@ -166,8 +166,22 @@ void gemm_nt_q5_0_q8_0(const void *A_q8, const void *B, const float *bias, float
 #define CKQ_CK_DT_Q6_K 8
 #define CKQ_CK_DT_Q8_0 9
 #define CKQ_CK_DT_Q5_0 11
-void fused_mlp_swiglu_prefill_w1w2_quant(const float *x, const void *W1, const float *B1, int w1_dt,
-                                         const void *W2, const float *B2, int w2_dt, float *output,
+/* The dtype parameters have the reference's own enum type when its header
+ * (include/ckernel_dtype.h:27-50, guard CKERNEL_DTYPE_H) has been included
+ * before this one, so both declarations of the function agree in one
+ * translation unit; otherwise an enum of the same enumerator values (and so
+ * the same size and calling convention) stands in for it. */
+#ifdef CKERNEL_DTYPE_H
+typedef CKDataType ckq_ck_dtype;
+#else
+typedef enum {
+    CKQ_CK_DTYPE_FP32 = 0, CKQ_CK_DTYPE_BF16, CKQ_CK_DTYPE_FP16, CKQ_CK_DTYPE_INT8, CKQ_CK_DTYPE_INT4,
+    CKQ_CK_DTYPE_Q4_0, CKQ_CK_DTYPE_Q4_1, CKQ_CK_DTYPE_Q4_K, CKQ_CK_DTYPE_Q6_K, CKQ_CK_DTYPE_Q8_0,
+    CKQ_CK_DTYPE_Q8_K, CKQ_CK_DTYPE_Q5_0, CKQ_CK_DTYPE_Q5_1, CKQ_CK_DTYPE_Q5_K, CKQ_CK_DTYPE_COUNT
+} ckq_ck_dtype;
+#endif
+void fused_mlp_swiglu_prefill_w1w2_quant(const float *x, const void *W1, const float *B1, ckq_ck_dtype w1_dt,
+                                         const void *W2, const float *B2, ckq_ck_dtype w2_dt, float *output,
                                          int seq_len, int embed_dim, int aligned_embed_dim,
                                          int intermediate_dim, int aligned_intermediate_dim, void *scratch);
 size_t fused_mlp_swiglu_prefill_w1w2_quant_scratch_size(int aligned_embed_dim, int aligned_intermediate_dim);
@@ -246,7 +260,7 @@ int ckq_gemm_nt_f32act_dev(int fmt, const float *A, const void *B, const float *
  * per-token projection set of a decoder layer (Q/K/V/O, gate/up, down) is one
  * such list.  Entry i computes C[m*ldc + n] as ckq_gemm_nt_dev does, with the
  * same bits.  Up to four consecutive entries of one format, input width and
- * token count (at most eight tokens, K * tokens <= 49152; their row counts may
+ * token count (at most eight tokens; their row counts may
  * differ), none of which writes memory another reads or writes (Q/K/V,
  * gate/up of a decode step), are issued as ONE launch. */
 typedef struct {

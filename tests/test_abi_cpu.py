@@ -105,6 +105,50 @@ def test_manifest_hook_parses_without_touching_a_device(L, tmp_path):
     assert L.ckq_weights_resident(ctypes.byref(nbytes)) == 0 and nbytes.value == 0
 
 
+def test_header_compiles_next_to_the_reference_headers(tmp_path):
+    """One translation unit with the reference's own headers and this library's:
+    every shared prototype must be declaration-compatible (the fused MLP takes
+    the reference's CKDataType, include/ckernel_engine.h:666-680)."""
+    ref_inc = "/root/reference/include"
+    if not os.path.exists(os.path.join(ref_inc, "ckernel_engine.h")):
+        pytest.skip("reference checkout not present")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    src = tmp_path / "tu.c"
+    src.write_text('#include "ckernel_engine.h"\n#include "ckernel_quant.h"\n#include "ck_parity_api.h"\n'
+                   '#include "ckernel_quant_hip.h"\n'
+                   'void (*p)(const float *, const void *, const float *, CKDataType, const void *, const float *,\n'
+                   '          CKDataType, float *, int, int, int, int, int, void *) = fused_mlp_swiglu_prefill_w1w2_quant;\n'
+                   'int main(void) { return 0; }\n')
+    r = subprocess.run(["gcc", "-std=gnu11", "-Wall", "-Werror", "-I" + ref_inc, "-I" + os.path.join(root, "include"),
+                        "-c", str(src), "-o", str(tmp_path / "tu.o")], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    # and on its own, as C and as C++
+    alone = tmp_path / "alone.c"
+    alone.write_text('#include "ckernel_quant_hip.h"\nint main(void) { return (int)sizeof(ckq_ck_dtype) - 4; }\n')
+    for cc, std in (("gcc", "-std=gnu11"), ("g++", "-std=c++17")):
+        r = subprocess.run([cc, std, "-Wall", "-Werror", "-x", "c" if cc == "gcc" else "c++",
+                            "-I" + os.path.join(root, "include"), "-c", str(alone), "-o", str(tmp_path / "a.o")],
+                           capture_output=True, text=True)
+        assert r.returncode == 0, r.stderr
+
+
+def test_grid_chunk_index_arithmetic(L):
+    """Launches whose token tiles exceed gridDim.y's 65 535 are issued in chunks;
+    the chunks must tile [0, total) exactly, in order, without overlap."""
+    L.ckq_grid_chunk.restype = None
+    L.ckq_grid_chunk.argtypes = [ctypes.c_long] * 3 + [ctypes.POINTER(ctypes.c_long)] * 2
+    for total, per in ((1, 65535), (65535, 65535), (65536, 65535), (70000, 65535), (131072, 65535),
+                       (8 * 65535 + 3, 8 * 65535), (200000, 2 * 65535)):
+        covered, c = 0, 0
+        while c * per < total:
+            first, count = ctypes.c_long(), ctypes.c_long()
+            L.ckq_grid_chunk(total, per, c, ctypes.byref(first), ctypes.byref(count))
+            assert first.value == covered and 0 < count.value <= per
+            covered += count.value
+            c += 1
+        assert covered == total and c == -(-total // per)
+
+
 def test_no_device_fails_loudly():
     """Without a GPU a compute call must not succeed silently: the library
     reports the HIP error and aborts the process."""
