@@ -118,6 +118,9 @@ _SIGS = {
     "ckq_gemm_nt_f32act_dev": (_i, [_i, _vp, _vp, _vp, _vp, _i, _i, _i, _c.c_long, _vp]),
     "ckq_matmul_sequence_dev": (_i, [_vp, _i, _i, _vp]),
     "ckq_subblock_dots_dev": (_i, [_i, _vp, _vp, _vp, _i, _i, _vp]),
+    "ckq_subblock_dots_tokens_dev": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "ckq_subblock_dots_group_dev": (_i, [_i, _i, _vp, _vp, _vp, _vp, _i, _i, _vp]),
+    "ckq_gemm_block_sums_dev": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "ckq_copy_dev": (_i, [_vp, _vp, _c.c_size_t, _vp]),
     "ckq_read_dev": (_i, [_vp, _c.c_size_t, _vp, _vp]),
     "ckq_init": (_i, []),

@@ -51,6 +51,10 @@ __device__ __forceinline__ float h2f(u32 h)
 /* Sign-extend byte `idx` (0..3) of a dword. */
 __device__ __forceinline__ int sbyte(u32 v, int idx) { return (int)(v << (24 - 8 * idx)) >> 24; }
 
+/* Wave index as a scalar: lets the compiler keep row indices, row base
+ * addresses and loop control in SGPRs (uniform branches, scalar address math). */
+__device__ __forceinline__ int wave_in_block() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
+
 /* ---- DPP reductions -------------------------------------------------------
  * Fixed summation tree, so results do not depend on scheduling. */
 template <int CTRL, int ROW_MASK = 0xF>

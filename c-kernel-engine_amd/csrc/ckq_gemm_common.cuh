@@ -1,0 +1,135 @@
+/*
+ * ckq_gemm_common.cuh - what the four matrix-core GEMM kernels share: operand
+ * vector types, the launch arguments, the K-split bookkeeping and the entry
+ * points of each kernel's translation unit.
+ */
+#pragma once
+#include <mutex>
+#include "ckq_device.cuh"
+#include "ckq_launch.h"
+
+typedef int   ckq_v4i  __attribute__((ext_vector_type(4)));
+typedef int   ckq_v16i __attribute__((ext_vector_type(16)));
+typedef float ckq_v16f __attribute__((ext_vector_type(16)));
+typedef __bf16 ckq_v8bf __attribute__((ext_vector_type(8)));
+typedef unsigned short ckq_v2u16 __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) void ckq_lds_void;
+typedef const __attribute__((address_space(1))) void ckq_glb_void;
+
+struct GemmArgs {
+    const uint8_t *A;     /* Q8_K activations, M rows of nb blocks */
+    const uint8_t *B;     /* Q4_K weights, N rows of nb blocks */
+    const float   *bias;  /* N or null */
+    float         *C;     /* M x ldc */
+    int  M, N, nb;
+    long ldc;
+    int  ntt, nnt;        /* token tiles, weight-row tiles */
+    /* split K: blockIdx.y = s handles K-steps [s * k_per, min(k_steps, (s + 1) * k_per)) and
+     * writes its partial tile, without bias, to part + s * M * N (row pitch N) */
+    int    splits, k_per;
+    float *part;
+    /* dump builds only: the exact integer block sums behind every output,
+     * dump[((t * N + n) * nblk + b) * per + i] (per = 2: I1, I2 for Q4_K and
+     * Q5_K; per = 1 for Q6_K and, with nblk = K / 32, for Q8_0) */
+    int32_t *dump;
+};
+
+/* Where a lane of a dump build stores the sums of output (token offset `tok`
+ * from the lane's first token, its row): nothing for rows or tokens outside
+ * the matrix. */
+/* A uniform value the compiler must take as new each time: keeps the 64 store
+ * addresses of a dump from being hoisted out of the K loop into registers. */
+__device__ __forceinline__ size_t gemm_opaque(size_t v)
+{
+    asm volatile("" : "+s"(v));
+    return v;
+}
+
+struct GemmDumpLane {
+    int32_t *p;          /* &dump[((t_first * N + n) * nblk + b) * per] */
+    size_t   tok_stride; /* N * nblk * per */
+    int      tok_left;   /* tokens from t_first to the end of the matrix */
+    bool     row_ok;
+    __device__ __forceinline__ void put(int tok, int i, int v) const
+    {
+        if (row_ok && tok < tok_left) p[(size_t)tok * tok_stride + i] = v;
+    }
+};
+
+/* What one block of a GEMM launch does: which tile id, which K-steps, where it
+ * writes and whether it adds the bias. */
+struct GemmOut { float *C; long ldc; const float *bias; };
+struct GemmWork { int id, k0, k1; GemmOut out; };
+__device__ __forceinline__ GemmWork gemm_work(const GemmArgs &a, int k_steps)
+{
+    const int id = blockIdx.x;
+    if (a.splits <= 1) return {id, 0, k_steps, {a.C, a.ldc, a.bias}};
+    const int k0 = (int)blockIdx.y * a.k_per;
+    return {id, k0, min(k_steps, k0 + a.k_per),
+            {a.part + (size_t)blockIdx.y * (size_t)a.M * (size_t)a.N, (long)a.N, nullptr}};
+}
+
+/* Split K when the tile grid leaves most of the chip idle: `tiles` blocks of
+ * `k_steps` loop iterations each.  Returns the number of splits (1 = none) so
+ * that tiles * splits approaches the CU count while every split keeps at
+ * least four iterations. */
+static int gemm_choose_splits(int tiles, int k_steps)
+{
+    if (tiles >= 160 || k_steps < 8) return 1;
+    int s = 256 / tiles;
+    if (s > k_steps / 4) s = k_steps / 4;
+    if (s > 16) s = 16;
+    return s < 2 ? 1 : s;
+}
+
+constexpr int GEMM_TILE_ROWS = 128;    /* weight rows per tile, all four kernels */
+
+/* Scratch for the partial tiles of K-split launches (kind 0) and for weights
+ * rewritten for another kernel (kind 1): one grow-only device buffer per
+ * stream and kind (work on one stream is ordered, so consecutive launches may
+ * share it).  Growing it allocates and therefore synchronises.  The caller
+ * holds gemm_split_mutex() from here until its last kernel is enqueued, so two
+ * host threads launching on one stream cannot interleave their kernel pairs.
+ * Defined in ckq_kernels.hip. */
+std::recursive_mutex &gemm_split_mutex();
+int gemm_workspace(int kind, hipStream_t s, size_t bytes, float **out);
+/* C = bias + partial 0 + partial 1 + ... in that order (ckq_kernels.hip). */
+int gemm_launch_reduce(float *C, long ldc, const float *part, const float *bias, int M, int N, int splits, hipStream_t s);
+
+/* Common launch tail: sets up the split, launches `kernel` on grid (x, splits)
+ * and, when split, the ordered reduction. */
+template <class Kernel>
+static int gemm_launch_split(Kernel kernel, GemmArgs &g, unsigned grid_x, int k_steps, hipStream_t s, unsigned threads = 256)
+{
+    g.splits = gemm_choose_splits(g.ntt * g.nnt, k_steps);
+    g.k_per = (k_steps + g.splits - 1) / g.splits;
+    g.splits = (k_steps + g.k_per - 1) / g.k_per;          /* no empty split */
+    g.part = nullptr;
+    if (g.splits <= 1) {
+        hipLaunchKernelGGL(kernel, dim3(grid_x, 1u), dim3(threads), 0, s, g);
+        return (int)hipGetLastError();
+    }
+    std::lock_guard<std::recursive_mutex> lock(gemm_split_mutex());
+    int rc = gemm_workspace(0, s, (size_t)g.splits * (size_t)g.M * (size_t)g.N * sizeof(float), &g.part);
+    if (rc) return rc;
+    hipLaunchKernelGGL(kernel, dim3(grid_x, (unsigned)g.splits), dim3(threads), 0, s, g);
+    rc = (int)hipGetLastError();
+    if (rc) return rc;
+    return gemm_launch_reduce(g.C, g.ldc, g.part, g.bias, g.M, g.N, g.splits, s);
+}
+
+
+/* packed u16x2 multiply-add, lane-wise (v_pk_mad_u16) */
+__device__ __forceinline__ u32 pk_mad_u16(u32 a, u32 b, u32 c)
+{
+    const ckq_v2u16 x = __builtin_bit_cast(ckq_v2u16, a), y = __builtin_bit_cast(ckq_v2u16, b),
+                    z = __builtin_bit_cast(ckq_v2u16, c);
+    return __builtin_bit_cast(u32, (ckq_v2u16)(x * y + z));
+}
+
+/* The four kernels, one translation unit each: C[m*ldc + n] = dot(B row n, A row m) (+ bias[n]).
+ * `sums` non-NULL runs the dump build of the kernel (GemmArgs::dump). */
+int launch_gemm_q4k_mfma(const void *A, const void *B, const float *bias, float *C, int M, int N, int K, long ldc, int32_t *sums, hipStream_t s);
+int launch_gemm_q5k_mfma(const void *A, const void *B, const float *bias, float *C, int M, int N, int K, long ldc, int32_t *sums, hipStream_t s);
+int launch_gemm_q6k_mfma(const void *A, const void *B, const float *bias, float *C, int M, int N, int K, long ldc, int32_t *sums, hipStream_t s);
+int launch_gemm_q80_mfma(const void *A, const void *B, const float *bias, float *C, int M, int N, int K, long ldc, int32_t *sums, hipStream_t s);

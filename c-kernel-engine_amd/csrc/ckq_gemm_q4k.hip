@@ -1,5 +1,5 @@
 /*
- * ckq_gemm_mfma.cuh - prefill GEMM, Q4_K weights x Q8_K activations, on the
+ * ckq_gemm_q4k.hip - prefill GEMM, Q4_K weights x Q8_K activations, on the
  * gfx950 int8 matrix cores.
  *
  *   C[t][n] = sum_b dx(t,b) * ( dw(n,b) * I1(t,n,b) - dmin(n,b) * I2(t,n,b) ) (+ bias[n])
@@ -37,125 +37,7 @@
  * 32w..32w+31.  Grid: token tiles fastest inside an XCD so the eight XCD L2s
  * each see a weight tile once.
  */
-#pragma once
-#include "ckq_device.cuh"
-
-typedef int   ckq_v4i  __attribute__((ext_vector_type(4)));
-typedef int   ckq_v16i __attribute__((ext_vector_type(16)));
-typedef float ckq_v16f __attribute__((ext_vector_type(16)));
-typedef __bf16 ckq_v8bf __attribute__((ext_vector_type(8)));
-typedef unsigned short ckq_v2u16 __attribute__((ext_vector_type(2)));
-typedef __attribute__((address_space(3))) void ckq_lds_void;
-typedef const __attribute__((address_space(1))) void ckq_glb_void;
-
-struct GemmArgs {
-    const uint8_t *A;     /* Q8_K activations, M rows of nb blocks */
-    const uint8_t *B;     /* Q4_K weights, N rows of nb blocks */
-    const float   *bias;  /* N or null */
-    float         *C;     /* M x ldc */
-    int  M, N, nb;
-    long ldc;
-    int  ntt, nnt;        /* token tiles, weight-row tiles */
-    /* split K: blockIdx.y = s handles K-steps [s * k_per, min(k_steps, (s + 1) * k_per)) and
-     * writes its partial tile, without bias, to part + s * M * N (row pitch N) */
-    int    splits, k_per;
-    float *part;
-};
-
-/* What one block of a GEMM launch does: which tile id, which K-steps, where it
- * writes and whether it adds the bias. */
-struct GemmOut { float *C; long ldc; const float *bias; };
-struct GemmWork { int id, k0, k1; GemmOut out; };
-__device__ __forceinline__ GemmWork gemm_work(const GemmArgs &a, int k_steps)
-{
-    const int id = blockIdx.x;
-    if (a.splits <= 1) return {id, 0, k_steps, {a.C, a.ldc, a.bias}};
-    const int k0 = (int)blockIdx.y * a.k_per;
-    return {id, k0, min(k_steps, k0 + a.k_per),
-            {a.part + (size_t)blockIdx.y * (size_t)a.M * (size_t)a.N, (long)a.N, nullptr}};
-}
-
-/* C = bias + partial 0 + partial 1 + ... in that order: the result does not
- * depend on which block finished first.  One thread per output. */
-__global__ void __launch_bounds__(256) gemm_splitk_reduce_kernel(float *__restrict__ C, long ldc, const float *__restrict__ part,
-                                                                 const float *__restrict__ bias, int M, int N, int splits)
-{
-    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x, mn = (size_t)M * (size_t)N;
-    if (i >= mn) return;
-    const int t = (int)(i / (size_t)N), n = (int)(i % (size_t)N);
-    float v = part[i];
-    for (int s = 1; s < splits; ++s) v += part[(size_t)s * mn + i];
-    C[(size_t)t * ldc + n] = bias ? v + bias[n] : v;
-}
-
-/* Split K when the tile grid leaves most of the chip idle: `tiles` blocks of
- * `k_steps` loop iterations each.  Returns the number of splits (1 = none) so
- * that tiles * splits approaches the CU count while every split keeps at
- * least four iterations. */
-static int gemm_choose_splits(int tiles, int k_steps)
-{
-    if (tiles >= 160 || k_steps < 8) return 1;
-    int s = 256 / tiles;
-    if (s > k_steps / 4) s = k_steps / 4;
-    if (s > 16) s = 16;
-    return s < 2 ? 1 : s;
-}
-
-/* Scratch for the partial tiles of K-split launches: one grow-only device
- * buffer per stream (work on one stream is ordered, so consecutive launches
- * may share it).  Growing it allocates and therefore synchronises.  The
- * caller holds g_split_mu from here until the reduction is enqueued, so two
- * host threads launching on one stream cannot interleave their kernel pairs. */
-#include <mutex>
-constexpr int GEMM_TILE_ROWS = 128;    /* weight rows per tile, all four kernels */
-static std::recursive_mutex g_split_mu;
-/* kind 0: partial tiles of a K split; kind 1: weights rewritten for another kernel */
-static int gemm_workspace(int kind, hipStream_t s, size_t bytes, float **out)
-{
-    struct Slot { hipStream_t s; int kind; void *p; size_t cap; bool used; };
-    static Slot slots[32];
-    Slot *sl = nullptr;
-    for (auto &c : slots) if (c.used && c.s == s && c.kind == kind) { sl = &c; break; }
-    if (!sl) for (auto &c : slots) if (!c.used) { sl = &c; c.used = true; c.s = s; c.kind = kind; c.p = nullptr; c.cap = 0; break; }
-    if (!sl) return (int)hipErrorOutOfMemory;
-    if (sl->cap < bytes) {
-        if (sl->p) {
-            hipError_t e = hipStreamSynchronize(s);
-            if (e != hipSuccess) return (int)e;
-            (void)hipFree(sl->p);
-            sl->p = nullptr; sl->cap = 0;
-        }
-        const size_t cap = bytes + bytes / 2;
-        hipError_t e = hipMalloc(&sl->p, cap);
-        if (e != hipSuccess) return (int)e;
-        sl->cap = cap;
-    }
-    *out = (float *)sl->p;
-    return 0;
-}
-
-/* Common launch tail: sets up the split, launches `kernel` on grid (x, splits)
- * and, when split, the ordered reduction. */
-template <class Kernel>
-static int gemm_launch_split(Kernel kernel, GemmArgs &g, unsigned grid_x, int k_steps, hipStream_t s, unsigned threads = 256)
-{
-    g.splits = gemm_choose_splits(g.ntt * g.nnt, k_steps);
-    g.k_per = (k_steps + g.splits - 1) / g.splits;
-    g.splits = (k_steps + g.k_per - 1) / g.k_per;          /* no empty split */
-    g.part = nullptr;
-    if (g.splits <= 1) {
-        hipLaunchKernelGGL(kernel, dim3(grid_x, 1u), dim3(threads), 0, s, g);
-        return (int)hipGetLastError();
-    }
-    std::lock_guard<std::recursive_mutex> lock(g_split_mu);
-    int rc = gemm_workspace(0, s, (size_t)g.splits * (size_t)g.M * (size_t)g.N * sizeof(float), &g.part);
-    if (rc) return rc;
-    hipLaunchKernelGGL(kernel, dim3(grid_x, (unsigned)g.splits), dim3(threads), 0, s, g);
-    const size_t mn = (size_t)g.M * (size_t)g.N;
-    hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, s,
-                       g.C, g.ldc, g.part, g.bias, g.M, g.N, g.splits);
-    return (int)hipGetLastError();
-}
+#include "ckq_gemm_common.cuh"
 
 #ifndef CKQ_GEMM_WPE
 #define CKQ_GEMM_WPE 2          /* waves per SIMD the register budget is sized for */
@@ -188,9 +70,9 @@ struct GemmStage {
  * of sub-blocks 0-3 are expanded during pass 1, those of 4-7 during pass 2,
  * and the fp32 combine of tokens 0-31 runs under pass 4.  Activation operands
  * are read from LDS two steps ahead.  Scheduling barriers pin that order. */
-template <class CopyFn>
+template <bool DUMP, class CopyFn>
 __device__ __forceinline__ void gemm_block_pipe(const GemmStage &st, u32 wofs, const u32 (&aofs)[8], int col, int half,
-                                                ckq_v16f (&acc)[2], CopyFn copy_one)
+                                                ckq_v16f (&acc)[2], CopyFn copy_one, const GemmDumpLane &dl)
 {
 #define CKQ_PIN() __builtin_amdgcn_sched_barrier(0)
     auto lds16 = [&](const uint8_t *p) { return *reinterpret_cast<const ckq_v4i *>(p); };
@@ -238,9 +120,15 @@ __device__ __forceinline__ void gemm_block_pipe(const GemmStage &st, u32 wofs, c
     auto combine = [&](int ts, int r) {
         const float4 d4 = dx[r >> 2];
         const float dxr = (r & 3) == 0 ? d4.x : (r & 3) == 1 ? d4.y : (r & 3) == 2 ? d4.z : d4.w;
-        const float f = (float)((aH[ts][r] << 3) + aL[ts][r]);
+        const int i1 = (aH[ts][r] << 3) + aL[ts][r];
+        const float f = (float)i1;
         const float u = dw * f - dmin * i2[r];
         acc[ts][r] += u * dxr;
+        if constexpr (DUMP) {
+            const int tok = 32 * ts + 8 * (r >> 2) + (r & 3);
+            dl.put(tok, 0, i1);
+            dl.put(tok, 1, (int)i2[r]);
+        }
     };
     auto load_dx = [&](int ts) {
 #pragma unroll
@@ -304,7 +192,7 @@ __device__ __forceinline__ void gemm_block_pipe(const GemmStage &st, u32 wofs, c
  * grid of T tiles takes ceil(T / 256) rounds of half-length tiles instead of
  * ceil(T / 512) rounds of full-length ones: 688 tiles need 3 x 0.5 instead of
  * 2 x 1. */
-template <int WPE, int KG>
+template <int WPE, int KG, bool DUMP = false>
 __global__ void __launch_bounds__(256 * KG, KG == 2 ? 1 : WPE) gemm_q4k_mfma_kernel(GemmArgs a)
 {
     constexpr int BM = GEMM_BM;
@@ -408,7 +296,15 @@ __global__ void __launch_bounds__(256 * KG, KG == 2 ? 1 : WPE) gemm_q4k_mfma_ker
         const int b = b0 + grp + KG * it, cur = it & 1;
         copy_begin(min(b + KG, last), cur ^ 1);
         __builtin_amdgcn_sched_barrier(0);
-        if (KG == 1 || b < b1) gemm_block_pipe(stage[cur], wofs_l, aofs, col, half, acc, copy_one);
+        GemmDumpLane dl = {};
+        if constexpr (DUMP) {
+            const int n = n0 + wave * 32 + col, tf = t0 + 4 * half;
+            dl.tok_stride = gemm_opaque((size_t)a.N * a.nb * 2);
+            dl.p = a.dump + ((size_t)tf * a.N + n) * a.nb * 2 + (size_t)b * 2;
+            dl.tok_left = a.M - tf;
+            dl.row_ok = n < a.N && b < b1;
+        }
+        if (KG == 1 || b < b1) gemm_block_pipe<DUMP>(stage[cur], wofs_l, aofs, col, half, acc, copy_one, dl);
         __builtin_amdgcn_sched_barrier(0);
         side_store(cur ^ 1);
         __builtin_amdgcn_s_waitcnt(0x0070);
@@ -447,10 +343,11 @@ __global__ void __launch_bounds__(256 * KG, KG == 2 ? 1 : WPE) gemm_q4k_mfma_ker
     }
 }
 
-static int launch_gemm_q4k_mfma(const void *A, const void *B, const float *bias, float *C,
-                                int M, int N, int K, long ldc, hipStream_t s)
+int launch_gemm_q4k_mfma(const void *A, const void *B, const float *bias, float *C,
+                         int M, int N, int K, long ldc, int32_t *sums, hipStream_t s)
 {
-    GemmArgs g;
+    GemmArgs g = {};
+    g.dump = sums;
     g.A = (const uint8_t *)A; g.B = (const uint8_t *)B; g.bias = bias; g.C = C;
     g.M = M; g.N = N; g.nb = K / 256; g.ldc = ldc;
     /* lane offsets inside a tile are 32-bit */
@@ -464,7 +361,11 @@ static int launch_gemm_q4k_mfma(const void *A, const void *B, const float *bias,
      * independent blocks per CU interleave better than two groups in lockstep
      * (11008x4096: 78 us against 88). */
     const int tiles = g.ntt * g.nnt, sp = gemm_choose_splits(tiles, g.nb);
-    if (tiles * sp <= 256 && (g.nb + sp - 1) / sp >= 8)
-        return gemm_launch_split(gemm_q4k_mfma_kernel<CKQ_GEMM_WPE, 2>, g, (unsigned)(g.ntt * nnt8), g.nb, s, 512);
+    const bool two_groups = tiles * sp <= 256 && (g.nb + sp - 1) / sp >= 8;
+    if (sums) {
+        if (two_groups) return gemm_launch_split(gemm_q4k_mfma_kernel<CKQ_GEMM_WPE, 2, true>, g, (unsigned)(g.ntt * nnt8), g.nb, s, 512);
+        return gemm_launch_split(gemm_q4k_mfma_kernel<CKQ_GEMM_WPE, 1, true>, g, (unsigned)(g.ntt * nnt8), g.nb, s, 256);
+    }
+    if (two_groups) return gemm_launch_split(gemm_q4k_mfma_kernel<CKQ_GEMM_WPE, 2>, g, (unsigned)(g.ntt * nnt8), g.nb, s, 512);
     return gemm_launch_split(gemm_q4k_mfma_kernel<CKQ_GEMM_WPE, 1>, g, (unsigned)(g.ntt * nnt8), g.nb, s, 256);
 }

@@ -1,5 +1,5 @@
 /*
- * ckq_gemm_q5k_mfma.cuh - prefill GEMM, Q5_K weights x Q8_K activations, on the
+ * ckq_gemm_q5k.hip - prefill GEMM, Q5_K weights x Q8_K activations, on the
  * gfx950 int8 matrix cores.
  *
  *   C[t][n] = sum_b (dw(n,b) * dx(t,b)) * (float) I1 - (dmin(n,b) * dx(t,b)) * (float) I2   (+ bias[n])
@@ -29,8 +29,7 @@
  *
  * Block = 4 waves = 64 tokens x 128 weight rows; wave w owns rows 32w..32w+31.
  */
-#pragma once
-#include "ckq_gemm_q6k_mfma.cuh"
+#include "ckq_gemm_common.cuh"
 
 constexpr int GEMM5_BM = 64, GEMM5_BN = 128, GEMM5_ROW = 176;
 
@@ -43,9 +42,9 @@ struct Gemm5Stage {
 
 /* One 256-block of a tile.  The planes of slab s+1 are expanded between the
  * MFMAs of slab s; copy_one(i) issues one global->LDS copy of a later block. */
-template <int NCOPY, class CopyFn>
+template <int NCOPY, bool DUMP, class CopyFn>
 __device__ __forceinline__ void gemm5_block(const Gemm5Stage &st, u32 wrow, const u32 (&aofs)[8], int col, int half,
-                                            ckq_v16f (&acc)[2], CopyFn copy_one)
+                                            ckq_v16f (&acc)[2], CopyFn copy_one, const GemmDumpLane &dl)
 {
 #define CKQ_PIN() __builtin_amdgcn_sched_barrier(0)
     auto lds16 = [&](const void *p) { return *reinterpret_cast<const ckq_v4i *>(p); };
@@ -164,13 +163,20 @@ __device__ __forceinline__ void gemm5_block(const Gemm5Stage &st, u32 wrow, cons
         for (int r = 0; r < 16; ++r) {
             const float4 d4 = dx[ts][r >> 2];
             const float dxr = (r & 3) == 0 ? d4.x : (r & 3) == 1 ? d4.y : (r & 3) == 2 ? d4.z : d4.w;
-            const float f1 = (float)((iH[ts][r] << 8) + iL[ts][r]);
-            const float f2 = (float)((mH[ts][r] << 8) + mL[ts][r]);
+            const int i1 = (iH[ts][r] << 8) + iL[ts][r], i2 = (mH[ts][r] << 8) + mL[ts][r];
+            const float f1 = (float)i1;
+            const float f2 = (float)i2;
             acc[ts][r] += (dw * dxr) * f1 - (dmin * dxr) * f2;
+            if constexpr (DUMP) {
+                const int tok = 32 * ts + 8 * (r >> 2) + (r & 3);
+                dl.put(tok, 0, i1);
+                dl.put(tok, 1, i2);
+            }
         }
 #undef CKQ_PIN
 }
 
+template <bool DUMP>
 __global__ void __launch_bounds__(256, 1) gemm_q5k_mfma_kernel(GemmArgs a)
 {
     constexpr int BM = GEMM5_BM, NST = 3;
@@ -264,7 +270,15 @@ __global__ void __launch_bounds__(256, 1) gemm_q5k_mfma_kernel(GemmArgs a)
     for (int b = b0; b < b1; ++b) {
         copy_begin(min(b + NST - 1, last), pf);
         __builtin_amdgcn_sched_barrier(0);
-        gemm5_block<NCOPY>(stage[cur], wrow, aofs, col, half, acc, copy_one);
+        GemmDumpLane dl = {};
+        if constexpr (DUMP) {
+            const int n = n0 + wave * 32 + col, tf = t0 + 4 * half;
+            dl.tok_stride = gemm_opaque((size_t)a.N * a.nb * 2);
+            dl.p = a.dump + ((size_t)tf * a.N + n) * a.nb * 2 + (size_t)b * 2;
+            dl.tok_left = a.M - tf;
+            dl.row_ok = n < a.N;
+        }
+        gemm5_block<NCOPY, DUMP>(stage[cur], wrow, aofs, col, half, acc, copy_one, dl);
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_waitcnt(0x0070 | (NCOPY & 15) | ((NCOPY >> 4) << 14));
         __builtin_amdgcn_s_barrier();
@@ -286,10 +300,11 @@ __global__ void __launch_bounds__(256, 1) gemm_q5k_mfma_kernel(GemmArgs a)
     }
 }
 
-static int launch_gemm_q5k_mfma(const void *A, const void *B, const float *bias, float *C,
-                                int M, int N, int K, long ldc, hipStream_t s)
+int launch_gemm_q5k_mfma(const void *A, const void *B, const float *bias, float *C,
+                         int M, int N, int K, long ldc, int32_t *sums, hipStream_t s)
 {
-    GemmArgs g;
+    GemmArgs g = {};
+    g.dump = sums;
     g.A = (const uint8_t *)A; g.B = (const uint8_t *)B; g.bias = bias; g.C = C;
     g.M = M; g.N = N; g.nb = K / 256; g.ldc = ldc;
     /* lane offsets inside a tile are 32-bit */
@@ -297,5 +312,6 @@ static int launch_gemm_q5k_mfma(const void *A, const void *B, const float *bias,
     g.ntt = (M + GEMM5_BM - 1) / GEMM5_BM;
     g.nnt = (N + GEMM5_BN - 1) / GEMM5_BN;
     const int nnt8 = (g.nnt + 7) / 8 * 8;
-    return gemm_launch_split(gemm_q5k_mfma_kernel, g, (unsigned)(g.ntt * nnt8), g.nb, s);
+    if (sums) return gemm_launch_split(gemm_q5k_mfma_kernel<true>, g, (unsigned)(g.ntt * nnt8), g.nb, s);
+    return gemm_launch_split(gemm_q5k_mfma_kernel<false>, g, (unsigned)(g.ntt * nnt8), g.nb, s);
 }

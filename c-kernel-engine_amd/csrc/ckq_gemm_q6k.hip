@@ -1,5 +1,5 @@
 /*
- * ckq_gemm_q6k_mfma.cuh - prefill GEMM, Q6_K weights x Q8_K activations, on the
+ * ckq_gemm_q6k.hip - prefill GEMM, Q6_K weights x Q8_K activations, on the
  * gfx950 int8 matrix cores.
  *
  *   C[t][n] = sum_b (dw(n,b) * dx(t,b)) * (float) I(t,n,b)   (+ bias[n])
@@ -30,8 +30,7 @@
  *   slab s and larger token tiles (TH = 4) amortise it where the grid is big
  *   enough to fill the chip with them.
  */
-#pragma once
-#include "ckq_gemm_mfma.cuh"
+#include "ckq_gemm_common.cuh"
 
 constexpr int GEMM6_BN  = 128;   /* weight rows per tile */
 constexpr int GEMM6_ROW = 224;   /* LDS bytes per staged weight block: 14 chunks */
@@ -42,12 +41,6 @@ template <int TH> struct Gemm6Stage {
     float   d[32 * TH];                /* block scale of each token */
 };
 
-__device__ __forceinline__ u32 pk_mad_u16(u32 a, u32 b, u32 c)
-{
-    const ckq_v2u16 x = __builtin_bit_cast(ckq_v2u16, a), y = __builtin_bit_cast(ckq_v2u16, b),
-                    z = __builtin_bit_cast(ckq_v2u16, c);
-    return __builtin_bit_cast(u32, (ckq_v2u16)(x * y + z));
-}
 
 /* What a lane reads from a stage before it can start on a block: its row's
  * raw Q6_K block (the 16-byte runs its k-half touches) and the activation
@@ -83,8 +76,8 @@ template <int TH> struct Gemm6Sums {
     float    dw;
 };
 
-template <int TH>
-__device__ __forceinline__ void gemm6_combine(const Gemm6Sums<TH> &p, ckq_v16f (&acc)[TH])
+template <int TH, bool DUMP>
+__device__ __forceinline__ void gemm6_combine(const Gemm6Sums<TH> &p, ckq_v16f (&acc)[TH], const GemmDumpLane &dl)
 {
 #pragma unroll
     for (int ts = 0; ts < TH; ++ts)
@@ -92,8 +85,9 @@ __device__ __forceinline__ void gemm6_combine(const Gemm6Sums<TH> &p, ckq_v16f (
         for (int r = 0; r < 16; ++r) {
             const float4 d4 = p.dx[ts][r >> 2];
             const float dxr = (r & 3) == 0 ? d4.x : (r & 3) == 1 ? d4.y : (r & 3) == 2 ? d4.z : d4.w;
-            const float f = (float)((p.iH[ts][r] << 8) + p.iL[ts][r]);
-            acc[ts][r] += (p.dw * dxr) * f;
+            const int i = (p.iH[ts][r] << 8) + p.iL[ts][r];
+            acc[ts][r] += (p.dw * dxr) * (float)i;
+            if constexpr (DUMP) dl.put(32 * ts + 8 * (r >> 2) + (r & 3), 0, i);
         }
 }
 
@@ -175,7 +169,7 @@ __device__ __forceinline__ void gemm6_slabs(const Gemm6Stage<TH> &st, const Gemm
 #undef CKQ_PIN
 }
 
-template <int TH>
+template <int TH, bool DUMP = false>
 __global__ void __launch_bounds__(256, 1) gemm_q6k_mfma_kernel(GemmArgs a)
 {
     constexpr int BM = 32 * TH;
@@ -275,6 +269,14 @@ __global__ void __launch_bounds__(256, 1) gemm_q6k_mfma_kernel(GemmArgs a)
         copy_begin(min(b + NST - 1, last), pf);
         __builtin_amdgcn_sched_barrier(0);
         Gemm6Sums<TH> sums;
+        GemmDumpLane dl = {};
+        if constexpr (DUMP) {
+            const int n = n0 + wave * 32 + col, tf = t0 + 4 * half;
+            dl.tok_stride = gemm_opaque((size_t)a.N * a.nb);
+            dl.p = a.dump + ((size_t)tf * a.N + n) * a.nb + (size_t)b;
+            dl.tok_left = a.M - tf;
+            dl.row_ok = n < a.N;
+        }
         gemm6_slabs<TH, NCOPY>(stage[cur], head, aofs, half, sums, copy_one);
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (NST == 3) __builtin_amdgcn_s_waitcnt(0x0070 | (NCOPY & 15) | ((NCOPY >> 4) << 14));
@@ -288,9 +290,9 @@ __global__ void __launch_bounds__(256, 1) gemm_q6k_mfma_kernel(GemmArgs a)
         if constexpr (TH == 2) {
             gemm6_head_read<TH>(stage[cur], wrow, aofs[0], half, head);
             __builtin_amdgcn_sched_barrier(0);
-            gemm6_combine<TH>(sums, acc);
+            gemm6_combine<TH, DUMP>(sums, acc, dl);
         } else {
-            gemm6_combine<TH>(sums, acc);
+            gemm6_combine<TH, DUMP>(sums, acc, dl);
             __builtin_amdgcn_sched_barrier(0);
             gemm6_head_read<TH>(stage[cur], wrow, aofs[0], half, head);
         }
@@ -311,10 +313,11 @@ __global__ void __launch_bounds__(256, 1) gemm_q6k_mfma_kernel(GemmArgs a)
     }
 }
 
-static int launch_gemm_q6k_mfma(const void *A, const void *B, const float *bias, float *C,
-                                int M, int N, int K, long ldc, hipStream_t s)
+int launch_gemm_q6k_mfma(const void *A, const void *B, const float *bias, float *C,
+                         int M, int N, int K, long ldc, int32_t *sums, hipStream_t s)
 {
-    GemmArgs g;
+    GemmArgs g = {};
+    g.dump = sums;
     g.A = (const uint8_t *)A; g.B = (const uint8_t *)B; g.bias = bias; g.C = C;
     g.M = M; g.N = N; g.nb = K / 256; g.ldc = ldc;
     /* lane offsets inside a tile are 32-bit */
@@ -325,8 +328,10 @@ static int launch_gemm_q6k_mfma(const void *A, const void *B, const float *bias,
     const int ntt4 = (M + 127) / 128;
     if (ntt4 * g.nnt > 128) {
         g.ntt = ntt4;
+        if (sums) return gemm_launch_split(gemm_q6k_mfma_kernel<4, true>, g, (unsigned)(g.ntt * nnt8), g.nb, s);
         return gemm_launch_split(gemm_q6k_mfma_kernel<4>, g, (unsigned)(g.ntt * nnt8), g.nb, s);
     }
     g.ntt = (M + 63) / 64;
+    if (sums) return gemm_launch_split(gemm_q6k_mfma_kernel<2, true>, g, (unsigned)(g.ntt * nnt8), g.nb, s);
     return gemm_launch_split(gemm_q6k_mfma_kernel<2>, g, (unsigned)(g.ntt * nnt8), g.nb, s);
 }

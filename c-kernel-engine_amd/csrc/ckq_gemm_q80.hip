@@ -1,5 +1,5 @@
 /*
- * ckq_gemm_q80_mfma.cuh - prefill GEMM, Q8_0 weights x Q8_0 activations, on the
+ * ckq_gemm_q80.hip - prefill GEMM, Q8_0 weights x Q8_0 activations, on the
  * gfx950 int8 matrix cores.
  *
  *   C[t][n] = sum_j (dw(n,j) * dx(t,j)) * (float) S(t,n,j)   (+ bias[n])
@@ -30,8 +30,7 @@
  *
  * Block = 4 waves = 64 tokens x 128 weight rows; wave w owns rows 32w..32w+31.
  */
-#pragma once
-#include "ckq_gemm_mfma.cuh"
+#include "ckq_gemm_common.cuh"
 
 constexpr int GEMM8_BM = 64, GEMM8_BN = 128, GEMM8_KB = 4;   /* tokens, rows, 32-blocks per iteration */
 
@@ -52,6 +51,7 @@ __device__ __forceinline__ float scale_product(int h, float x)
     return r;
 }
 
+template <bool DUMP>
 __global__ void __launch_bounds__(256, 2) gemm_q80_mfma_kernel(GemmArgs a)
 {
     constexpr int BM = GEMM8_BM, BN = GEMM8_BN, KB = GEMM8_KB, NST = 2;
@@ -201,6 +201,14 @@ __global__ void __launch_bounds__(256, 2) gemm_q80_mfma_kernel(GemmArgs a)
                 const float dx = h2f(dxh[j & 1][ts]);
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[ts][r] += scale_product(dwh[j & 1][r >> 2][r & 3], dx) * (float)d[k & 1][r];
+                if constexpr (DUMP) {
+                    const int t = t0 + col + 32 * ts;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int n = n0 + 32 * wave + 8 * (r >> 2) + 4 * half + (r & 3);
+                        if (t < a.M && n < a.N) a.dump[((size_t)t * a.N + n) * nblk + (size_t)(it * KB + j)] = d[k & 1][r];
+                    }
+                }
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -233,10 +241,11 @@ __global__ void __launch_bounds__(256, 2) gemm_q80_mfma_kernel(GemmArgs a)
     }
 }
 
-static int launch_gemm_q80_mfma(const void *A, const void *B, const float *bias, float *C,
-                                int M, int N, int K, long ldc, hipStream_t s)
+int launch_gemm_q80_mfma(const void *A, const void *B, const float *bias, float *C,
+                         int M, int N, int K, long ldc, int32_t *sums, hipStream_t s)
 {
-    GemmArgs g;
+    GemmArgs g = {};
+    g.dump = sums;
     g.A = (const uint8_t *)A; g.B = (const uint8_t *)B; g.bias = bias; g.C = C;
     g.M = M; g.N = N; g.nb = K / 32; g.ldc = ldc;
     /* lane offsets inside a tile are 32-bit */
@@ -244,5 +253,6 @@ static int launch_gemm_q80_mfma(const void *A, const void *B, const float *bias,
     g.ntt = (M + GEMM8_BM - 1) / GEMM8_BM;
     g.nnt = (N + GEMM8_BN - 1) / GEMM8_BN;
     const int nnt8 = (g.nnt + 7) / 8 * 8;
-    return gemm_launch_split(gemm_q80_mfma_kernel, g, (unsigned)(g.ntt * nnt8), (g.nb + GEMM8_KB - 1) / GEMM8_KB, s);
+    if (sums) return gemm_launch_split(gemm_q80_mfma_kernel<true>, g, (unsigned)(g.ntt * nnt8), (g.nb + GEMM8_KB - 1) / GEMM8_KB, s);
+    return gemm_launch_split(gemm_q80_mfma_kernel<false>, g, (unsigned)(g.ntt * nnt8), (g.nb + GEMM8_KB - 1) / GEMM8_KB, s);
 }

@@ -1191,7 +1191,7 @@ int ckq_matmul_sequence_dev(const ckq_matmul_op *ops, int nops, int repeat, void
                     y[j] = ops[i + j].C; W[j] = ops[i + j].B; X[j] = ops[i + j].A_q8; b[j] = ops[i + j].bias;
                     rows[j] = ops[i + j].N; ld[j] = ops[i + j].ldc;
                 }
-                rc = ckq_launch_gemv_group(o->fmt, n, y, W, X, b, rows, ld, o->K, o->M, stream);
+                rc = ckq_launch_gemv_group(o->fmt, n, y, W, X, b, rows, ld, o->K, o->M, NULL, stream);
             } else {
                 rc = ckq_gemm_nt_dev(o->fmt, o->A_q8, o->B, o->bias, o->C, o->M, o->N, o->K, o->ldc, stream);
             }
@@ -1207,6 +1207,29 @@ int ckq_subblock_dots_dev(int fmt, int32_t *out, const void *W, const void *x_q8
     if (fmt != CKQ_FMT_Q4_K && fmt != CKQ_FMT_Q5_K && fmt != CKQ_FMT_Q6_K && fmt != CKQ_FMT_Q8_0 && fmt != CKQ_FMT_Q5_0)
         return CKQ_EFORMAT;
     return ckq_launch_gemv(fmt, NULL, W, x_q8, NULL, M, K, 1, M, 0, M, out, stream);
+}
+
+int ckq_subblock_dots_tokens_dev(int fmt, int32_t *out, const void *W, const void *X_q8, int M, int K, int ntok, void *stream)
+{
+    if (!out) return CKQ_EINVAL;
+    if (fmt != CKQ_FMT_Q4_K && fmt != CKQ_FMT_Q5_K && fmt != CKQ_FMT_Q6_K && fmt != CKQ_FMT_Q8_0 && fmt != CKQ_FMT_Q5_0)
+        return CKQ_EFORMAT;
+    return ckq_launch_gemv(fmt, NULL, W, X_q8, NULL, M, K, ntok, M, 0, M, out, stream);
+}
+
+int ckq_subblock_dots_group_dev(int fmt, int n, int32_t *out, const void *const *W, const void *const *X_q8, const int *rows,
+                                int K, int ntok, void *stream)
+{
+    if (!out) return CKQ_EINVAL;
+    if (fmt != CKQ_FMT_Q4_K && fmt != CKQ_FMT_Q5_K && fmt != CKQ_FMT_Q6_K && fmt != CKQ_FMT_Q8_0 && fmt != CKQ_FMT_Q5_0)
+        return CKQ_EFORMAT;
+    return ckq_launch_gemv_group(fmt, n, NULL, W, X_q8, NULL, rows, NULL, K, ntok, out, stream);
+}
+
+int ckq_gemm_block_sums_dev(int fmt, const void *A_q8, const void *B, const float *bias, float *C, int32_t *sums,
+                            int M, int N, int K, void *stream)
+{
+    return ckq_launch_gemm_block_sums(fmt, A_q8, B, bias, C, sums, M, N, K, N, stream);
 }
 
 int ckq_copy_dev(void *dst, const void *src, size_t bytes, void *stream)

@@ -22,8 +22,6 @@
 #include "ckq_formats.cuh"
 #include "ckq_launch.h"
 
-__device__ __forceinline__ int wave_in_block();
-
 /* ========================================================================= */
 /* GEMV                                                                       */
 /* ========================================================================= */
@@ -73,236 +71,63 @@ static bool gemm_on_matrix_cores(int ntok, size_t weight_bytes, size_t budget_mb
     return passes * per > (budget_mb << 20);
 }
 
-constexpr int CKQ_GROUP_MAX = 4;   /* independent matmuls of one shape in one launch */
+#include "ckq_gemv.cuh"
+#include "ckq_gemm_common.cuh"
 
-struct GemvArgs {
-    float         *y;
-    const uint8_t *W;
-    const uint8_t *X;
-    const float   *bias;
-    int32_t       *sub;
-    int  nrows, npos, ntok, row0, row1, nsub_row;
-    long wrow, xrow, ldy;
-};
-
-/* Problems 1..3 of a grouped launch (blockIdx.z = g > 0); problem 0 is in GemvArgs. */
-struct GemvGroup {
-    float         *y[CKQ_GROUP_MAX - 1];
-    const uint8_t *W[CKQ_GROUP_MAX - 1];
-    const uint8_t *X[CKQ_GROUP_MAX - 1];
-    const float   *bias[CKQ_GROUP_MAX - 1];
-    int nrows[CKQ_GROUP_MAX - 1];           /* rows of each further problem (the grid covers the largest) */
-    int ldy[CKQ_GROUP_MAX - 1];             /* and its output row stride */
-    int n;                                  /* problems in the launch, 1 = not grouped */
-};
-
-/* Wave index as a scalar: lets the compiler keep row indices, row base
- * addresses and loop control in SGPRs (uniform branches, scalar address math). */
-__device__ __forceinline__ int wave_in_block() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
-
-#include "ckq_gemm_mfma.cuh"
-#include "ckq_gemm_q6k_mfma.cuh"
-#include "ckq_gemm_q80_mfma.cuh"
-#include "ckq_gemm_q5k_mfma.cuh"
-
-/*
- * Tiled kernel (token tiles MT >= 1, and the sub-block-dot dump).  One wave
- * handles (64/LPR)*RPI weight rows: LPR lanes share a row, lane l of the group
- * owns positions l, l+LPR, ... (PPL of them per pass).  All weight and
- * activation loads of a pass are issued before anything is decoded.  There is
- * no loop over rows: the grid supplies the parallelism.  The fp32 partials are
- * summed over the LPR lanes with a fixed DPP tree; the last lane of the group
- * stores.
- */
-template <class F, int LPR, int PPL, int MT, int RPI, bool DUMP, int WPB, bool LDSX, bool GRP = false>
-__global__ void __launch_bounds__(64 * WPB) __attribute__((amdgpu_waves_per_eu(MT == 1 && !DUMP && PPL == 1 && RPI == 1 ? F::OCC1 : MT == 1 && !DUMP && PPL == 1 && RPI == 2 && LPR == 64 ? F::OCC2 : MT >= 4 && PPL == 1 ? 4 : 1)))
-gemv_kernel(const uint8_t *W, const uint8_t *X, long wrow, long xrow, int row0, int row1, int npos, int ntok,
-            float *y, const float *bias, long ldy, int32_t *sub, int nsub_row, int nrows, GemvGroup grp)
+/* C = bias + partial 0 + partial 1 + ... in that order: the result does not
+ * depend on which block finished first.  One thread per output. */
+__global__ void __launch_bounds__(256) gemm_splitk_reduce_kernel(float *__restrict__ C, long ldc, const float *__restrict__ part,
+                                                                 const float *__restrict__ bias, int M, int N, int splits)
 {
-    /* The arguments are scalars, those the first loads need in front: the
-     * first fourteen registers' worth arrive preloaded with the wave (build
-     * flag -amdgpu-kernarg-preload-count) instead of through a scalar load
-     * that every wave waits for before it can issue its first weight load. */
-    const int g = GRP ? (int)blockIdx.z : 0;
-    const int row1g = GRP && g ? grp.nrows[g - 1] : row1;    /* problems of a group may differ in their row count */
-    const long ldyg = GRP && g ? (long)grp.ldy[g - 1] : ldy;
-    const GemvArgs a = {y, W, X, bias, sub, nrows, npos, ntok, row0, row1g, nsub_row, wrow, xrow, ldyg};
-    constexpr int SLOTS = 64 / LPR;
-    extern __shared__ __attribute__((aligned(16))) uint8_t xs[];   /* LDSX: the MT activation rows */
-    /* grouped launch: blockIdx.z picks the problem (a separate instantiation: the extra
-     * argument loads lengthen the start of every wave, which a bandwidth-bound launch
-     * of a few microseconds feels) */
-    float *const         gy    = g == 0 ? a.y    : grp.y[g - 1];
-    const uint8_t *const gW    = g == 0 ? a.W    : grp.W[g - 1];
-    const uint8_t *const gX    = g == 0 ? a.X    : grp.X[g - 1];
-    const float *const   gbias = g == 0 ? a.bias : grp.bias[g - 1];
-    const int lane = threadIdx.x & 63, wave = wave_in_block();
-    const int slot = lane / LPR, l = lane % LPR;
-    const int wave_row = a.row0 + (blockIdx.x * WPB + wave) * (SLOTS * RPI);   /* uniform */
-    const bool live = wave_row < a.row1;
-    if (!LDSX && !live) return;
-    const int wrow_c = min(wave_row, a.row1 - 1);
-    const int rbase = wave_row + slot * RPI;
-    const int t0 = blockIdx.y * MT;
-    const uint8_t *wbase = gW + (size_t)wrow_c * a.wrow;                      /* uniform */
-
-    /* Every wave of the block reads the same activation rows: they are staged
-     * once in LDS instead of once per wave through the vector cache.  Their
-     * loads go out first, all at once (one round trip, they hit in L2), the
-     * weight loads follow, and only then are the staged values written. */
-    constexpr int XNT = 64 * WPB, XU = MT == 1 ? 2 : 4;
-    const uint8_t *xsrc = gX + (size_t)t0 * a.xrow;
-    const int xbytes = (int)((long)min(MT, a.ntok - t0) * a.xrow), xn = xbytes / F::XS_SRC;   /* staging units */
-    const u32 xcap = (u32)((long)MT * a.xrow / F::XS_SRC);                                     /* units of a full tile */
-    u32 xv[XU][F::XS_REGS];
-    if (LDSX) {
-#pragma unroll
-        for (int u = 0; u < XU; ++u) {
-            const int i = u * XNT + (int)threadIdx.x;
-            if (i < xn) F::xs_ld(xv[u], xsrc + (u32)F::XS_SRC * (u32)i);
-        }
-    }
-
-    float acc[RPI][MT];
-#pragma unroll
-    for (int r = 0; r < RPI; ++r)
-#pragma unroll
-        for (int t = 0; t < MT; ++t) acc[r][t] = 0.0f;
-
-    u32 rowoff[RPI];   /* byte offset of the lane's r-th row from wbase, clamped to the last row */
-#pragma unroll
-    for (int r = 0; r < RPI; ++r) rowoff[r] = (u32)(min(rbase + r, a.row1 - 1) - wrow_c) * (u32)a.wrow;
-
-    for (int p0 = 0; p0 < a.npos; p0 += LPR * PPL) {
-        typename F::Wt  w[RPI][PPL];
-        typename F::Act act[MT >= 4 ? 1 : MT][PPL];   /* wide tiles stream their activations instead */
-#pragma unroll
-        for (int p = 0; p < PPL; ++p) {
-            const int pos = min(p0 + p * LPR + l, a.npos - 1);
-            const typename F::Off o = F::w_off(pos);
-#pragma unroll
-            for (int r = 0; r < RPI; ++r) {
-                typename F::Off orow = o;
-                F::off_shift(orow, rowoff[r]);
-                F::load_w(w[r][p], wbase, orow);
-            }
-        }
-        if (LDSX && p0 == 0) {
-            /* the staged activations' loads are older than the weight loads
-             * just issued, so waiting for them does not wait for the weights */
-#pragma unroll
-            for (int u = 0; u < XU; ++u) {
-                const int i = u * XNT + (int)threadIdx.x;
-                if (i < xn) F::xs_st(xs, xv[u], (u32)i, xcap);
-            }
-            for (int i = XNT * XU + (int)threadIdx.x; i < xn; i += XNT) {       /* long token tiles */
-                u32 v[F::XS_REGS];
-                F::xs_ld(v, xsrc + (u32)F::XS_SRC * (u32)i);
-                F::xs_st(xs, v, (u32)i, xcap);
-            }
-            if (F::XS_SRC == 16) {
-                const int tail = (xbytes & 15) >> 1;  /* plain-copy images: rows are a whole number of 2-byte units */
-                if ((int)threadIdx.x < tail) {
-                    const u32 o = 16u * (u32)xn + 2u * threadIdx.x;
-                    *reinterpret_cast<uint16_t *>(xs + o) = (uint16_t)ld2(xsrc + o);
-                }
-            }
-            __syncthreads();
-        }
-        if constexpr (MT >= 4) {
-            /* wide token tiles: the weights of a position are decoded once, then
-             * the tokens' activations stream through from LDS one at a time
-             * (holding all of them in registers would leave two waves per SIMD) */
-#pragma unroll
-            for (int p = 0; p < PPL; ++p) {
-                const int  upos  = p0 + p * LPR + l;
-                const bool valid = upos < a.npos;
-                const int  pos   = min(upos, a.npos - 1);
-                typename F::Dec dec[RPI];
-#pragma unroll
-                for (int r = 0; r < RPI; ++r) F::decode(dec[r], w[r][p], pos);
-#pragma unroll
-                for (int t = 0; t < MT; ++t) {
-                    typename F::Act at;
-                    if (LDSX) {
-                        const int tl = min(t, a.ntok - t0 - 1);                    /* uniform */
-                        F::load_act_lds(at, xs, tl, pos, (u32)a.xrow, a.npos, xcap);
-                    } else {
-                        const int tok = min(t0 + t, a.ntok - 1);                   /* uniform */
-                        F::load_act(at, gX + (size_t)tok * a.xrow, pos);
-                    }
-#pragma unroll
-                    for (int r = 0; r < RPI; ++r) {
-                        int sub[F::NSUB];
-                        const float v = F::dot(dec[r], at, sub);
-                        acc[r][t] += valid ? v : 0.0f;
-                    }
-                }
-            }
-        } else {
-#pragma unroll
-        for (int p = 0; p < PPL; ++p) {
-            const int pos = min(p0 + p * LPR + l, a.npos - 1);
-#pragma unroll
-            for (int t = 0; t < MT; ++t) {
-                if (LDSX) {
-                    const int tl = min(t, a.ntok - t0 - 1);                    /* uniform */
-                    F::load_act_lds(act[t][p], xs, tl, pos, (u32)a.xrow, a.npos, xcap);
-                } else {
-                    const int tok = min(t0 + t, a.ntok - 1);                   /* uniform */
-                    F::load_act(act[t][p], gX + (size_t)tok * a.xrow, pos);
-                }
-            }
-        }
-#pragma unroll
-        for (int p = 0; p < PPL; ++p) {
-            const int  upos  = p0 + p * LPR + l;
-            const bool valid = upos < a.npos;
-            const int  pos   = min(upos, a.npos - 1);
-#pragma unroll
-            for (int r = 0; r < RPI; ++r) {
-                typename F::Dec dec;
-                F::decode(dec, w[r][p], pos);
-#pragma unroll
-                for (int t = 0; t < MT; ++t) {
-                    int sub[F::NSUB];
-                    const float v = F::dot(dec, act[t][p], sub);
-                    acc[r][t] += valid ? v : 0.0f;
-                    if (DUMP && t == 0 && valid && rbase + r < a.row1) {
-#pragma unroll
-                        for (int i = 0; i < F::NSUB; ++i)
-                            a.sub[(size_t)(rbase + r) * a.nsub_row + F::sub_index(pos, i)] = sub[i];
-                    }
-                }
-            }
-        }
-        }
-    }
-
-#pragma unroll
-    for (int r = 0; r < RPI; ++r)
-#pragma unroll
-        for (int t = 0; t < MT; ++t) {
-            const float s = group_sum<LPR>(acc[r][t]);
-            const int row = rbase + r, tok = t0 + t;
-            if (!DUMP && l == LPR - 1 && row < a.row1 && tok < a.ntok)
-                gy[(size_t)tok * a.ldy + row] = gbias ? s + gbias[row] : s;
-        }
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x, mn = (size_t)M * (size_t)N;
+    if (i >= mn) return;
+    const int t = (int)(i / (size_t)N), n = (int)(i % (size_t)N);
+    float v = part[i];
+    for (int s = 1; s < splits; ++s) v += part[(size_t)s * mn + i];
+    C[(size_t)t * ldc + n] = bias ? v + bias[n] : v;
 }
 
-/* The group of the launch in flight on this thread (set by ckq_launch_gemv_group
- * around its dispatch; every other launch sees n = 1). */
-static thread_local GemvGroup t_group = {{}, {}, {}, {}, {}, {}, 1};
 
-/* Rows the grid has to cover: the computed range, or the largest problem of a group. */
-static int launch_rows(const GemvArgs &a) { return t_group.n > 1 ? a.nrows : a.row1 - a.row0; }
+static std::recursive_mutex g_split_mu;
+std::recursive_mutex &gemm_split_mutex() { return g_split_mu; }
 
-/* Token tiles a launch can carry in gridDim.y; longer token lists go out as
- * several launches over consecutive token ranges. */
-constexpr int CKQ_GRID_Y_MAX = 65535;
+/* Grow-only device scratch per (stream, kind); see ckq_gemm_common.cuh. */
+/* kind 0: partial tiles of a K split; kind 1: weights rewritten for another kernel */
+int gemm_workspace(int kind, hipStream_t s, size_t bytes, float **out)
+{
+    struct Slot { hipStream_t s; int kind; void *p; size_t cap; bool used; };
+    static Slot slots[32];
+    Slot *sl = nullptr;
+    for (auto &c : slots) if (c.used && c.s == s && c.kind == kind) { sl = &c; break; }
+    if (!sl) for (auto &c : slots) if (!c.used) { sl = &c; c.used = true; c.s = s; c.kind = kind; c.p = nullptr; c.cap = 0; break; }
+    if (!sl) return (int)hipErrorOutOfMemory;
+    if (sl->cap < bytes) {
+        if (sl->p) {
+            hipError_t e = hipStreamSynchronize(s);
+            if (e != hipSuccess) return (int)e;
+            (void)hipFree(sl->p);
+            sl->p = nullptr; sl->cap = 0;
+        }
+        const size_t cap = bytes + bytes / 2;
+        hipError_t e = hipMalloc(&sl->p, cap);
+        if (e != hipSuccess) return (int)e;
+        sl->cap = cap;
+    }
+    *out = (float *)sl->p;
+    return 0;
+}
 
-/* Token range [t, t + n) of a launch chunked over gridDim.y: chunk c of size
- * `per` tokens.  Host arithmetic only (also used by the index test). */
+
+int gemm_launch_reduce(float *C, long ldc, const float *part, const float *bias, int M, int N, int splits, hipStream_t s)
+{
+    const size_t mn = (size_t)M * (size_t)N;
+    hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, s,
+                       C, ldc, part, bias, M, N, splits);
+    return (int)hipGetLastError();
+}
+
+/* Token range [*first, *first + *count) of chunk c of a launch chunked over
+ * gridDim.y in pieces of `per` tokens.  Host arithmetic only. */
 extern "C" void ckq_grid_chunk(long total, long per, long c, long *first, long *count)
 {
     *first = c * per;
@@ -310,93 +135,6 @@ extern "C" void ckq_grid_chunk(long total, long per, long c, long *first, long *
     if (*count < 0) *count = 0;
 }
 
-template <class F, int LPR, int PPL, int MT, int RPI, bool DUMP, int WPB, bool LDSX>
-static int launch_one(const GemvArgs &a0, hipStream_t s)
-{
-    constexpr int rows_per_block = WPB * (64 / LPR) * RPI;
-    const int nr = launch_rows(a0);
-    const size_t lds = LDSX ? F::xs_lds_bytes((size_t)MT * (size_t)a0.xrow) : 0;
-    if (t_group.n > 1) {
-        if constexpr (!DUMP && LDSX) {                   /* grouped launches stage their activations in LDS */
-            dim3 grid((nr + rows_per_block - 1) / rows_per_block, (a0.ntok + MT - 1) / MT, (unsigned)t_group.n);
-            hipLaunchKernelGGL((gemv_kernel<F, LPR, PPL, MT, RPI, DUMP, WPB, LDSX, true>), grid, dim3(64 * WPB), lds, s,
-                               a0.W, a0.X, a0.wrow, a0.xrow, a0.row0, a0.row1, a0.npos, a0.ntok, a0.y, a0.bias, a0.ldy, a0.sub,
-                               a0.nsub_row, a0.nrows, t_group);
-            return (int)hipGetLastError();
-        }
-        return CKQ_EINVAL;
-    }
-    const long per = (long)MT * CKQ_GRID_Y_MAX;
-    for (long c = 0; c * per < a0.ntok; ++c) {
-        long first, count;
-        ckq_grid_chunk(a0.ntok, per, c, &first, &count);
-        GemvArgs a = a0;
-        a.X = a0.X + (size_t)first * (size_t)a0.xrow;
-        a.y = a0.y ? a0.y + (size_t)first * (size_t)a0.ldy : nullptr;
-        a.ntok = (int)count;
-        dim3 grid((nr + rows_per_block - 1) / rows_per_block, (a.ntok + MT - 1) / MT, 1);
-        hipLaunchKernelGGL((gemv_kernel<F, LPR, PPL, MT, RPI, DUMP, WPB, LDSX>), grid, dim3(64 * WPB), lds, s,
-                           a.W, a.X, a.wrow, a.xrow, a.row0, a.row1, a.npos, a.ntok, a.y, a.bias, a.ldy, a.sub,
-                           a.nsub_row, a.nrows, t_group);
-        const int rc = (int)hipGetLastError();
-        if (rc) return rc;
-    }
-    return 0;
-}
-
-/* Activation rows are staged in LDS when the token tile fits in 64 KB. */
-template <class F, int LPR, int PPL, int MT, int RPI, int WPB>
-static int launch_tile(const GemvArgs &a, hipStream_t s)
-{
-    if (F::xs_lds_bytes((size_t)MT * (size_t)a.xrow) <= 65536) return launch_one<F, LPR, PPL, MT, RPI, false, WPB, true>(a, s);
-    return launch_one<F, LPR, PPL, MT, RPI, false, WPB, false>(a, s);
-}
-
-/* Rows per wave-slot and waves per block for each token tile: one row per
- * slot in 256-thread blocks for the bandwidth-bound single-token case (as many
- * of the matrix's loads in flight as the CUs can hold, small barrier groups),
- * fewer rows in flight as the tile grows. */
-template <class F, int LPR, int PPL>
-static int launch_mt(const GemvArgs &a, bool dump, int max_mt, hipStream_t s)
-{
-    if (dump) {
-        if constexpr (F::TOKEN_TILES) return launch_one<F, LPR, PPL, 1, 1, true, 4, false>(a, s);
-        return CKQ_EINVAL;
-    }
-    if (a.ntok == 1 || max_mt == 1) {
-        /* 256-thread blocks; a second row per slot once the matrix needs more
-         * than two rounds of resident waves anyway (halves the activation
-         * staging per weight byte) */
-        const long waves = ((long)launch_rows(a) * LPR + 63) / 64;
-        if (PPL == 1 && waves > 16384) return launch_tile<F, LPR, PPL, 1, 2, 4>(a, s);
-        /* rows longer than one pass: each staged activation row is shared
-         * between eight weight rows, as 512-thread blocks (a whole number of
-         * blocks per CU on the usual projection shapes) or, for the largest
-         * matrices, two rows per slot */
-        if (PPL > 1 && launch_rows(a) >= 8192) return launch_tile<F, LPR, PPL, 1, 2, 4>(a, s);
-        if (PPL > 1 && launch_rows(a) >= 2048) return launch_tile<F, LPR, PPL, 1, 1, 8>(a, s);
-        return launch_tile<F, LPR, PPL, 1, 1, 4>(a, s);
-    }
-    if constexpr (F::TOKEN_TILES) {
-        if (a.ntok == 2) return launch_tile<F, LPR, PPL, 2, 2, 4>(a, s);
-        if (a.ntok <= 4) return launch_tile<F, LPR, PPL, 4, 2, 4>(a, s);
-        return launch_tile<F, LPR, PPL, 8, 2, 4>(a, s);   /* two rows per slot: the staged tile serves twice the weights */
-    }
-    return CKQ_EINVAL;   /* formats without token tiles are always launched with max_mt == 1 */
-}
-
-template <class F>
-static int launch_fmt(const GemvArgs &a, bool dump, int max_mt, hipStream_t s)
-{
-    const int np = a.npos;
-    if (np <= 8)  return launch_mt<F, 8, 1>(a, dump, max_mt, s);
-    if (np <= 16) return launch_mt<F, 16, 1>(a, dump, max_mt, s);
-    if (np <= 32) return launch_mt<F, 32, 1>(a, dump, max_mt, s);
-    if (np <= 64) return launch_mt<F, 64, 1>(a, dump, max_mt, s);
-    if (np <= 128) return launch_mt<F, 64, 2>(a, dump, max_mt, s);
-    if (np <= 192) return launch_mt<F, 64, 3>(a, dump, max_mt, s);
-    return launch_mt<F, 64, 4>(a, dump, max_mt, s);   /* longer rows loop in passes of 256 positions */
-}
 
 /* Q5_0 block -> Q8_0 block: the scale is kept, the 32 values become int8
  * q - 16.  One thread per block. */
@@ -431,18 +169,23 @@ static int launch_gemm_q50_via_q80(const void *A, const void *B, const float *bi
                        (const uint8_t *)B, (uint8_t *)tmp, nblocks);
     rc = (int)hipGetLastError();
     if (rc) return rc;
-    return launch_gemm_q80_mfma(A, tmp, bias, C, M, N, K, ldc, s);
+    return launch_gemm_q80_mfma(A, tmp, bias, C, M, N, K, ldc, nullptr, s);
 }
 
-static bool weights_dword_aligned(const GemvArgs &a)
+static bool weights_dword_aligned(const GemvArgs &a, const GemvGroup &grp)
 {
     uintptr_t bits = reinterpret_cast<uintptr_t>(a.W);
-    for (int i = 0; i + 1 < t_group.n; ++i) bits |= reinterpret_cast<uintptr_t>(t_group.W[i]);
+    for (int i = 0; i + 1 < grp.n; ++i) bits |= reinterpret_cast<uintptr_t>(grp.W[i]);
     return (bits & 3) == 0;
 }
 
-static int launch_gemv_args(int fmt, GemvArgs &a, int K, void *stream);
+static const GemvGroup k_no_group = {{}, {}, {}, {}, {}, {}, 1};
 
+static int launch_gemv_args(int fmt, GemvArgs &a, const GemvGroup &grp, int K, void *stream);
+
+/* `subdots`, when non-NULL, selects the dump build of the instantiation the
+ * same call would run without it: out[(t * nrows + row) * nsub + i], nothing
+ * is written to y. */
 extern "C" int ckq_launch_gemv(int fmt, float *y, const void *W, const void *X, const float *bias,
                                int nrows, int K, int ntok, long ldy, int row0, int row1,
                                int32_t *subdots, void *stream)
@@ -451,11 +194,11 @@ extern "C" int ckq_launch_gemv(int fmt, float *y, const void *W, const void *X, 
     if (row0 < 0) row0 = 0;
     if (row1 > nrows) row1 = nrows;
     if (row0 >= row1) return 0;
-    if (subdots && ntok != 1) return CKQ_EINVAL;
+    if (subdots && ntok > CKQ_STREAM_TOKENS) return CKQ_EINVAL;
     GemvArgs a = {};
     a.y = y; a.W = (const uint8_t *)W; a.X = (const uint8_t *)X; a.bias = bias; a.sub = subdots;
     a.nrows = nrows; a.ntok = ntok; a.row0 = row0; a.row1 = row1; a.ldy = ldy;
-    return launch_gemv_args(fmt, a, K, stream);
+    return launch_gemv_args(fmt, a, k_no_group, K, stream);
 }
 
 /* LDS bytes of the staged token tile of a grouped launch against the 64 KB a
@@ -477,30 +220,32 @@ static bool group_tile_fits_lds(int fmt, int K, int ntok)
 /* `n` (2..CKQ_GROUP_MAX) independent matmuls of one format and input width,
  * each with its own number of rows - the Q/K/V (grouped-query attention makes
  * K and V narrower than Q) or the gate/up projections of a token - as one
- * launch of the streaming
- * kernel: the launches' fixed start-up cost is paid once and the chip holds n
- * times the loads in flight.  Up to eight tokens; a token tile too large for
- * LDS is issued as separate launches. */
+ * launch of the streaming kernel: the launches' fixed start-up cost is paid
+ * once and the chip holds n times the loads in flight.  Up to eight tokens; a
+ * token tile too large for LDS is issued as separate launches.  `subdots`,
+ * when non-NULL, runs the dump build of the grouped instantiation instead:
+ * out[((g * ntok + t) * max_rows + row) * nsub + i]. */
 extern "C" int ckq_launch_gemv_group(int fmt, int n, float *const *y, const void *const *W, const void *const *X,
                                      const float *const *bias, const int *rows, const long *ldys, int K, int ntok,
-                                     void *stream)
+                                     int32_t *subdots, void *stream)
 {
-    if (n < 1 || n > CKQ_GROUP_MAX || !y || !W || !X || !rows || !ldys || K <= 0 || ntok < 1 || ntok > CKQ_STREAM_TOKENS)
+    if (n < 1 || n > CKQ_GROUP_MAX || !W || !X || !rows || K <= 0 || ntok < 1 || ntok > CKQ_STREAM_TOKENS)
         return CKQ_EINVAL;
+    if (!subdots && (!y || !ldys)) return CKQ_EINVAL;
     int nrows = 0;                                  /* the grid and the launch shape follow the largest problem */
     for (int i = 0; i < n; ++i) {
         if (rows[i] <= 0) return CKQ_EINVAL;
         if (rows[i] > nrows) nrows = rows[i];
     }
+    for (int i = 0; i < n && !subdots; ++i)
+        if (ldys[i] < rows[i] || ldys[i] > 0x7fffffff || !y[i]) return CKQ_EINVAL;
     for (int i = 0; i < n; ++i)
-        if (ldys[i] < rows[i] || ldys[i] > 0x7fffffff) return CKQ_EINVAL;
-    const long ldy = ldys[0];
-    for (int i = 0; i < n; ++i)
-        if (!y[i] || !W[i] || !X[i]) return CKQ_EINVAL;
+        if (!W[i] || !X[i]) return CKQ_EINVAL;
     /* Every grouped kernel stages its token tile in LDS.  A tile that does not
      * fit (the tile is the token count rounded up to 1, 2, 4 or 8 rows of
      * activations) goes out as n separate launches, which stream it instead. */
     if (n == 1 || !group_tile_fits_lds(fmt, K, ntok)) {
+        if (subdots) return CKQ_EINVAL;
         for (int i = 0; i < n; ++i) {
             const int rc = ckq_launch_gemv(fmt, y[i], W[i], X[i], bias ? bias[i] : nullptr, rows[i], K, ntok, ldys[i], 0,
                                            rows[i], nullptr, stream);
@@ -509,21 +254,21 @@ extern "C" int ckq_launch_gemv_group(int fmt, int n, float *const *y, const void
         return 0;
     }
     GemvArgs a = {};
-    a.y = y[0]; a.W = (const uint8_t *)W[0]; a.X = (const uint8_t *)X[0]; a.bias = bias ? bias[0] : nullptr; a.sub = nullptr;
-    a.nrows = nrows; a.ntok = ntok; a.row0 = 0; a.row1 = rows[0]; a.ldy = ldy;
+    GemvGroup grp = k_no_group;
+    a.y = subdots ? nullptr : y[0]; a.W = (const uint8_t *)W[0]; a.X = (const uint8_t *)X[0];
+    a.bias = bias && !subdots ? bias[0] : nullptr; a.sub = subdots;
+    a.nrows = nrows; a.ntok = ntok; a.row0 = 0; a.row1 = rows[0]; a.ldy = subdots ? nrows : ldys[0];
     for (int i = 1; i < n; ++i) {
-        t_group.y[i - 1] = y[i]; t_group.W[i - 1] = (const uint8_t *)W[i]; t_group.X[i - 1] = (const uint8_t *)X[i];
-        t_group.bias[i - 1] = bias ? bias[i] : nullptr;
-        t_group.nrows[i - 1] = rows[i];
-        t_group.ldy[i - 1] = (int)ldys[i];
+        grp.y[i - 1] = subdots ? nullptr : y[i]; grp.W[i - 1] = (const uint8_t *)W[i]; grp.X[i - 1] = (const uint8_t *)X[i];
+        grp.bias[i - 1] = bias && !subdots ? bias[i] : nullptr;
+        grp.nrows[i - 1] = rows[i];
+        grp.ldy[i - 1] = subdots ? nrows : (int)ldys[i];
     }
-    t_group.n = n;
-    const int rc = launch_gemv_args(fmt, a, K, stream);
-    t_group.n = 1;
-    return rc;
+    grp.n = n;
+    return launch_gemv_args(fmt, a, grp, K, stream);
 }
 
-static int launch_gemv_args(int fmt, GemvArgs &a, int K, void *stream)
+static int launch_gemv_args(int fmt, GemvArgs &a, const GemvGroup &grp, int K, void *stream)
 {
     float *const y = a.y;
     const void *const W = a.W, *const X = a.X;
@@ -532,63 +277,81 @@ static int launch_gemv_args(int fmt, GemvArgs &a, int K, void *stream)
     const long ldy = a.ldy;
     hipStream_t s = (hipStream_t)stream;
     const bool dump = a.sub != nullptr;
+    const bool whole = !dump && grp.n == 1 && row0 == 0 && row1 == nrows;   /* what a matrix-core GEMM can take */
     switch (fmt) {
     case CKQ_FMT_Q4_K:
         if (K % 256) return CKQ_ESHAPE;
-        if (!dump && row0 == 0 && row1 == nrows && gemm_on_matrix_cores(ntok, (size_t)nrows * (K / 256) * 144, 20))
-            return launch_gemm_q4k_mfma(X, W, bias, y, ntok, nrows, K, ldy, s);
+        if (whole && gemm_on_matrix_cores(ntok, (size_t)nrows * (K / 256) * 144, 20))
+            return launch_gemm_q4k_mfma(X, W, bias, y, ntok, nrows, K, ldy, nullptr, s);
         a.npos = K / 64; a.wrow = (long)(K / 256) * 144; a.xrow = (long)(K / 256) * 292; a.nsub_row = K / 32;
-        return launch_fmt<FmtQ4K>(a, dump, 8, s);
+        return ckq_gemv_launch_q4k(a, grp, s);
     case CKQ_FMT_Q5_K:
         if (K % 256) return CKQ_ESHAPE;
-        if (!dump && row0 == 0 && row1 == nrows && gemm_on_matrix_cores(ntok, (size_t)nrows * (K / 256) * 176, 40))
-            return launch_gemm_q5k_mfma(X, W, bias, y, ntok, nrows, K, ldy, s);
+        if (whole && gemm_on_matrix_cores(ntok, (size_t)nrows * (K / 256) * 176, 40))
+            return launch_gemm_q5k_mfma(X, W, bias, y, ntok, nrows, K, ldy, nullptr, s);
         a.npos = K / 64; a.wrow = (long)(K / 256) * 176; a.xrow = (long)(K / 256) * 292; a.nsub_row = K / 32;
-        return launch_fmt<FmtQ5K>(a, dump, 8, s);
+        return ckq_gemv_launch_q5k(a, grp, s);
     case CKQ_FMT_Q6_K:
         if (K % 256) return CKQ_ESHAPE;
-        if (!dump && row0 == 0 && row1 == nrows && gemm_on_matrix_cores(ntok, (size_t)nrows * (K / 256) * 210, 20))
-            return launch_gemm_q6k_mfma(X, W, bias, y, ntok, nrows, K, ldy, s);
+        if (whole && gemm_on_matrix_cores(ntok, (size_t)nrows * (K / 256) * 210, 20))
+            return launch_gemm_q6k_mfma(X, W, bias, y, ntok, nrows, K, ldy, nullptr, s);
         a.npos = K / 64; a.wrow = (long)(K / 256) * 210; a.xrow = (long)(K / 256) * 292; a.nsub_row = K / 16;
-        return launch_fmt<FmtQ6K>(a, dump, 8, s);
+        return ckq_gemv_launch_q6k(a, grp, s);
     case CKQ_FMT_Q8_0:
         if (K % 32) return CKQ_ESHAPE;
-        if (!dump && row0 == 0 && row1 == nrows &&
-            gemm_q80_on_matrix_cores(ntok, (size_t)nrows * (K / 32) * 34, K % 64 == 0 && weights_dword_aligned(a)))
-            return launch_gemm_q80_mfma(X, W, bias, y, ntok, nrows, K, ldy, s);
+        if (whole && gemm_q80_on_matrix_cores(ntok, (size_t)nrows * (K / 32) * 34, K % 64 == 0 && weights_dword_aligned(a, grp)))
+            return launch_gemm_q80_mfma(X, W, bias, y, ntok, nrows, K, ldy, nullptr, s);
         a.wrow = (long)(K / 32) * 34; a.xrow = (long)(K / 32) * 34; a.nsub_row = K / 32;
         /* rows of an even number of blocks at dword-aligned addresses: two blocks per position, aligned loads */
-        if (K % 64 == 0 && weights_dword_aligned(a)) {
+        if (K % 64 == 0 && weights_dword_aligned(a, grp)) {
             a.npos = K / 64;
-            return launch_fmt<FmtQ80P>(a, dump, 8, s);
+            return ckq_gemv_launch_q80p(a, grp, s);
         }
         a.npos = K / 32;
-        return launch_fmt<FmtQ80>(a, dump, 8, s);
+        return ckq_gemv_launch_q80(a, grp, s);
     case CKQ_FMT_Q5_0:
         if (K % 32) return CKQ_ESHAPE;
         /* prefill: the blocks are rewritten as Q8_0 blocks (same scale, values
          * q - 16: every dot product is unchanged) and go to the Q8_0 GEMM */
-        if (!dump && row0 == 0 && row1 == nrows && gemm_on_matrix_cores(ntok, (size_t)nrows * (K / 32) * 22, 20))
+        if (whole && gemm_on_matrix_cores(ntok, (size_t)nrows * (K / 32) * 22, 20))
             return launch_gemm_q50_via_q80(X, W, bias, y, ntok, nrows, K, ldy, s);
         a.npos = K / 32; a.wrow = (long)(K / 32) * 22; a.xrow = (long)(K / 32) * 34; a.nsub_row = K / 32;
-        return launch_fmt<FmtQ50>(a, dump, 8, s);
+        return ckq_gemv_launch_q50(a, grp, s);
     case CKQ_KERNEL_Q80_F32:
         if (K % 32) return CKQ_ESHAPE;
-        if (dump) return CKQ_EINVAL;
+        if (dump || grp.n > 1) return CKQ_EINVAL;
         a.npos = K / 32; a.wrow = (long)(K / 32) * 34; a.xrow = (long)K * 4; a.nsub_row = K / 32;
-        return launch_fmt<FmtQ80F32>(a, false, 1, s);
+        return ckq_gemv_launch_q80_f32(a, grp, s);
     case CKQ_KERNEL_Q4K_F32:
         if (K % 256) return CKQ_ESHAPE;
-        if (dump) return CKQ_EINVAL;
+        if (dump || grp.n > 1) return CKQ_EINVAL;
         a.npos = K / 64; a.wrow = (long)(K / 256) * 144; a.xrow = (long)K * 4; a.nsub_row = K / 64;
-        return launch_fmt<FmtQ4KF32>(a, false, 1, s);
+        return ckq_gemv_launch_q4k_f32(a, grp, s);
     case CKQ_KERNEL_Q6K_F32:
         if (K % 256) return CKQ_ESHAPE;
-        if (dump) return CKQ_EINVAL;
+        if (dump || grp.n > 1) return CKQ_EINVAL;
         a.npos = K / 64; a.wrow = (long)(K / 256) * 210; a.xrow = (long)K * 4; a.nsub_row = K / 64;
-        return launch_fmt<FmtQ6KF32>(a, false, 1, s);
+        return ckq_gemv_launch_q6k_f32(a, grp, s);
     default:
         return CKQ_EFORMAT;
+    }
+}
+
+/* The matrix-core GEMM of `fmt`, whatever the token count, with its integer
+ * block sums stored next to the result: sums[((t * N + n) * nblk + b) * per + i],
+ * nblk = K / 256 and per = 2 (I1, I2) for Q4_K and Q5_K, per = 1 (I) for Q6_K,
+ * nblk = K / 32 and per = 1 (the block dot) for Q8_0.  For the exactness tests. */
+extern "C" int ckq_launch_gemm_block_sums(int fmt, const void *A, const void *B, const float *bias, float *C, int32_t *sums,
+                                          int M, int N, int K, long ldc, void *stream)
+{
+    if (!A || !B || !C || !sums || M <= 0 || N <= 0 || K <= 0 || ldc < N) return CKQ_EINVAL;
+    hipStream_t s = (hipStream_t)stream;
+    switch (fmt) {
+    case CKQ_FMT_Q4_K: return K % 256 ? CKQ_ESHAPE : launch_gemm_q4k_mfma(A, B, bias, C, M, N, K, ldc, sums, s);
+    case CKQ_FMT_Q5_K: return K % 256 ? CKQ_ESHAPE : launch_gemm_q5k_mfma(A, B, bias, C, M, N, K, ldc, sums, s);
+    case CKQ_FMT_Q6_K: return K % 256 ? CKQ_ESHAPE : launch_gemm_q6k_mfma(A, B, bias, C, M, N, K, ldc, sums, s);
+    case CKQ_FMT_Q8_0: return K % 32 ? CKQ_ESHAPE : launch_gemm_q80_mfma(A, B, bias, C, M, N, K, ldc, sums, s);
+    default: return CKQ_EFORMAT;
     }
 }
 

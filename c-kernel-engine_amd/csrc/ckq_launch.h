@@ -31,8 +31,9 @@ extern "C" {
  * (Q8_K, or Q8_0 / fp32 for the Q8_0 weight kernels).
  * `row0`/`row1` restrict the computed rows to [row0,row1) (thread-split entry
  * points); outputs outside the range are not touched.
- * `subdots`, when non-NULL (ntok must be 1), receives the raw integer
- * sub-block dots: nrows x (K/blk x per-block count) int32.
+ * `subdots`, when non-NULL (at most eight tokens), runs the dump build of the
+ * instantiation the call would otherwise run and receives the raw integer
+ * sub-block dots, subdots[(t * nrows + row) * nsub + i]; y is not written.
  */
 int ckq_launch_gemv(int fmt, float *y, const void *W, const void *X, const float *bias,
                     int nrows, int K, int ntok, long ldy, int row0, int row1,
@@ -40,13 +41,21 @@ int ckq_launch_gemv(int fmt, float *y, const void *W, const void *X, const float
 
 /* n (at most 4) independent matmuls of one format, input width and token count
  * (at most eight tokens; a token tile that does not fit in LDS is issued as
- * separate launches), problem i with rows[i] weight
- * rows and output row stride ldys[i], in one launch of the streaming kernel;
- * the arrays are host arrays (of device pointers), bias may be NULL or hold
- * NULL entries. */
+ * separate launches), problem i with rows[i] weight rows and output row stride
+ * ldys[i], in one launch of the streaming kernel; the arrays are host arrays
+ * (of device pointers), bias may be NULL or hold NULL entries.  `subdots`
+ * non-NULL runs the dump build of the grouped kernel instead (y, ldys and bias
+ * are then ignored): subdots[((g * ntok + t) * max_rows + row) * nsub + i]. */
 int ckq_launch_gemv_group(int fmt, int n, float *const *y, const void *const *W, const void *const *X,
                           const float *const *bias, const int *rows, const long *ldys, int K, int ntok,
-                          void *stream);
+                          int32_t *subdots, void *stream);
+
+/* The matrix-core GEMM of `fmt` for any token count, its integer block sums
+ * stored next to the result: sums[((t * N + n) * nblk + b) * per + i]; nblk =
+ * K / 256 and per = 2 (I1, I2) for Q4_K and Q5_K, per = 1 for Q6_K; nblk =
+ * K / 32, per = 1 for Q8_0. */
+int ckq_launch_gemm_block_sums(int fmt, const void *A, const void *B, const float *bias, float *C, int32_t *sums,
+                               int M, int N, int K, long ldc, void *stream);
 
 /* Kernel choice for more than eight tokens: 0 = by token count and weight size
  * (default), 1 = always the matrix-core GEMM, 2 = always the streaming kernel. */

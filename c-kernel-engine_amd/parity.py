@@ -200,6 +200,42 @@ def dev_subblock_dots(fmt, W_t, x_t, M, K):
     return out.view(M, per)
 
 
+def dev_subblock_dots_tokens(fmt, W_t, X_t, M, K, ntok):
+    """Raw integer sub-block dots of every (token, row), from the instantiation of
+    the streaming kernel a matmul of this shape and token count runs: [ntok, M, K/sub]."""
+    import torch
+    per = (K // 16) if fmt == "q6_k" else (K // 32)
+    out = torch.zeros(ntok * M * per, dtype=torch.int32, device=W_t.device)
+    check(lib().ckq_subblock_dots_tokens_dev(FMT[fmt], _dp(out), _dp(W_t), _dp(X_t), M, K, ntok, _stream()),
+          "ckq_subblock_dots_tokens_dev")
+    return out.view(ntok, M, per)
+
+
+def dev_subblock_dots_group(fmt, W_ts, X_ts, rows, K, ntok):
+    """The same dump from ONE grouped launch over the problems (W_ts[g], X_ts[g],
+    rows[g]): [n, ntok, max(rows), K/sub]; rows beyond rows[g] stay zero."""
+    import torch
+    n, per, mx = len(W_ts), (K // 16) if fmt == "q6_k" else (K // 32), max(rows)
+    out = torch.zeros(n * ntok * mx * per, dtype=torch.int32, device=W_ts[0].device)
+    Wp = (_vp * n)(*[w.data_ptr() for w in W_ts])
+    Xp = (_vp * n)(*[x.data_ptr() for x in X_ts])
+    rp = (ctypes.c_int * n)(*rows)
+    check(lib().ckq_subblock_dots_group_dev(FMT[fmt], n, _dp(out), ctypes.cast(Wp, _vp), ctypes.cast(Xp, _vp),
+                                            ctypes.cast(rp, _vp), K, ntok, _stream()), "ckq_subblock_dots_group_dev")
+    return out.view(n, ntok, mx, per)
+
+
+def dev_gemm_block_sums(fmt, A_t, B_t, bias_t, M, N, K):
+    """The matrix-core GEMM with its integer block sums: (C [M,N], sums [M,N,nblk,per])."""
+    import torch
+    nblk, per = (K // 32, 1) if fmt == "q8_0" else (K // 256, 1 if fmt == "q6_k" else 2)
+    c = torch.empty(M * N, dtype=torch.float32, device=B_t.device)
+    sums = torch.zeros(M * N * nblk * per, dtype=torch.int32, device=B_t.device)
+    check(lib().ckq_gemm_block_sums_dev(FMT[fmt], _dp(A_t), _dp(B_t), _dp(bias_t), _dp(c), _dp(sums), M, N, K, _stream()),
+          "ckq_gemm_block_sums_dev")
+    return c.view(M, N), sums.view(M, N, nblk, per)
+
+
 def dev_matmul_sequence(ops, repeat=1):
     """ops: list of (fmt, A_t, B_t, bias_t, C_t, M, N, K); enqueued back-to-back
     `repeat` times by one C call (no Python between launches)."""

@@ -281,6 +281,27 @@ int ckq_matmul_sequence_dev(const ckq_matmul_op *ops, int nops, int repeat, void
  * or 16 (Q6_K, sum of (q-32)*q8).  For the bit-exactness tests. */
 int ckq_subblock_dots_dev(int fmt, int32_t *out, const void *W, const void *x_q8, int M, int K, void *stream);
 
+/* The same dump for up to eight tokens, taken from the instantiation of the
+ * streaming kernel that ckq_gemm_nt_dev would run for this shape and token
+ * count (token tile, rows per wave, block size, staged activations):
+ * out[(t * M + row) * (K/sub) + i]. */
+int ckq_subblock_dots_tokens_dev(int fmt, int32_t *out, const void *W, const void *X_q8, int M, int K, int ntok, void *stream);
+/* And from the grouped launch of n (2..4) matmuls of one format, input width
+ * and token count that ckq_matmul_sequence_dev issues for independent entries:
+ * out[((g * ntok + t) * max_rows + row) * (K/sub) + i], max_rows = the largest
+ * rows[g]; W, X_q8 and rows are host arrays of n entries.  Returns CKQ_EINVAL
+ * when such a group would be issued as separate launches. */
+int ckq_subblock_dots_group_dev(int fmt, int n, int32_t *out, const void *const *W, const void *const *X_q8, const int *rows,
+                                int K, int ntok, void *stream);
+/* The matrix-core GEMM of `fmt` (whatever the token count and the policy) with
+ * the exact integer sums behind every output stored next to the result C[M,N]:
+ * sums[((t * N + n) * nblk + b) * per + i]; Q4_K and Q5_K: nblk = K/256, per = 2
+ * (I1 = sum sc * sub-block dot, I2 = sum min * stored bsum pair); Q6_K: nblk =
+ * K/256, per = 1 (sum sc * 16-run dot of q - 32); Q8_0: nblk = K/32, per = 1
+ * (the block dot).  For the bit-exactness tests of the prefill path. */
+int ckq_gemm_block_sums_dev(int fmt, const void *A_q8, const void *B, const float *bias, float *C, int32_t *sums,
+                            int M, int N, int K, void *stream);
+
 /* Streaming device copy of `bytes` (multiple of 16): calibration kernel for
  * memory counters. */
 int ckq_copy_dev(void *dst, const void *src, size_t bytes, void *stream);
