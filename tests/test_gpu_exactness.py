@@ -164,7 +164,7 @@ def test_gemm_mfma_block_sums_extremes():
     W[:, 16:] = 0xff
     A = np.zeros((M * nb, 292), np.uint8)
     A[:, 0:4] = np.frombuffer(np.float32(0.05).tobytes(), np.uint8)
-    q = np.where((np.arange(M * nb)[:, None] + np.arange(256)[None, :] // 64) % 2 == 0, -128, 127).astype(np.int8)
+    q = np.where((np.arange(M * nb)[:, None] + 0 * np.arange(256)[None, :]) % 2 == 0, -128, 127).astype(np.int8)
     A[:, 4:260] = q.view(np.uint8)
     A[:, 260:292] = q.reshape(-1, 16, 16).sum(axis=2).astype(np.int16).view(np.uint8).reshape(-1, 32)
     W, A = W.reshape(-1), A.reshape(-1)
