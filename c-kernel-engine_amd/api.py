@@ -103,6 +103,7 @@ _SIGS = {
     "ckq_quantize_q8_k_dev": (_i, [_vp, _vp, _i, _i, _vp]),
     "ckq_quantize_q8_0_dev": (_i, [_vp, _vp, _i, _i, _vp]),
     "ckq_gemm_nt_dev": (_i, [_i, _vp, _vp, _vp, _vp, _i, _i, _i, _l, _vp]),
+    "ckq_gemm_nt_noalloc_dev": (_i, [_i, _vp, _vp, _vp, _vp, _i, _i, _i, _l, _vp]),
     "ckq_gemv_q4_k_q8_k_dev": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
     "ckq_gemv_q5_k_q8_k_dev": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
     "ckq_gemv_q6_k_q8_k_dev": (_i, [_vp, _vp, _vp, _i, _i, _vp]),

@@ -28,6 +28,8 @@ struct GemmArgs {
      * writes its partial tile, without bias, to part + s * M * N (row pitch N) */
     int    splits, k_per;
     float *part;
+    float *ext_part;       /* caller-provided scratch for `part` (launch options), or null */
+    size_t ext_part_bytes;
     /* dump builds only: the exact integer block sums behind every output,
      * dump[((t * N + n) * nblk + b) * per + i] (per = 2: I1, I2 for Q4_K and
      * Q5_K; per = 1 for Q6_K and, with nblk = K / 32, for Q8_0) */
@@ -54,6 +56,17 @@ struct GemmDumpLane {
     {
         if (row_ok && tok < tok_left) p[(size_t)tok * tok_stride + i] = v;
     }
+};
+
+/* Launch options of the four GEMMs: `sums` non-NULL runs the dump build
+ * (GemmArgs::dump); `scratch` non-NULL is caller-provided device memory of
+ * scratch_bytes for the partial tiles of a K-split launch, used instead of the
+ * library's grow-only workspace (nothing is allocated then; a split that needs
+ * more returns CKQ_ESCRATCH). */
+struct GemmOpts {
+    int32_t *sums;
+    float   *scratch;
+    size_t   scratch_bytes;
 };
 
 /* What one block of a GEMM launch does: which tile id, which K-steps, where it
@@ -109,8 +122,21 @@ static int gemm_launch_split(Kernel kernel, GemmArgs &g, unsigned grid_x, int k_
         hipLaunchKernelGGL(kernel, dim3(grid_x, 1u), dim3(threads), 0, s, g);
         return (int)hipGetLastError();
     }
+    const size_t need = (size_t)g.splits * (size_t)g.M * (size_t)g.N * sizeof(float);
+    if (g.ext_part) {
+        /* caller-provided scratch: nothing is allocated and nothing is locked
+         * (calls that share the scratch must not overlap).  Every partial
+         * entry the reduction reads is written by the split kernel first, so
+         * the scratch needs no clearing. */
+        if (need > g.ext_part_bytes) return CKQ_ESCRATCH;
+        g.part = g.ext_part;
+        hipLaunchKernelGGL(kernel, dim3(grid_x, (unsigned)g.splits), dim3(threads), 0, s, g);
+        const int rc = (int)hipGetLastError();
+        if (rc) return rc;
+        return gemm_launch_reduce(g.C, g.ldc, g.part, g.bias, g.M, g.N, g.splits, s);
+    }
     std::lock_guard<std::recursive_mutex> lock(gemm_split_mutex());
-    int rc = gemm_workspace(0, s, (size_t)g.splits * (size_t)g.M * (size_t)g.N * sizeof(float), &g.part);
+    int rc = gemm_workspace(0, s, need, &g.part);
     if (rc) return rc;
     hipLaunchKernelGGL(kernel, dim3(grid_x, (unsigned)g.splits), dim3(threads), 0, s, g);
     rc = (int)hipGetLastError();
@@ -128,8 +154,8 @@ __device__ __forceinline__ u32 pk_mad_u16(u32 a, u32 b, u32 c)
 }
 
 /* The four kernels, one translation unit each: C[m*ldc + n] = dot(B row n, A row m) (+ bias[n]).
- * `sums` non-NULL runs the dump build of the kernel (GemmArgs::dump). */
-int launch_gemm_q4k_mfma(const void *A, const void *B, const float *bias, float *C, int M, int N, int K, long ldc, int32_t *sums, hipStream_t s);
-int launch_gemm_q5k_mfma(const void *A, const void *B, const float *bias, float *C, int M, int N, int K, long ldc, int32_t *sums, hipStream_t s);
-int launch_gemm_q6k_mfma(const void *A, const void *B, const float *bias, float *C, int M, int N, int K, long ldc, int32_t *sums, hipStream_t s);
-int launch_gemm_q80_mfma(const void *A, const void *B, const float *bias, float *C, int M, int N, int K, long ldc, int32_t *sums, hipStream_t s);
+ * See GemmOpts for the options. */
+int launch_gemm_q4k_mfma(const void *A, const void *B, const float *bias, float *C, int M, int N, int K, long ldc, const GemmOpts &opts, hipStream_t s);
+int launch_gemm_q5k_mfma(const void *A, const void *B, const float *bias, float *C, int M, int N, int K, long ldc, const GemmOpts &opts, hipStream_t s);
+int launch_gemm_q6k_mfma(const void *A, const void *B, const float *bias, float *C, int M, int N, int K, long ldc, const GemmOpts &opts, hipStream_t s);
+int launch_gemm_q80_mfma(const void *A, const void *B, const float *bias, float *C, int M, int N, int K, long ldc, const GemmOpts &opts, hipStream_t s);

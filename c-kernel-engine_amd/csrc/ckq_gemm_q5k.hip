@@ -301,10 +301,13 @@ __global__ void __launch_bounds__(256, 1) gemm_q5k_mfma_kernel(GemmArgs a)
 }
 
 int launch_gemm_q5k_mfma(const void *A, const void *B, const float *bias, float *C,
-                         int M, int N, int K, long ldc, int32_t *sums, hipStream_t s)
+                         int M, int N, int K, long ldc, const GemmOpts &opts, hipStream_t s)
 {
     GemmArgs g = {};
+    int32_t *const sums = opts.sums;
     g.dump = sums;
+    g.ext_part = opts.scratch;
+    g.ext_part_bytes = opts.scratch_bytes;
     g.A = (const uint8_t *)A; g.B = (const uint8_t *)B; g.bias = bias; g.C = C;
     g.M = M; g.N = N; g.nb = K / 256; g.ldc = ldc;
     /* lane offsets inside a tile are 32-bit */

@@ -71,6 +71,7 @@ const char *ckq_error_string(int code)
     case CKQ_EINVAL: return "invalid argument (NULL pointer or non-positive dimension)";
     case CKQ_ESHAPE: return "K is not a multiple of the quantization block size";
     case CKQ_EFORMAT: return "unknown weight format";
+    case CKQ_ESCRATCH: return "the call needs more scratch than ckq_gemm_nt_noalloc_dev holds (4 MiB); use ckq_gemm_nt_dev or fewer tokens per call";
     default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
     }
 }
@@ -131,6 +132,11 @@ static int init_locked(void)
     const char *gp = getenv("CKQ_GEMM_POLICY");
     if (gp && strcmp(gp, "matrix") == 0) ckq_launch_set_gemm_policy(CKQ_GEMM_MATRIX);
     if (gp && strcmp(gp, "stream") == 0) ckq_launch_set_gemm_policy(CKQ_GEMM_STREAM);
+    /* address of the static scratch of the entry point that allocates nothing, for this device */
+    {
+        const int rc = ckq_launch_noalloc_setup();
+        if (rc) return fail(rc, "ckq_launch_noalloc_setup");
+    }
     g_inited = 1;
     return 0;
 }
@@ -1087,6 +1093,12 @@ int ckq_gemm_nt_dev(int fmt, const void *A_q8, const void *B, const float *bias,
     if (fmt != CKQ_FMT_Q4_K && fmt != CKQ_FMT_Q5_K && fmt != CKQ_FMT_Q6_K && fmt != CKQ_FMT_Q8_0 && fmt != CKQ_FMT_Q5_0)
         return CKQ_EFORMAT;
     return ckq_launch_gemv(fmt, C, B, A_q8, bias, N, K, M, ldc, 0, N, NULL, stream);
+}
+
+int ckq_gemm_nt_noalloc_dev(int fmt, const void *A_q8, const void *B, const float *bias, float *C,
+                            int M, int N, int K, long ldc, void *stream)
+{
+    return ckq_launch_gemv_noalloc(fmt, C, B, A_q8, bias, N, K, M, ldc, stream);
 }
 
 #define DEFINE_DEV(NAME, FMT)                                                                                   \

@@ -169,7 +169,7 @@ static int launch_gemm_q50_via_q80(const void *A, const void *B, const float *bi
                        (const uint8_t *)B, (uint8_t *)tmp, nblocks);
     rc = (int)hipGetLastError();
     if (rc) return rc;
-    return launch_gemm_q80_mfma(A, tmp, bias, C, M, N, K, ldc, nullptr, s);
+    return launch_gemm_q80_mfma(A, tmp, bias, C, M, N, K, ldc, GemmOpts{}, s);
 }
 
 static bool weights_dword_aligned(const GemvArgs &a, const GemvGroup &grp)
@@ -181,7 +181,7 @@ static bool weights_dword_aligned(const GemvArgs &a, const GemvGroup &grp)
 
 static const GemvGroup k_no_group = {{}, {}, {}, {}, {}, {}, 1};
 
-static int launch_gemv_args(int fmt, GemvArgs &a, const GemvGroup &grp, int K, void *stream);
+static int launch_gemv_args(int fmt, GemvArgs &a, const GemvGroup &grp, int K, void *stream, const GemmOpts &opts = GemmOpts{});
 
 /* `subdots`, when non-NULL, selects the dump build of the instantiation the
  * same call would run without it: out[(t * nrows + row) * nsub + i], nothing
@@ -268,7 +268,7 @@ extern "C" int ckq_launch_gemv_group(int fmt, int n, float *const *y, const void
     return launch_gemv_args(fmt, a, grp, K, stream);
 }
 
-static int launch_gemv_args(int fmt, GemvArgs &a, const GemvGroup &grp, int K, void *stream)
+static int launch_gemv_args(int fmt, GemvArgs &a, const GemvGroup &grp, int K, void *stream, const GemmOpts &opts)
 {
     float *const y = a.y;
     const void *const W = a.W, *const X = a.X;
@@ -282,25 +282,25 @@ static int launch_gemv_args(int fmt, GemvArgs &a, const GemvGroup &grp, int K, v
     case CKQ_FMT_Q4_K:
         if (K % 256) return CKQ_ESHAPE;
         if (whole && gemm_on_matrix_cores(ntok, (size_t)nrows * (K / 256) * 144, 20))
-            return launch_gemm_q4k_mfma(X, W, bias, y, ntok, nrows, K, ldy, nullptr, s);
+            return launch_gemm_q4k_mfma(X, W, bias, y, ntok, nrows, K, ldy, opts, s);
         a.npos = K / 64; a.wrow = (long)(K / 256) * 144; a.xrow = (long)(K / 256) * 292; a.nsub_row = K / 32;
         return ckq_gemv_launch_q4k(a, grp, s);
     case CKQ_FMT_Q5_K:
         if (K % 256) return CKQ_ESHAPE;
         if (whole && gemm_on_matrix_cores(ntok, (size_t)nrows * (K / 256) * 176, 40))
-            return launch_gemm_q5k_mfma(X, W, bias, y, ntok, nrows, K, ldy, nullptr, s);
+            return launch_gemm_q5k_mfma(X, W, bias, y, ntok, nrows, K, ldy, opts, s);
         a.npos = K / 64; a.wrow = (long)(K / 256) * 176; a.xrow = (long)(K / 256) * 292; a.nsub_row = K / 32;
         return ckq_gemv_launch_q5k(a, grp, s);
     case CKQ_FMT_Q6_K:
         if (K % 256) return CKQ_ESHAPE;
         if (whole && gemm_on_matrix_cores(ntok, (size_t)nrows * (K / 256) * 210, 20))
-            return launch_gemm_q6k_mfma(X, W, bias, y, ntok, nrows, K, ldy, nullptr, s);
+            return launch_gemm_q6k_mfma(X, W, bias, y, ntok, nrows, K, ldy, opts, s);
         a.npos = K / 64; a.wrow = (long)(K / 256) * 210; a.xrow = (long)(K / 256) * 292; a.nsub_row = K / 16;
         return ckq_gemv_launch_q6k(a, grp, s);
     case CKQ_FMT_Q8_0:
         if (K % 32) return CKQ_ESHAPE;
         if (whole && gemm_q80_on_matrix_cores(ntok, (size_t)nrows * (K / 32) * 34, K % 64 == 0 && weights_dword_aligned(a, grp)))
-            return launch_gemm_q80_mfma(X, W, bias, y, ntok, nrows, K, ldy, nullptr, s);
+            return launch_gemm_q80_mfma(X, W, bias, y, ntok, nrows, K, ldy, opts, s);
         a.wrow = (long)(K / 32) * 34; a.xrow = (long)(K / 32) * 34; a.nsub_row = K / 32;
         /* rows of an even number of blocks at dword-aligned addresses: two blocks per position, aligned loads */
         if (K % 64 == 0 && weights_dword_aligned(a, grp)) {
@@ -313,8 +313,10 @@ static int launch_gemv_args(int fmt, GemvArgs &a, const GemvGroup &grp, int K, v
         if (K % 32) return CKQ_ESHAPE;
         /* prefill: the blocks are rewritten as Q8_0 blocks (same scale, values
          * q - 16: every dot product is unchanged) and go to the Q8_0 GEMM */
-        if (whole && gemm_on_matrix_cores(ntok, (size_t)nrows * (K / 32) * 22, 20))
+        if (whole && gemm_on_matrix_cores(ntok, (size_t)nrows * (K / 32) * 22, 20)) {
+            if (opts.scratch) return CKQ_ESCRATCH;       /* the rewritten weights would need an allocation */
             return launch_gemm_q50_via_q80(X, W, bias, y, ntok, nrows, K, ldy, s);
+        }
         a.npos = K / 32; a.wrow = (long)(K / 32) * 22; a.xrow = (long)(K / 32) * 34; a.nsub_row = K / 32;
         return ckq_gemv_launch_q50(a, grp, s);
     case CKQ_KERNEL_Q80_F32:
@@ -337,6 +339,55 @@ static int launch_gemv_args(int fmt, GemvArgs &a, const GemvGroup &grp, int K, v
     }
 }
 
+/* ---- the entry point that allocates nothing ---------------------------------
+ * Scratch for the partial tiles of a K-split GEMM, held in the code object:
+ * every device the library runs on holds its own copy, at its own address,
+ * until the process ends.  Host code never uses the array's name as an
+ * address: the per-device address comes from hipGetSymbolAddress, once per
+ * device, with that device current.  The array keeps the last call's
+ * contents; nothing in it has to start at zero (the split kernel writes every
+ * partial entry the reduction reads).  Calls that overlap on one GPU race. */
+static __device__ __align__(256) unsigned char scratch[CKQ_NOALLOC_SCRATCH_BYTES];
+constexpr int CKQ_MAX_DEVICES = 64;
+static std::atomic<void *> g_scratch_ptr[CKQ_MAX_DEVICES];
+
+static int noalloc_scratch(void **out)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= CKQ_MAX_DEVICES) return (int)hipErrorInvalidDevice;
+    void *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!p) return (int)hipErrorInvalidSymbol;
+        g_scratch_ptr[dev].store(p, std::memory_order_release);
+    }
+    *out = p;
+    return 0;
+}
+
+extern "C" int ckq_launch_noalloc_setup(void)
+{
+    void *p;
+    return noalloc_scratch(&p);
+}
+
+extern "C" int ckq_launch_gemv_noalloc(int fmt, float *y, const void *W, const void *X, const float *bias,
+                                       int nrows, int K, int ntok, long ldy, void *stream)
+{
+    if (fmt != CKQ_FMT_Q4_K && fmt != CKQ_FMT_Q5_K && fmt != CKQ_FMT_Q6_K && fmt != CKQ_FMT_Q8_0) return CKQ_EFORMAT;
+    if (!y || !W || !X || nrows <= 0 || K <= 0 || ntok <= 0 || ldy < nrows) return CKQ_EINVAL;
+    void *p = nullptr;
+    const int rc = noalloc_scratch(&p);
+    if (rc) return rc;
+    GemvArgs a = {};
+    a.y = y; a.W = (const uint8_t *)W; a.X = (const uint8_t *)X; a.bias = bias; a.sub = nullptr;
+    a.nrows = nrows; a.ntok = ntok; a.row0 = 0; a.row1 = nrows; a.ldy = ldy;
+    return launch_gemv_args(fmt, a, k_no_group, K, stream, GemmOpts{nullptr, (float *)p, CKQ_NOALLOC_SCRATCH_BYTES});
+}
+
 /* The matrix-core GEMM of `fmt`, whatever the token count, with its integer
  * block sums stored next to the result: sums[((t * N + n) * nblk + b) * per + i],
  * nblk = K / 256 and per = 2 (I1, I2) for Q4_K and Q5_K, per = 1 (I) for Q6_K,
@@ -347,10 +398,10 @@ extern "C" int ckq_launch_gemm_block_sums(int fmt, const void *A, const void *B,
     if (!A || !B || !C || !sums || M <= 0 || N <= 0 || K <= 0 || ldc < N) return CKQ_EINVAL;
     hipStream_t s = (hipStream_t)stream;
     switch (fmt) {
-    case CKQ_FMT_Q4_K: return K % 256 ? CKQ_ESHAPE : launch_gemm_q4k_mfma(A, B, bias, C, M, N, K, ldc, sums, s);
-    case CKQ_FMT_Q5_K: return K % 256 ? CKQ_ESHAPE : launch_gemm_q5k_mfma(A, B, bias, C, M, N, K, ldc, sums, s);
-    case CKQ_FMT_Q6_K: return K % 256 ? CKQ_ESHAPE : launch_gemm_q6k_mfma(A, B, bias, C, M, N, K, ldc, sums, s);
-    case CKQ_FMT_Q8_0: return K % 32 ? CKQ_ESHAPE : launch_gemm_q80_mfma(A, B, bias, C, M, N, K, ldc, sums, s);
+    case CKQ_FMT_Q4_K: return K % 256 ? CKQ_ESHAPE : launch_gemm_q4k_mfma(A, B, bias, C, M, N, K, ldc, GemmOpts{sums, nullptr, 0}, s);
+    case CKQ_FMT_Q5_K: return K % 256 ? CKQ_ESHAPE : launch_gemm_q5k_mfma(A, B, bias, C, M, N, K, ldc, GemmOpts{sums, nullptr, 0}, s);
+    case CKQ_FMT_Q6_K: return K % 256 ? CKQ_ESHAPE : launch_gemm_q6k_mfma(A, B, bias, C, M, N, K, ldc, GemmOpts{sums, nullptr, 0}, s);
+    case CKQ_FMT_Q8_0: return K % 32 ? CKQ_ESHAPE : launch_gemm_q80_mfma(A, B, bias, C, M, N, K, ldc, GemmOpts{sums, nullptr, 0}, s);
     default: return CKQ_EFORMAT;
     }
 }

@@ -18,6 +18,7 @@ extern "C" {
 #define CKQ_EINVAL  (-1)  /* NULL pointer / non-positive dimension */
 #define CKQ_ESHAPE  (-2)  /* K not a multiple of the block size */
 #define CKQ_EFORMAT (-3)  /* unknown format tag */
+#define CKQ_ESCRATCH (-4) /* the call needs more scratch than the entry point that allocates nothing holds */
 
 /* Weight-format tags as in ckq_blocks.h, plus the fp32-activation variants
  * (X is then ntok rows of K floats). */
@@ -79,6 +80,17 @@ int ckq_launch_rmsnorm_q8_k_fused(const float *input, const float *gamma, void *
  * rows from `tokens` on are zero. */
 int ckq_launch_dequant_rows(int fmt, const void *table, const int32_t *ids, int vocab, const float *pos,
                             float *out, int n_valid, int n_row, int tokens, int n_out_rows, void *stream);
+
+/* ckq_launch_gemv for callers that must not allocate: a K-split matrix-core
+ * GEMM takes its partial tiles from a static device array of
+ * CKQ_NOALLOC_SCRATCH_BYTES instead of the grow-only workspace; a split that
+ * needs more returns CKQ_ESCRATCH.  Formats Q4_K, Q5_K, Q6_K, Q8_0.
+ * ckq_launch_noalloc_setup() resolves the array's address for the current
+ * device (once per device; also done by the first call on a device). */
+#define CKQ_NOALLOC_SCRATCH_BYTES ((size_t)4 << 20)
+int ckq_launch_noalloc_setup(void);
+int ckq_launch_gemv_noalloc(int fmt, float *y, const void *W, const void *X, const float *bias,
+                            int nrows, int K, int ntok, long ldy, void *stream);
 
 /* Host arithmetic of launches chunked over gridDim.y (at most 65 535 token
  * tiles per launch): chunk c of `per` tokens out of `total` covers

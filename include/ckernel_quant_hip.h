@@ -222,6 +222,23 @@ int ckq_quantize_q8_0_dev(const float *x, void *y, int num_rows, int k, void *st
 int ckq_gemm_nt_dev(int fmt, const void *A_q8, const void *B, const float *bias, float *C,
                     int M, int N, int K, long ldc, void *stream);
 
+/* ckq_gemm_nt_dev for callers that cannot allocate device memory.  It has no
+ * counterpart in the reference; it is for code under HIP graph capture, tight
+ * serving loops and harnesses that forbid hipMalloc.  Same arithmetic, same
+ * kernel choice and the same bits as ckq_gemm_nt_dev (formats CKQ_FMT_Q4_K,
+ * _Q5_K, _Q6_K, _Q8_0); the partial tiles of a K-split matrix-core GEMM live in
+ * a static device array of 4 MiB (one copy per GPU, held until the process
+ * ends) instead of the library's grow-only workspace.  A call whose split
+ * needs more (splits x M x N x 4 bytes; up to 16 splits are taken when the
+ * tile grid is smaller than the chip) returns CKQ_ESCRATCH (-4) and enqueues
+ * nothing: pass fewer tokens per call, or use ckq_gemm_nt_dev; no call allocates,
+ * frees or synchronizes.  Every call on a GPU shares that GPU's array: calls
+ * that overlap on one GPU (two streams, two threads) race.  The array's
+ * address is resolved once per device, by ckq_init() or by the first call on
+ * that device. */
+int ckq_gemm_nt_noalloc_dev(int fmt, const void *A_q8, const void *B, const float *bias, float *C,
+                            int M, int N, int K, long ldc, void *stream);
+
 /* Named forms mirroring Part 1. */
 int ckq_gemv_q4_k_q8_k_dev(float *y, const void *W, const void *x_q8, int M, int K, void *stream);
 int ckq_gemv_q5_k_q8_k_dev(float *y, const void *W, const void *x_q8, int M, int K, void *stream);
