@@ -288,3 +288,48 @@ def norm_err(y, ref):
     ref = np.asarray(ref, np.float64).reshape(-1)
     den = np.max(np.abs(ref))
     return float(np.max(np.abs(y - ref)) / den) if den > 0 else float(np.max(np.abs(y - ref)))
+
+
+# ---- the reference's thread pool as caller -------------------------------------------
+
+POOL_LIB = os.path.join(ORACLE_DIR, "_ref", "libckref_pool.so")
+
+
+def ref_pool(kernel_lib_path):
+    """The reference's thread pool + parallel decode dispatch (oracle/_ref/libckref_pool.so,
+    built from the reference's ck_threadpool.c, ckernel_strict.c and ck_parallel_decode.c),
+    with its undefined kernel symbols bound to the library at `kernel_lib_path`.
+
+    That library is (re)opened RTLD_GLOBAL first; the pool library is opened with lazy
+    binding, because it also names kernels that no quantized-path library defines and
+    that are never called here (ctypes itself always binds eagerly).  Returns None when
+    the pool library has not been built (no reference checkout at build time)."""
+    if not os.path.exists(POOL_LIB):
+        return None
+    key = "pool:" + kernel_lib_path
+    if key not in _cache:
+        ctypes.CDLL(kernel_lib_path, mode=ctypes.RTLD_GLOBAL)
+        libc = ctypes.CDLL(None)
+        libc.dlopen.restype = ctypes.c_void_p
+        libc.dlopen.argtypes = [ctypes.c_char_p, ctypes.c_int]
+        handle = libc.dlopen(POOL_LIB.encode(), os.RTLD_LAZY | os.RTLD_GLOBAL)
+        if not handle:
+            raise OSError("dlopen(%s) failed" % POOL_LIB)
+        L = ctypes.CDLL(POOL_LIB, handle=handle)
+        for name in ("gemv_q4_k_q8_k_parallel_dispatch", "gemv_q6_k_q8_k_parallel_dispatch",
+                     "gemv_q8_0_q8_0_parallel_dispatch", "gemv_q5_k_parallel_dispatch"):
+            fn = getattr(L, name)
+            fn.restype = None
+            fn.argtypes = [vp, vp, vp, ctypes.c_int, ctypes.c_int]
+        L.ck_set_num_threads.argtypes = [ctypes.c_int]
+        L.ck_threadpool_global.restype = vp
+        L.ck_threadpool_n_threads.argtypes = [vp]
+        _cache[key] = L
+    return _cache[key]
+
+
+def ref_pool_set_threads(pool, n):
+    """Recreate the reference's global pool with n threads."""
+    pool.ck_threadpool_global_destroy()
+    pool.ck_set_num_threads(n)
+    assert pool.ck_threadpool_n_threads(pool.ck_threadpool_global()) == n
