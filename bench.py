@@ -8,6 +8,12 @@ back-to-back on one stream.  Consecutive steps read different copies of the
 weight matrix, enough of them to exceed the 256 MB Infinity Cache, so the
 figure is an HBM figure; the cache-resident rate is reported beside it.
 
+Timing: whatever --steps says, the headline is the MEDIAN over 10 repetitions
+of max(256, steps) back-to-back launches each, every repetition bracketed by
+HIP events on the launch stream, after one untimed repetition (min and max are
+reported beside it).  The prefill GEMM is timed the same way, 5 repetitions of
+20 launches.
+
 Prints ONE JSON line:  python bench.py [--gpus 1] [--steps K] [--warmup W]
 """
 import argparse
@@ -15,6 +21,8 @@ import ctypes
 import importlib
 import json
 import os
+import re
+import statistics
 import sys
 import threading
 import time
@@ -25,9 +33,28 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 # HBM bytes per headline launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by the
-# same counters on the plain copy kernel (2.000 and 1.000); measurement recorded in
-# profiles/gemv_q4_k_11008x4096_hbm_traffic_pmc.txt
-TRAFFIC_BYTES_PER_LAUNCH = 25528524
+# same counters on the plain copy kernel: read from the committed counter summary
+# (its "traffic_bytes_per_launch:" and "kernel:" lines), so the figure and the kernel
+# it was taken on travel together; null when the summary is missing.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "gemv_q4_k_11008x4096_hbm_traffic_pmc.txt")
+REPS, LAUNCHES_PER_REP = 10, 256
+GEMM_REPS, GEMM_LAUNCHES_PER_REP = 5, 20
+
+
+def traffic_from_profile():
+    try:
+        text = open(TRAFFIC_PROFILE).read()
+    except OSError:
+        return None, None
+    m = re.search(r"^traffic_bytes_per_launch:\s*(\d+)", text, re.M)
+    k = re.search(r"^kernel:\s*(.+)$", text, re.M)
+    return (int(m.group(1)) if m else None), (k.group(1).strip() if k else None)
+
+
+def summarize(per_launch_seconds):
+    """median / min / max of the repetitions, in seconds per launch."""
+    v = sorted(per_launch_seconds)
+    return statistics.median(v), v[0], v[-1]
 INT8_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA, published
 MALL_BYTES = 256 << 20
 
@@ -70,14 +97,29 @@ class Harness:
             copies.append(torch.roll(base, shifts=i * 17, dims=0).contiguous().reshape(-1))
         return W, copies
 
-    def time_gemv(self, fmt, rows, K, M, copies, xq_d, steps, warmup):
-        """Average seconds per launch over `steps` back-to-back launches,
-        measured with events on the launch stream."""
+    def timed_reps(self, run, launches, reps):
+        """`reps` repetitions of run(launches), each bracketed by events on the
+        launch stream (torch's current stream, the one every *_dev call here is
+        given), after one untimed repetition.  Returns seconds per launch of
+        every repetition."""
+        torch = self.torch
+        run(launches)
+        torch.cuda.synchronize()
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+        for e0, e1 in ev:
+            e0.record()
+            run(launches)
+            e1.record()
+        torch.cuda.synchronize()
+        return [e0.elapsed_time(e1) * 1e-3 / launches for e0, e1 in ev]
+
+    def time_gemv(self, fmt, rows, K, M, copies, xq_d, launches=LAUNCHES_PER_REP, reps=REPS, warmup=0):
+        """Seconds per launch (median, min, max over the repetitions) of
+        back-to-back launches rotating through the weight copies; one C call
+        enqueues a whole repetition, so no Python runs between launches."""
         torch, P = self.torch, self.P
         out = torch.empty(M * rows, dtype=torch.float32, device="cuda")
         n = len(copies)
-        # one C call enqueues a whole rotation through the weight copies, so no
-        # Python runs between launches
         ops = [(fmt, xq_d, c, None, out, M, rows, K) for c in copies]
 
         def run(count):
@@ -87,43 +129,44 @@ class Harness:
             if rest:
                 P.dev_matmul_sequence(ops[:rest], repeat=1)
 
-        run(warmup)
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        t0 = time.perf_counter()
-        e0.record()
-        run(steps)
-        e1.record()
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
-        return e0.elapsed_time(e1) * 1e-3 / steps, wall / steps
+        if warmup:
+            run(warmup)
+        return summarize(self.timed_reps(run, launches, reps))
 
-
-    def time_read_floor(self, copies, nbytes, steps, warmup):
-        """Seconds per launch of the plain read kernel over the same rotated
-        weight buffers: what a launch costs that only pulls `nbytes` from HBM."""
+    def time_read_floor(self, copies, nbytes, launches=LAUNCHES_PER_REP, reps=5):
+        """Seconds per launch of kernels that only pull `nbytes` out of the same
+        rotated weight buffers: the one-load-per-lane read, and the fastest of a
+        small search over the tuned streaming read (grid = what the chip holds,
+        several loads in flight per lane)."""
         torch, L = self.torch, self.L
         sink = torch.zeros(4, dtype=torch.int32, device="cuda")
         stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
         n = len(copies)
+        ptrs = [ctypes.c_void_p(c.data_ptr()) for c in copies]
+        sp = ctypes.c_void_p(sink.data_ptr())
 
-        def run(count):
+        def plain(count):
             for i in range(count):
-                L.ckq_read_dev(ctypes.c_void_p(copies[i % n].data_ptr()), nbytes, ctypes.c_void_p(sink.data_ptr()), stream)
+                L.ckq_read_dev(ptrs[i % n], nbytes, sp, stream)
 
-        run(warmup)
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        run(steps)
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1e-3 / steps
+        res = {"plain": summarize(self.timed_reps(plain, launches, reps))[0]}
+        cus = torch.cuda.get_device_properties(0).multi_processor_count
+        best = None
+        for bpc in (2, 4, 8):
+            for unroll in (1, 2, 4, 8):
+                def tuned(count, b=bpc * cus, u=unroll):
+                    for i in range(count):
+                        L.ckq_read_tuned_dev(ptrs[i % n], nbytes, sp, b, u, stream)
+                t = summarize(self.timed_reps(tuned, launches, 3))[0]
+                if best is None or t < best[0]:
+                    best = (t, bpc * cus, unroll)
+        res["tuned"], res["tuned_blocks"], res["tuned_unroll"] = best
+        return res
 
-    def time_sequence(self, layers, steps, warmup):
+    def time_sequence(self, layers, launches, reps=5):
         """layers: list of op lists (one per rotated weight set); a step is one
-        pass over one layer's ops.  Returns seconds per step."""
-        torch, P = self.torch, self.P
+        pass over one layer's ops.  Returns median seconds per step."""
+        P = self.P
         flat = [op for layer in layers for op in layer]
         n = len(layers)
 
@@ -134,14 +177,47 @@ class Harness:
             for layer in layers[:rest]:
                 P.dev_matmul_sequence(layer, repeat=1)
 
-        run(warmup)
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        run(steps)
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1e-3 / steps
+        return summarize(self.timed_reps(run, launches, reps))[0]
+
+
+def drop_in_latency(H, W, xq, rows, K):
+    """Wall-clock microseconds per synchronous host-pointer call (PCIe copies of
+    x and y and a stream synchronisation included): what a generated model pays
+    per call when it links this library in place of the CPU kernels.  Never the
+    roofline figure."""
+    import numpy as np
+    T, L = H.T, H.L
+    p = T.ptr
+    y = np.zeros(rows, np.float32)
+
+    def med(fn, n):
+        fn(); fn()
+        ts = []
+        for _ in range(n):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return round(statistics.median(ts) * 1e6, 1)
+
+    out = {"shape": "Q4_K %dx%d, weights resident, x_q8 %d B up and y %d B down per call" % (rows, K, len(xq), 4 * rows)}
+    out["gemv_q4_k_q8_k"] = med(lambda: L.gemv_q4_k_q8_k(p(y), p(W), p(xq), rows, K), 200)
+    xf = T.normal(K, 0.0, 1.0, seed=5)
+    q = np.zeros(len(xq), np.uint8)
+    out["quantize_row_q8_k_K%d" % K] = med(lambda: L.quantize_row_q8_k(p(xf), p(q), K), 200)
+    pool = T.ref_pool(H.ckq.lib_path())
+    if pool is None:
+        out["pool_16_threads"] = None
+    else:
+        # the reference's own caller: ck_threadpool dispatching gemv_q4_k_q8_k_parallel_simd(ith, nth)
+        for threads in (8, 16):
+            T.ref_pool_set_threads(pool, threads)
+            for whole, tag in ((0, "rows"), (1, "whole")):
+                L.ckq_set_parallel_whole(whole)
+                out["parallel_dispatch_%d_threads_%s" % (threads, tag)] = med(
+                    lambda: pool.gemv_q4_k_q8_k_parallel_dispatch(p(y), p(W), p(xq), rows, K), 100)
+        L.ckq_set_parallel_whole(-1)          # back to the library's default
+        pool.ck_threadpool_global_destroy()
+    return out
 
 
 def cpu_baseline(rows, K, seconds_budget=12.0):
@@ -182,27 +258,41 @@ def cpu_baseline(rows, K, seconds_budget=12.0):
         t0 = time.perf_counter()
         one_call(threads)
         per = max(time.perf_counter() - t0, 1e-6)
-        iters = int(max(3, min(200, (seconds_budget / 2) / per)))
-        t0 = time.perf_counter()
+        iters = int(max(5, min(200, (seconds_budget / 2) / per)))
+        ts = []
         for _ in range(iters):
+            t0 = time.perf_counter()
             one_call(threads)
-        res[threads] = ((time.perf_counter() - t0) / iters, iters)
+            ts.append(time.perf_counter() - t0)
+        res[threads] = (statistics.median(ts), sum(ts) / len(ts), iters)
     bytes_ = gemv_bytes("q4_k", rows, K)
-    sec, iters = res[nth]
+    med, mean, iters = res[nth]
+    model = "unknown"
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
     return {
-        "value": round(bytes_ / sec / 1e9, 3), "unit": "GB/s", "cores": nth, "kind": kind,
-        "sample": "%d calls of %s %dx%d M=1 row-split over %d threads (%.2f ms/call); single thread %.2f ms/call = %.3f GB/s"
-                  % (iters, fn_name, rows, K, nth, sec * 1e3, res[1][0] * 1e3, bytes_ / res[1][0] / 1e9),
+        "value": round(bytes_ / med / 1e9, 3), "unit": "GB/s", "cores": nth, "kind": kind,
+        "host_cores": os.cpu_count(), "cpu_model": model,
+        "median_ms": round(med * 1e3, 4), "mean_ms": round(mean * 1e3, 4),
+        "single_thread_gbs": round(bytes_ / res[1][0] / 1e9, 3),
+        "sample": "%d calls of %s %dx%d M=1 row-split over %d threads (median %.2f ms/call, mean %.2f); "
+                  "single thread median %.2f ms/call" % (iters, fn_name, rows, K, nth, med * 1e3, mean * 1e3, res[1][0] * 1e3),
     }
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=2000)
-    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=32)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-extras", action="store_true", help="only the headline workload")
+    ap.add_argument("--no-extras", action="store_true", help="only the headline workload and the prefill GEMM")
+    ap.add_argument("--no-latency", action="store_true", help="skip the host-pointer (drop-in) latency leg")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch the plain copy kernel on a 256 MiB buffer (known traffic), for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings")
@@ -234,11 +324,13 @@ def main():
     err = T.norm_err(y, T.oracle_gemv("q4_k", W, xq_d.cpu().numpy(), rows, K))
     assert err <= 1e-4, "parity check failed before timing: %g" % err
 
-    sec, wall = H.time_gemv("q4_k", rows, K, M, copies, xq_d, a.steps, a.warmup)
+    launches = max(LAUNCHES_PER_REP, a.steps)
+    sec, sec_min, sec_max = H.time_gemv("q4_k", rows, K, M, copies, xq_d, launches, REPS, warmup=a.warmup)
     bytes_ = gemv_bytes("q4_k", rows, K, M)
     gbs = bytes_ / sec / 1e9
-    sec_hot, _ = H.time_gemv("q4_k", rows, K, M, copies[:1], xq_d, a.steps, a.warmup)
-    sec_read = H.time_read_floor(copies, len(W), min(a.steps, 500), 50)
+    sec_hot, _, _ = H.time_gemv("q4_k", rows, K, M, copies[:1], xq_d, launches, 5)
+    read = H.time_read_floor(copies, len(W))
+    traffic, traffic_kernel = traffic_from_profile()
 
     out = {
         "metric": "Q4_K GEMV GB/s (% HBM peak) at M=1; Q4_K x Q8_K GEMM TOPS at M=512",
@@ -248,25 +340,36 @@ def main():
         "config": {"workload": "Q4_K x Q8_K GEMV N=11008 K=4096 M=1", "weights": "seeded N(0,0.02) -> Q4_K",
                    "activations": "seeded N(0,1) -> Q8_K (quantized on the GPU)",
                    "weight_copies_rotated": len(copies), "bytes_per_step": bytes_},
+        "timing": {"method": "median of %d repetitions of %d back-to-back launches, HIP events on the launch stream, "
+                             "after one untimed repetition" % (REPS, launches),
+                   "median_us": round(sec * 1e6, 3), "min_us": round(sec_min * 1e6, 3), "max_us": round(sec_max * 1e6, 3)},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH},
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_kernel": traffic_kernel},
         "pct_hbm_peak": round(100.0 * gbs / HBM_PEAK_GBS, 2),
         "cache_resident_gbs": round(bytes_ / sec_hot / 1e9, 2),
-        # one launch of a kernel that only reads the same weight bytes from the same rotated buffers
-        "plain_read_same_bytes": {"us": round(sec_read * 1e6, 3), "gbs": round(len(W) / sec_read / 1e9, 1),
-                                  "gemv_over_read": round(sec / sec_read, 3)},
-        "host_wall_ms_per_step": round(wall * 1e3, 6),
+        # launches that only read the same weight bytes from the same rotated buffers: one 16-byte load per
+        # lane, and the fastest tuned streaming read (grid = resident blocks, several loads in flight per lane)
+        "plain_read_same_bytes": {"us": round(read["plain"] * 1e6, 3), "gbs": round(len(W) / read["plain"] / 1e9, 1),
+                                  "gemv_over_read": round(sec / read["plain"], 3)},
+        "tuned_read_same_bytes": {"us": round(read["tuned"] * 1e6, 3), "gbs": round(len(W) / read["tuned"] / 1e9, 1),
+                                  "blocks": read["tuned_blocks"], "loads_in_flight_per_lane": read["tuned_unroll"],
+                                  "gemv_over_read": round(sec / read["tuned"], 3)},
         "parity_norm_err": err,
     }
 
+    # the GEMM half of the metric: prefill, M=512 x N=11008 x K=4096
+    Mg = 512
+    xg = P.dev_quantize(P.to_device(T.normal(Mg * K, seed=99)), "q8_k", rows=Mg)
+    sg, sg_min, sg_max = H.time_gemv("q4_k", rows, K, Mg, copies[:2], xg, GEMM_LAUNCHES_PER_REP, GEMM_REPS)
+    ops = 2.0 * Mg * rows * K
+    out["roofline_gemm"] = {"bound": "mfma", "achieved": round(ops / sg / 1e12, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                            "frac": round(ops / sg / 1e12 / INT8_PEAK_TOPS, 4),
+                            "workload": "Q4_K x Q8_K GEMM M=512 N=11008 K=4096", "ops_per_launch": ops,
+                            "median_us": round(sg * 1e6, 2), "min_us": round(sg_min * 1e6, 2), "max_us": round(sg_max * 1e6, 2),
+                            "method": "median of %d repetitions of %d launches" % (GEMM_REPS, GEMM_LAUNCHES_PER_REP)}
+
     if not a.no_extras:
         extras = {}
-        # prefill GEMM, M=512 x N=11008 x K=4096
-        Mg = 512
-        xg = P.dev_quantize(P.to_device(T.normal(Mg * K, seed=99)), "q8_k", rows=Mg)
-        steps_g = max(3, min(20, a.steps // 100))
-        sg, _ = H.time_gemv("q4_k", rows, K, Mg, copies[:2], xg, steps_g, 2)
-        ops = 2.0 * Mg * rows * K
         extras["gemm_q4_k_q8_k_M512"] = {"tops": round(ops / sg / 1e12, 2), "ms": round(sg * 1e3, 4),
                                          "frac_int8_peak": round(ops / sg / 1e12 / INT8_PEAK_TOPS, 4),
                                          "ops_per_call": ops, "kernel": "two-plane int8 MFMA (v_mfma_i32_32x32x32_i8) + bf16 MFMA min term"}
@@ -274,7 +377,7 @@ def main():
         r6, k6 = 4096, 11008
         _, cps6 = H.weight_copies("q6_k", r6, k6, seed=66, min_total=1)
         x6 = P.dev_quantize(P.to_device(T.normal(Mg * k6, seed=67)), "q8_k", rows=Mg)
-        s6, _ = H.time_gemv("q6_k", r6, k6, Mg, cps6[:2] if len(cps6) > 1 else cps6, x6, steps_g, 2)
+        s6, _, _ = H.time_gemv("q6_k", r6, k6, Mg, cps6[:2] if len(cps6) > 1 else cps6, x6, GEMM_LAUNCHES_PER_REP, GEMM_REPS)
         ops6 = 2.0 * Mg * r6 * k6
         extras["gemm_q6_k_q8_k_M512_4096x11008"] = {"tops": round(ops6 / s6 / 1e12, 2), "ms": round(s6 * 1e3, 4),
                                                     "frac_int8_peak": round(ops6 / s6 / 1e12 / INT8_PEAK_TOPS, 4),
@@ -286,7 +389,7 @@ def main():
         for name8, r8, k8 in (("gemm_q8_0_q8_0_M512_9728x896", 9728, 896), ("gemm_q8_0_q8_0_M512_11008x4096", 11008, 4096)):
             _, cps8 = H.weight_copies("q8_0", r8, k8, seed=88, min_total=1)
             x8 = P.dev_quantize(P.to_device(T.normal(Mg * k8, seed=89)), "q8_0", rows=Mg)
-            s8, _ = H.time_gemv("q8_0", r8, k8, Mg, cps8[:2], x8, steps_g, 2)
+            s8, _, _ = H.time_gemv("q8_0", r8, k8, Mg, cps8[:2], x8, GEMM_LAUNCHES_PER_REP, GEMM_REPS)
             ops8 = 2.0 * Mg * r8 * k8
             extras[name8] = {"tops": round(ops8 / s8 / 1e12, 2), "ms": round(s8 * 1e3, 4),
                              "frac_int8_peak": round(ops8 / s8 / 1e12 / INT8_PEAK_TOPS, 4), "ops_per_call": ops8,
@@ -320,7 +423,7 @@ def main():
                                 ("lm_head_q8_0_151936x896", "q8_0", 151936, 896)):
             _, cps = H.weight_copies(fmt, r, k, seed=r + k)
             xq = P.dev_quantize(P.to_device(T.normal(k, seed=k)), T.act_fmt(fmt))
-            s, _ = H.time_gemv(fmt, r, k, 1, cps, xq, max(50, a.steps // 4), 20)
+            s, _, _ = H.time_gemv(fmt, r, k, 1, cps, xq, 128, 5)
             b = gemv_bytes(fmt, r, k)
             extras[name] = {"gbs": round(b / s / 1e9, 1), "us": round(s * 1e6, 2), "frac_hbm": round(b / s / 1e9 / HBM_PEAK_GBS, 4)}
             del cps
@@ -385,7 +488,7 @@ def main():
                 if li == 0:
                     lbytes += gemv_bytes(fmt, r, k)
             layers.append(ops)
-        s = H.time_sequence(layers, max(40, a.steps // 10), 8)
+        s = H.time_sequence(layers, 64, 5)
         extras["layer_7b_projection_set_M1"] = {"us": round(s * 1e6, 2), "gbs": round(lbytes / s / 1e9, 1), "bytes": lbytes,
                                                 "frac_hbm": round(lbytes / s / 1e9 / HBM_PEAK_GBS, 4), "launches": 4,
                                                 "note": "Q+K+V and gate+up each as one grouped launch"}
@@ -416,7 +519,7 @@ def main():
                 if hi == 0:
                     nbytes += gemv_bytes("q8_0", 151936, 896, Mb)
                 layers.append(ops)
-            s = H.time_sequence(layers, max(20, a.steps // 40), 4)
+            s = H.time_sequence(layers, 32, 5)
             small["M%d" % Mb] = {"us": round(s * 1e6, 2), "gbs": round(nbytes / s / 1e9, 1), "tokens_per_s": round(Mb / s, 1)}
             del layers
         extras["small_model_decode_q5_k_layer_plus_q8_0_head"] = small
@@ -424,6 +527,8 @@ def main():
         torch.cuda.empty_cache()
         out["extras"] = extras
 
+    if not a.no_latency:
+        out["drop_in_latency_us"] = drop_in_latency(H, W, xq_d.cpu().numpy(), rows, K)
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline(rows, K)
     print(json.dumps(out))

@@ -124,6 +124,7 @@ _SIGS = {
     "ckq_gemm_block_sums_dev": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "ckq_copy_dev": (_i, [_vp, _vp, _c.c_size_t, _vp]),
     "ckq_read_dev": (_i, [_vp, _c.c_size_t, _vp, _vp]),
+    "ckq_read_tuned_dev": (_i, [_vp, _c.c_size_t, _vp, _i, _i, _vp]),
     "ckq_init": (_i, []),
     "ckq_synchronize": (_i, []),
     "ckq_weights_register": (_i, [_vp, _c.c_size_t]),

@@ -100,6 +100,7 @@ void ckq_grid_chunk(long total, long per, long c, long *first, long *count);
 /* Plain device copy kernel (calibration of the memory counters / roofline). */
 int ckq_launch_copy(void *dst, const void *src, size_t bytes, void *stream);
 int ckq_launch_read(const void *src, size_t bytes, void *sink, void *stream);
+int ckq_launch_read_tuned(const void *src, size_t bytes, void *sink, int blocks, int unroll, void *stream);
 
 #ifdef __cplusplus
 }

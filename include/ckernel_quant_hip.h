@@ -328,6 +328,11 @@ int ckq_copy_dev(void *dst, const void *src, size_t bytes, void *stream);
  * of it is the time floor of a GEMV whose weights are `bytes` large; the
  * benchmark reports it beside the GEMV figure. */
 int ckq_read_dev(const void *src, size_t bytes, void *sink, void *stream);
+/* The same read as a tuned streaming kernel: `blocks` blocks of 256 threads
+ * stride through the buffer, every lane with `unroll` (1, 2, 4 or 8)
+ * independent 16-byte loads in flight per trip.  The benchmark searches
+ * (blocks, unroll) and reports the fastest as the launch floor. */
+int ckq_read_tuned_dev(const void *src, size_t bytes, void *sink, int blocks, int unroll, void *stream);
 
 /* ======================================================================== */
 /* Library control                                                           */
@@ -358,8 +363,13 @@ int  ckq_weights_resident(size_t *bytes);
 void ckq_weights_invalidate(const void *W);
 void ckq_weights_clear(void);
 void ckq_weights_set_cache(int enabled);
-/* Thread-split entry points: 0 (default) = every call computes its own row
- * range; 1 = the ith==0 call computes all rows and the others return. */
+/* Thread-split entry points (*_parallel, *_parallel_simd): 1 (default; also
+ * CKQ_PARALLEL_MODE=whole) = the ith == 0 call computes all rows in one launch
+ * and the other threads return at once, which is what a thread pool that calls
+ * every ith wants (one upload, launch and download instead of nth serialized
+ * ones); 0 (CKQ_PARALLEL_MODE=rows) = every call computes exactly its own row
+ * range, for callers that invoke single ith values; a negative value restores
+ * the default. */
 void ckq_set_parallel_whole(int enabled);
 /* Which kernel serves a matmul of more than eight tokens (up to eight always
  * take the weight-streaming kernel, one pass over the weights).  AUTO, the

@@ -193,6 +193,10 @@ def test_parallel_union_equals_serial(fmt):
     rows, K = 301, 1024
     W, _, xq = make_case(fmt, rows, K, "rand", 5)
     serial = P.gemv(fmt, W, xq, rows, K)
+    # default ("whole") mode: the union over ith is the serial result, computed by the ith == 0 call
+    y = P.gemv_parallel(fmt, W, xq, rows, K, 8, True)
+    assert np.array_equal(y, serial)
+    ckq.lib().ckq_set_parallel_whole(0)             # "rows" mode: every call computes its own range
     for nth in (1, 3, 8, 64):
         for simd in (False, True):
             say("parallel", fmt, "nth", nth, "simd", simd)
@@ -212,8 +216,11 @@ def test_parallel_union_equals_serial(fmt):
         fn = getattr(ckq.lib(), P._GEMV[fmt] + "_parallel_simd")
         fn(T.ptr(y), T.ptr(W), T.ptr(xq), rows, K, 0, 8)
         assert np.array_equal(y, serial)
+        y = np.full(rows, -5.0, np.float32)
+        fn(T.ptr(y), T.ptr(W), T.ptr(xq), rows, K, 3, 8)     # another ith: returns at once
+        assert np.all(y == -5.0)
     finally:
-        ckq.lib().ckq_set_parallel_whole(0)
+        ckq.lib().ckq_set_parallel_whole(-1)
 
 
 # ---- batched decode / small GEMM -------------------------------------------------------

@@ -33,7 +33,7 @@ def pool():
         pytest.skip("oracle/_ref/libckref_pool.so has not been built (needs the reference checkout at build time)")
     yield p
     p.ck_threadpool_global_destroy()
-    L.ckq_set_parallel_whole(0)
+    L.ckq_set_parallel_whole(-1)
     L.ckq_weights_clear()
 
 
