@@ -285,6 +285,44 @@ def cpu_baseline(rows, K, seconds_budget=12.0):
     }
 
 
+# name -> (format, output rows, K, tokens): single workloads a profiler run can ask for with --only
+PROFILE_WORKLOADS = {
+    "gemv_q4_k_11008x4096": ("q4_k", 11008, 4096, 1),
+    "gemm_q4_k_M512_11008x4096": ("q4_k", 11008, 4096, 512),
+    "gemv_q6_k_32000x4096": ("q6_k", 32000, 4096, 1),
+    "gemv_q6_k_4096x11008": ("q6_k", 4096, 11008, 1),
+    "gemm_q6_k_M512_4096x11008": ("q6_k", 4096, 11008, 512),
+    "gemv_q4_k_4096x4096": ("q4_k", 4096, 4096, 1),
+}
+
+
+def copy_calibration(H):
+    """The plain copy kernel on 256 MiB, eight launches: known traffic for
+    scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings."""
+    torch = H.torch
+    n = 256 << 20
+    src = torch.empty(n, dtype=torch.uint8, device="cuda").random_(0, 255)
+    dst = torch.empty_like(src)
+    for _ in range(8):
+        H.ckq.api.check(H.L.ckq_copy_dev(ctypes.c_void_p(dst.data_ptr()), ctypes.c_void_p(src.data_ptr()), n,
+                                         ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)), "ckq_copy_dev")
+    torch.cuda.synchronize()
+
+
+def run_only(H, name, steps, warmup, calibrate):
+    fmt, rows, K, M = PROFILE_WORKLOADS[name]
+    P, T = H.P, H.T
+    _, copies = H.weight_copies(fmt, rows, K, seed=rows + K, min_total=(3 * MALL_BYTES // 2) if M == 1 else 1)
+    if M > 1:
+        copies = copies[:2]
+    x = P.dev_quantize(P.to_device(T.normal(M * K, 0.0, 1.0, seed=K + M)), T.act_fmt(fmt), rows=M)
+    if calibrate:
+        copy_calibration(H)
+    med, lo, hi = H.time_gemv(fmt, rows, K, M, copies, x, max(1, steps), 3, warmup=warmup)
+    print(json.dumps({"only": name, "launches_per_repetition": max(1, steps), "repetitions": 4,
+                      "median_us": round(med * 1e6, 3), "min_us": round(lo * 1e6, 3), "max_us": round(hi * 1e6, 3)}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -293,6 +331,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="only the headline workload and the prefill GEMM")
     ap.add_argument("--no-latency", action="store_true", help="skip the host-pointer (drop-in) latency leg")
+    ap.add_argument("--only", choices=sorted(PROFILE_WORKLOADS),
+                    help="launch just this workload --steps times and exit (for rocprofv3 runs): no parity guard, "
+                         "no CPU leg, a short JSON line")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch the plain copy kernel on a 256 MiB buffer (known traffic), for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings")
@@ -302,6 +343,9 @@ def main():
                  "rows, one all-gather per matmul; nothing here uses a second GPU)" % a.gpus)
 
     H = Harness()
+    if a.only:
+        run_only(H, a.only, a.steps, a.warmup, a.calibrate_copy)
+        return
     torch, P, T = H.torch, H.P, H.T
     rows, K, M = 11008, 4096, 1
     xf = T.normal(K, 0.0, 1.0, seed=4242)
@@ -309,14 +353,7 @@ def main():
     W, copies = H.weight_copies("q4_k", rows, K, seed=4243)
 
     if a.calibrate_copy:
-        n = 256 << 20
-        src = torch.empty(n, dtype=torch.uint8, device="cuda").random_(0, 255)
-        dst = torch.empty_like(src)
-        for _ in range(8):
-            H.ckq.api.check(H.L.ckq_copy_dev(ctypes.c_void_p(dst.data_ptr()), ctypes.c_void_p(src.data_ptr()), n,
-                                             ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)), "ckq_copy_dev")
-        torch.cuda.synchronize()
-        del src, dst
+        copy_calibration(H)
 
     # parity guard on the exact buffers being timed
     import numpy as np
