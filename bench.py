@@ -529,7 +529,35 @@ def main():
         extras["layer_7b_projection_set_M1"] = {"us": round(s * 1e6, 2), "gbs": round(lbytes / s / 1e9, 1), "bytes": lbytes,
                                                 "frac_hbm": round(lbytes / s / 1e9 / HBM_PEAK_GBS, 4), "launches": 4,
                                                 "note": "Q+K+V and gate+up each as one grouped launch"}
-        del layers, keep
+        # the same layer as the REAL chain, activation quantizers included, one C call per layer:
+        # RMSNorm->Q8_K | Q+K+V | Q8_K(attention output; V's output stands in) | O | RMSNorm->Q8_K |
+        # gate+up | SiLU(gate)*up->Q8_K | down: four matmul launches and four producer launches
+        f32z = lambda n: torch.zeros(n, dtype=torch.float32, device="cuda")
+        u8z = lambda n: torch.zeros(n, dtype=torch.uint8, device="cuda")
+        xres = P.to_device(T.normal(4096, 0.0, 1.0, seed=32))
+        gam = P.to_device(T.normal(4096, 1.0, 0.2, seed=33))
+        chains = []
+        for ops in layers:
+            (q_, k_, v_, o_, g_, u_, d_) = ops
+            xq_, aq_, fq_ = u8z(4672), u8z(4672), u8z(4672)
+            hq_ = u8z(43 * 292)
+            keep += [xq_, aq_, fq_, hq_]
+            chains.append([
+                ("rmsnorm_q8_k", xres, gam, xq_, 1, 4096, 4096, 1e-5),
+                ("q4_k", xq_, q_[2], None, q_[4], 1, 4096, 4096), ("q4_k", xq_, k_[2], None, k_[4], 1, 4096, 4096),
+                ("q4_k", xq_, v_[2], None, v_[4], 1, 4096, 4096),
+                ("quantize_q8_k", v_[4], None, aq_, 1, 4096),
+                ("q4_k", aq_, o_[2], None, o_[4], 1, 4096, 4096),
+                ("rmsnorm_q8_k", o_[4], gam, fq_, 1, 4096, 4096, 1e-5),
+                ("q4_k", fq_, g_[2], None, g_[4], 1, 11008, 4096), ("q4_k", fq_, u_[2], None, u_[4], 1, 11008, 4096),
+                ("swiglu_q8_k", g_[4], u_[4], hq_, 1, 11008, 11008),
+                ("q6_k", hq_, d_[2], None, d_[4], 1, 4096, 11008)])
+        sc = H.time_sequence(chains, 64, 5)
+        extras["layer_7b_decode_chain_M1"] = {"us": round(sc * 1e6, 2), "matmul_only_us": round(s * 1e6, 2),
+                                              "producers_us": round((sc - s) * 1e6, 2), "launches": 8,
+                                              "gbs_of_weight_bytes": round(lbytes / sc / 1e9, 1),
+                                              "note": "norm->Q8_K, Q+K+V, Q8_K, O, norm->Q8_K, gate+up, SwiGLU->Q8_K, down in one C call"}
+        del layers, keep, chains
         torch.cuda.empty_cache()
 
         # small-model batched decode (Qwen2-0.5B-like: hidden 896 padded to K=1024, Q5_K

@@ -145,7 +145,10 @@ _SIGS = {
 class MatmulOp(ctypes.Structure):
     """ckq_matmul_op of include/ckernel_quant_hip.h."""
     _fields_ = [("fmt", _i), ("M", _i), ("N", _i), ("K", _i), ("ldc", _l),
-                ("A_q8", _vp), ("B", _vp), ("bias", _vp), ("C", _vp)]
+                ("A_q8", _vp), ("B", _vp), ("bias", _vp), ("C", _vp), ("eps", _c.c_float)]
+
+
+STEP = {"quantize_q8_k": 32, "quantize_q8_0": 33, "rmsnorm_q8_k": 34, "swiglu_q8_k": 35}
 
 
 _lib = None

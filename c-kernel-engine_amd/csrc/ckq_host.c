@@ -1183,6 +1183,23 @@ static int ops_independent(const ckq_matmul_op *p, const ckq_matmul_op *q)
     return 1;
 }
 
+/* A producer entry of a sequence: the activation quantizer in front of the matmuls that follow. */
+static int issue_producer(const ckq_matmul_op *o, void *stream)
+{
+    if (!o->A_q8 || !o->C || o->M <= 0 || o->K <= 0) return CKQ_EINVAL;
+    const long ld = o->ldc ? o->ldc : o->K;
+    switch (o->fmt) {
+    case CKQ_STEP_QUANTIZE_Q8_K: return ckq_launch_quantize_q8_k((const float *)o->A_q8, o->C, o->M, o->K, stream);
+    case CKQ_STEP_QUANTIZE_Q8_0: return ckq_launch_quantize_q8_0((const float *)o->A_q8, o->C, o->M, o->K, stream);
+    case CKQ_STEP_RMSNORM_Q8_K:
+        if (ld > 0x7fffffff) return CKQ_EINVAL;
+        return ckq_launch_rmsnorm_q8_k_fused((const float *)o->A_q8, (const float *)o->B, o->C, o->M, o->K, (int)ld, o->eps, stream);
+    case CKQ_STEP_SWIGLU_Q8_K:
+        return ckq_launch_swiglu_q8_k((const float *)o->A_q8, (const float *)o->B, o->C, o->M, o->K, ld, stream);
+    default: return CKQ_EFORMAT;
+    }
+}
+
 int ckq_matmul_sequence_dev(const ckq_matmul_op *ops, int nops, int repeat, void *stream)
 {
     if (!ops || nops <= 0 || repeat <= 0) return CKQ_EINVAL;
@@ -1190,6 +1207,12 @@ int ckq_matmul_sequence_dev(const ckq_matmul_op *ops, int nops, int repeat, void
     for (int r = 0; r < repeat; ++r)
         for (int i = 0; i < nops;) {
             const ckq_matmul_op *o = &ops[i];
+            if (o->fmt >= CKQ_STEP_QUANTIZE_Q8_K && o->fmt <= CKQ_STEP_SWIGLU_Q8_K) {
+                const int rc = issue_producer(o, stream);
+                if (rc) return rc;
+                ++i;
+                continue;
+            }
             /* consecutive entries of one shape that do not depend on each other
              * (Q/K/V, gate/up) go out as one launch */
             int n = 1;

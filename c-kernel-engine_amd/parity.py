@@ -9,7 +9,7 @@ import ctypes
 
 import numpy as np
 
-from .api import BLOCK_ELEMS, FMT, MatmulOp, check, lib, row_bytes
+from .api import BLOCK_ELEMS, FMT, STEP, MatmulOp, check, lib, row_bytes
 
 _vp = ctypes.c_void_p
 
@@ -237,10 +237,20 @@ def dev_gemm_block_sums(fmt, A_t, B_t, bias_t, M, N, K):
 
 
 def dev_matmul_sequence(ops, repeat=1):
-    """ops: list of (fmt, A_t, B_t, bias_t, C_t, M, N, K); enqueued back-to-back
-    `repeat` times by one C call (no Python between launches)."""
+    """ops: list of matmul entries (fmt, A_t, B_t, bias_t, C_t, M, N, K) and producer
+    entries (step, A_t, B_t or None, C_t, M, K[, ld[, eps]]) with step one of
+    "quantize_q8_k", "quantize_q8_0", "rmsnorm_q8_k", "swiglu_q8_k"; enqueued
+    back-to-back `repeat` times by one C call (no Python between launches)."""
     arr = (MatmulOp * len(ops))()
-    for i, (fmt, A_t, B_t, bias_t, C_t, M, N, K) in enumerate(ops):
-        arr[i] = MatmulOp(FMT[fmt], M, N, K, N, A_t.data_ptr(), B_t.data_ptr(),
-                          bias_t.data_ptr() if bias_t is not None else None, C_t.data_ptr())
+    for i, op in enumerate(ops):
+        if op[0] in STEP:
+            step, A_t, B_t, C_t, M, K = op[:6]
+            ld = op[6] if len(op) > 6 else 0
+            eps = op[7] if len(op) > 7 else 0.0
+            arr[i] = MatmulOp(STEP[step], M, 0, K, ld, A_t.data_ptr(), B_t.data_ptr() if B_t is not None else None,
+                              None, C_t.data_ptr(), eps)
+        else:
+            fmt, A_t, B_t, bias_t, C_t, M, N, K = op
+            arr[i] = MatmulOp(FMT[fmt], M, N, K, N, A_t.data_ptr(), B_t.data_ptr(),
+                              bias_t.data_ptr() if bias_t is not None else None, C_t.data_ptr(), 0.0)
     check(lib().ckq_matmul_sequence_dev(ctypes.cast(arr, _vp), len(ops), repeat, _stream()), "ckq_matmul_sequence_dev")

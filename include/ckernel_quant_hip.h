@@ -273,23 +273,38 @@ int ckq_swiglu_q8_k_dev(const float *gate, const float *up, void *y, int rows, i
 int ckq_gemm_nt_f32act_dev(int fmt, const float *A, const void *B, const float *bias, float *C,
                            int M, int N, int K, long ldc, void *stream);
 
-/* A list of matmuls enqueued back-to-back, the whole list `repeat` times: the
- * per-token projection set of a decoder layer (Q/K/V/O, gate/up, down) is one
- * such list.  Entry i computes C[m*ldc + n] as ckq_gemm_nt_dev does, with the
- * same bits.  Up to four consecutive entries of one format, input width and
- * token count (at most eight tokens; their row counts may
- * differ), none of which writes memory another reads or writes (Q/K/V,
- * gate/up of a decode step), are issued as ONE launch. */
+/* A list of steps enqueued back-to-back, the whole list `repeat` times: the
+ * per-token chain of a decoder layer (norm -> Q8_K -> Q/K/V ... -> down) is one
+ * such list.  A matmul entry (fmt = a ckq_format weight tag) computes
+ * C[m*ldc + n] as ckq_gemm_nt_dev does, with the same bits.  Up to four
+ * consecutive matmul entries of one format, input width and token count (at
+ * most eight tokens; their row counts may differ), none of which writes memory
+ * another reads or writes (Q/K/V, gate/up of a decode step), are issued as ONE
+ * launch.  A producer entry (fmt = one of CKQ_STEP_*) runs the activation
+ * quantizer that feeds the matmuls after it, so that a whole chain is one C
+ * call:
+ *   CKQ_STEP_QUANTIZE_Q8_K  C = Q8_K blocks of the M rows of K floats at A_q8 (contiguous rows)
+ *   CKQ_STEP_QUANTIZE_Q8_0  the same with Q8_0 blocks
+ *   CKQ_STEP_RMSNORM_Q8_K   C = Q8_K(RMSNorm(row) * gamma): M rows of K floats at A_q8, rows ldc floats
+ *                           apart (0 = K), gamma at B, epsilon in eps (rmsnorm_q8_k_fused)
+ *   CKQ_STEP_SWIGLU_Q8_K    C = Q8_K(SiLU(gate) * up): gate at A_q8, up at B, M rows of K floats, rows
+ *                           ldc floats apart (0 = K) (ckq_swiglu_q8_k_dev)
+ * N and bias are unused by producer entries; C is the block buffer. */
+#define CKQ_STEP_QUANTIZE_Q8_K 32
+#define CKQ_STEP_QUANTIZE_Q8_0 33
+#define CKQ_STEP_RMSNORM_Q8_K  34
+#define CKQ_STEP_SWIGLU_Q8_K   35
 typedef struct {
-    int          fmt;    /* ckq_format weight tag */
+    int          fmt;    /* ckq_format weight tag, or a CKQ_STEP_* producer tag */
     int          M;      /* tokens */
     int          N;      /* output rows */
     int          K;      /* input width */
-    long         ldc;    /* output row stride (elements) */
-    const void  *A_q8;   /* activations, M rows */
-    const void  *B;      /* weights, N rows */
+    long         ldc;    /* output row stride (elements); producers: input row stride */
+    const void  *A_q8;   /* activations, M rows; producers: fp32 input */
+    const void  *B;      /* weights, N rows; producers: gamma / up */
     const float *bias;   /* N, or NULL */
-    float       *C;      /* M x ldc */
+    float       *C;      /* M x ldc; producers: the quantized blocks */
+    float        eps;    /* CKQ_STEP_RMSNORM_Q8_K only */
 } ckq_matmul_op;
 int ckq_matmul_sequence_dev(const ckq_matmul_op *ops, int nops, int repeat, void *stream);
 

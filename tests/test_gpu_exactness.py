@@ -6,6 +6,7 @@ GEMMs, fp16 scales at the ends of their range, and parity at the benchmark's
 batched-decode and grouped-launch shapes.  Expected integers come from NumPy
 decoders written from the format definitions (tests/ckq_testlib.py), not from
 the oracle's C code."""
+import ctypes
 import importlib
 import sys
 
@@ -325,6 +326,59 @@ def test_sequence_group_whose_tile_exceeds_lds_is_issued_separately():
     P.dev_matmul_sequence([(fmt, xd, Wd[i], None, outs[i], M, N, K) for i in range(2)])
     for i in range(2):
         assert T.norm_err(outs[i].cpu().numpy().reshape(M, N), T.oracle_gemm_nt(fmt, xq, Ws[i], None, M, N, K)) <= TOL, i
+
+
+def test_sequence_with_producer_steps():
+    """A decode layer's chain as ONE C call: RMSNorm->Q8_K, Q/K/V (one grouped
+    launch), Q8_K of the attention output, O, RMSNorm->Q8_K, gate/up (grouped),
+    SiLU(gate)*up->Q8_K, down.  Every buffer has the bits of the same steps issued
+    one call at a time; the producers are bit-exact with the oracle."""
+    import torch
+    D, F, KV, M = 1024, 2816, 256, 1
+    x = T.normal(M * D, 0.0, 1.0, 91)
+    gam1, gam2 = T.normal(D, 1.0, 0.2, seed=92), T.normal(D, 1.0, 0.2, seed=93)
+    Wq, Wk, Wv = (T.synth_weights("q4_k", n, D, seed=94 + i) for i, n in enumerate((D, KV, KV)))
+    Wo = T.synth_weights("q4_k", D, D, seed=97)
+    Wg, Wu = T.synth_weights("q4_k", F, D, seed=98), T.synth_weights("q4_k", F, D, seed=99)
+    Wd = T.synth_weights("q6_k", D, F, seed=100)
+    dev = {k: P.to_device(v) for k, v in dict(x=x, g1=gam1, g2=gam2, Wq=Wq, Wk=Wk, Wv=Wv, Wo=Wo, Wg=Wg, Wu=Wu, Wd=Wd).items()}
+    f32 = lambda n: torch.zeros(n, dtype=torch.float32, device="cuda")
+    u8 = lambda n: torch.zeros(n, dtype=torch.uint8, device="cuda")
+
+    def buffers():
+        return dict(xq=u8(T.row_bytes("q8_k", D)), q=f32(D), k=f32(KV), v=f32(KV), aq=u8(T.row_bytes("q8_k", D)), o=f32(D),
+                    fq=u8(T.row_bytes("q8_k", D)), g=f32(F), u=f32(F), hq=u8(T.row_bytes("q8_k", F)), y=f32(D))
+
+    def steps(b):
+        return [("rmsnorm_q8_k", dev["x"], dev["g1"], b["xq"], M, D, D, 1e-5),
+                ("q4_k", b["xq"], dev["Wq"], None, b["q"], M, D, D),
+                ("q4_k", b["xq"], dev["Wk"], None, b["k"], M, KV, D),
+                ("q4_k", b["xq"], dev["Wv"], None, b["v"], M, KV, D),
+                ("quantize_q8_k", b["q"], None, b["aq"], M, D),              # stands in for the attention output
+                ("q4_k", b["aq"], dev["Wo"], None, b["o"], M, D, D),
+                ("rmsnorm_q8_k", b["o"], dev["g2"], b["fq"], M, D, D, 1e-5),
+                ("q4_k", b["fq"], dev["Wg"], None, b["g"], M, F, D),
+                ("q4_k", b["fq"], dev["Wu"], None, b["u"], M, F, D),
+                ("swiglu_q8_k", b["g"], b["u"], b["hq"], M, F, F),
+                ("q6_k", b["hq"], dev["Wd"], None, b["y"], M, D, F)]
+
+    say("decode chain with producer steps, one call")
+    one = buffers()
+    P.dev_matmul_sequence(steps(one), repeat=2)
+    sep = buffers()
+    for st in steps(sep):
+        P.dev_matmul_sequence([st])
+    torch.cuda.synchronize()
+    for name in one:
+        assert torch.equal(one[name], sep[name]), name
+    # producers against the oracle, matmuls against the oracle on the device's own activations
+    xq = one["xq"].cpu().numpy()
+    want = np.zeros_like(xq)
+    T.oracle().orc_rmsnorm_q8_k_fused(T.ptr(x), T.ptr(gam1), T.ptr(want), M, D, D, ctypes.c_float(1e-5))
+    assert np.array_equal(xq, want)
+    assert np.array_equal(one["aq"].cpu().numpy(), T.oracle_quantize(one["q"].cpu().numpy(), "q8_k"))
+    assert T.norm_err(one["q"].cpu().numpy(), T.oracle_gemv("q4_k", Wq, xq, D, D)) <= TOL
+    assert T.norm_err(one["y"].cpu().numpy(), T.oracle_gemv("q6_k", Wd, one["hq"].cpu().numpy(), D, F)) <= TOL
 
 
 # ---- host-pointer paths with the weight cache off, long contexts ---------------------------------------
