@@ -557,8 +557,32 @@ def main():
                                               "producers_us": round((sc - s) * 1e6, 2), "launches": 8,
                                               "gbs_of_weight_bytes": round(lbytes / sc / 1e9, 1),
                                               "note": "norm->Q8_K, Q+K+V, Q8_K, O, norm->Q8_K, gate+up, SwiGLU->Q8_K, down in one C call"}
-        del layers, keep, chains
+        # the same chain with the plain quantizer step folded into its consumer (the O
+        # projection quantizes the attention output while it stages it): seven launches
+        fused = []
+        for ch in chains:
+            fused.append(ch[:4] + [("q4_k+f32q", ch[4][1], ch[5][2], None, ch[5][4], 1, 4096, 4096)] + ch[6:])
+        sf = H.time_sequence(fused, 64, 5)
+        extras["layer_7b_decode_chain_M1"]["quantizer_in_consumer_us"] = round(sf * 1e6, 2)
+        del layers, keep, chains, fused
         torch.cuda.empty_cache()
+
+        # fp32 -> Q8_K as its own launch in front of the GEMV against the same step inside the
+        # GEMV's activation staging (every block of the GEMV then quantizes the row itself)
+        qic = {}
+        for fmt, r, k in (("q4_k", 4096, 4096), ("q4_k", 11008, 4096), ("q6_k", 4096, 11008)):
+            _, cps = H.weight_copies(fmt, r, k, seed=r + k + 7)
+            xf = P.to_device(T.normal(k, 0.0, 1.0, seed=51))
+            xq = torch.zeros(T.row_bytes("q8_k", k), dtype=torch.uint8, device="cuda")
+            y = torch.zeros(r, dtype=torch.float32, device="cuda")
+            two = H.time_sequence([[("quantize_q8_k", xf, None, xq, 1, k), (fmt, xq, c, None, y, 1, r, k)] for c in cps], 128, 5)
+            one = H.time_sequence([[(fmt + "+f32q", xf, c, None, y, 1, r, k)] for c in cps], 128, 5)
+            alone = H.time_sequence([[(fmt, xq, c, None, y, 1, r, k)] for c in cps], 128, 5)
+            qic["%s_%dx%d" % (fmt, r, k)] = {"quantizer_then_gemv_us": round(two * 1e6, 2), "quantizer_in_gemv_us": round(one * 1e6, 2),
+                                             "gemv_alone_us": round(alone * 1e6, 2)}
+            del cps
+            torch.cuda.empty_cache()
+        extras["quantizer_in_consumer_M1"] = qic
 
         # small-model batched decode (Qwen2-0.5B-like: hidden 896 padded to K=1024, Q5_K
         # projections, Q8_0 LM head 151936x896), M tokens per step

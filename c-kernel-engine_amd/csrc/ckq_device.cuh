@@ -83,3 +83,51 @@ __device__ __forceinline__ T group_sum(T v)
     if (LANES >= 64) v += dpp_get<0x143, 0xC>(v); /* row_bcast31 into rows 2,3 */
     return v;
 }
+
+/* x86 cvtps2dq + saturating packs: round to nearest even, NaN -> -128. */
+__device__ __forceinline__ int rne_sat_i8(float p)
+{
+    if (p != p) return -128;
+    const float r = __builtin_rintf(p);
+    return (int)fminf(fmaxf(r, -128.0f), 127.0f);
+}
+
+/* One wave turns 256 fp32 values (lane l holds elements 4l..4l+3 in e) into
+ * the 292-byte Q8_K block at `out` (global or LDS), with the reference's rules
+ * (quantize_row_q8_k_sse.c:22-82): the scale comes from the FIRST element of
+ * largest magnitude, sign kept, iscale = -127/max, q = RNE(x*iscale)
+ * saturated, bsums over 16 elements, d = 1/iscale; an all-zero block is 292
+ * zero bytes. */
+__device__ __forceinline__ void q8k_quantize_block(const float (&e)[4], int lane, uint8_t *out)
+{
+    float amax = 0.0f, smax = 0.0f;
+    int idx = 4 * lane;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float ax = fabsf(e[i]);
+        if (ax > amax) { amax = ax; smax = e[i]; idx = 4 * lane + i; }
+    }
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const float oa = __shfl_xor(amax, off), os = __shfl_xor(smax, off);
+        const int   oi = __shfl_xor(idx, off);
+        if (oa > amax || (oa == amax && oi < idx)) { amax = oa; smax = os; idx = oi; }
+    }
+    if (amax == 0.0f) {
+        reinterpret_cast<u32 *>(out)[lane] = 0;
+        if (lane < 9) reinterpret_cast<u32 *>(out)[64 + lane] = 0;
+        return;
+    }
+    const float iscale = -127.0f / smax;
+    int q[4], s = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        q[i] = rne_sat_i8(__fmul_rn(e[i], iscale));
+        s += q[i];
+    }
+    const u32 packed = (u32)(q[0] & 0xff) | ((u32)(q[1] & 0xff) << 8) | ((u32)(q[2] & 0xff) << 16) | ((u32)(q[3] & 0xff) << 24);
+    reinterpret_cast<u32 *>(out + 4)[lane] = packed;
+    s = group_sum<4>(s);                       /* 16 consecutive elements = 4 lanes */
+    if ((lane & 3) == 3) reinterpret_cast<int16_t *>(out + 260)[lane >> 2] = (int16_t)s;
+    if (lane == 0) *reinterpret_cast<float *>(out) = 1.0f / iscale;
+}

@@ -22,6 +22,7 @@ struct GemvArgs {
     int32_t       *sub;
     int  nrows, npos, ntok, row0, row1, nsub_row;
     long wrow, xrow, ldy;
+    int  xq;        /* host side only: X holds fp32 rows that the kernel quantizes to Q8_K while staging them */
 };
 
 /* Problems 1..3 of a grouped launch (blockIdx.z = g > 0); problem 0 is in GemvArgs. */
@@ -46,7 +47,7 @@ struct GemvGroup {
  * summed over the LPR lanes with a fixed DPP tree; the last lane of the group
  * stores.
  */
-template <class F, int LPR, int PPL, int MT, int RPI, bool DUMP, int WPB, bool LDSX, bool GRP = false>
+template <class F, int LPR, int PPL, int MT, int RPI, bool DUMP, int WPB, bool LDSX, bool GRP = false, bool XQ = false>
 __global__ void __launch_bounds__(64 * WPB) __attribute__((amdgpu_waves_per_eu(DUMP ? 1 : MT == 1 && PPL == 1 && RPI == 1 ? F::OCC1 : MT == 1 && PPL == 1 && RPI == 2 && LPR == 64 ? F::OCC2 : MT >= 4 && PPL == 1 ? 4 : 1)))
 gemv_kernel(const uint8_t *W, const uint8_t *X, long wrow, long xrow, int row0, int row1, int npos, int ntok,
             float *y, const float *bias, long ldy, int32_t *sub, int nsub_row, int nrows, GemvGroup grp)
@@ -85,11 +86,28 @@ gemv_kernel(const uint8_t *W, const uint8_t *X, long wrow, long xrow, int row0, 
      * loads go out first, all at once (one round trip, they hit in L2), the
      * weight loads follow, and only then are the staged values written. */
     constexpr int XNT = 64 * WPB, XU = MT == 1 ? 2 : 4;
-    const uint8_t *xsrc = gX + (size_t)t0 * a.xrow;
-    const int xbytes = (int)((long)min(MT, a.ntok - t0) * a.xrow), xn = xbytes / F::XS_SRC;   /* staging units */
+    const int mt_live = min(MT, a.ntok - t0);
+    const uint8_t *xsrc = gX + (size_t)t0 * (XQ ? (size_t)a.npos * 256 : (size_t)a.xrow);   /* XQ: rows of fp32, 64 per position */
+    const int xbytes = (int)((long)mt_live * a.xrow), xn = xbytes / F::XS_SRC;   /* staging units */
     const u32 xcap = (u32)((long)MT * a.xrow / F::XS_SRC);                                     /* units of a full tile */
-    u32 xv[XU][F::XS_REGS];
-    if (LDSX) {
+    u32 xv[XQ ? 1 : XU][F::XS_REGS];
+    /* XQ: the tile's rows arrive as fp32 and are quantized to Q8_K here, one
+     * wave per 256-element block (blocks wave, wave+WPB, ... of the tile's
+     * contiguous rows), into the same LDS image the plain staging writes.
+     * This happens before the weight loads are issued, so that its registers
+     * are free again when the weights arrive; other resident blocks cover the
+     * round trip. */
+    if constexpr (XQ) {
+        const int qblocks = mt_live * (a.npos / 4);
+        for (int b = wave; b < qblocks; b += 2 * WPB) {
+            const bool two = b + WPB < qblocks;
+            const float4 v0 = reinterpret_cast<const float4 *>(xsrc + (size_t)b * 1024)[lane];
+            const float4 v1 = reinterpret_cast<const float4 *>(xsrc + (size_t)(two ? b + WPB : b) * 1024)[lane];
+            const float e0[4] = {v0.x, v0.y, v0.z, v0.w}, e1[4] = {v1.x, v1.y, v1.z, v1.w};
+            q8k_quantize_block(e0, lane, xs + (u32)b * 292u);
+            if (two) q8k_quantize_block(e1, lane, xs + (u32)(b + WPB) * 292u);
+        }
+    } else if (LDSX) {
 #pragma unroll
         for (int u = 0; u < XU; ++u) {
             const int i = u * XNT + (int)threadIdx.x;
@@ -121,7 +139,9 @@ gemv_kernel(const uint8_t *W, const uint8_t *X, long wrow, long xrow, int row0, 
                 F::load_w(w[r][p], wbase, orow);
             }
         }
-        if (LDSX && p0 == 0) {
+        if (XQ && p0 == 0) {
+            __syncthreads();
+        } else if (LDSX && p0 == 0) {
             /* the staged activations' loads are older than the weight loads
              * just issued, so waiting for them does not wait for the weights */
 #pragma unroll
@@ -236,7 +256,7 @@ static int launch_rows(const GemvArgs &a, const GemvGroup &grp) { return grp.n >
  * several launches over consecutive token ranges (ckq_grid_chunk). */
 constexpr int CKQ_GRID_Y_MAX = 65535;
 
-template <class F, int LPR, int PPL, int MT, int RPI, bool DUMP, int WPB, bool LDSX>
+template <class F, int LPR, int PPL, int MT, int RPI, bool DUMP, int WPB, bool LDSX, bool XQ = false>
 static int launch_one(const GemvArgs &a0, const GemvGroup &grp, hipStream_t s)
 {
     constexpr int rows_per_block = WPB * (64 / LPR) * RPI;
@@ -245,7 +265,7 @@ static int launch_one(const GemvArgs &a0, const GemvGroup &grp, hipStream_t s)
     if (grp.n > 1) {
         if constexpr (LDSX) {                            /* grouped launches stage their activations in LDS */
             dim3 grid((nr + rows_per_block - 1) / rows_per_block, (a0.ntok + MT - 1) / MT, (unsigned)grp.n);
-            hipLaunchKernelGGL((gemv_kernel<F, LPR, PPL, MT, RPI, DUMP, WPB, LDSX, true>), grid, dim3(64 * WPB), lds, s,
+            hipLaunchKernelGGL((gemv_kernel<F, LPR, PPL, MT, RPI, DUMP, WPB, LDSX, true, XQ>), grid, dim3(64 * WPB), lds, s,
                                a0.W, a0.X, a0.wrow, a0.xrow, a0.row0, a0.row1, a0.npos, a0.ntok, a0.y, a0.bias, a0.ldy, a0.sub,
                                a0.nsub_row, a0.nrows, grp);
             return (int)hipGetLastError();
@@ -258,11 +278,11 @@ static int launch_one(const GemvArgs &a0, const GemvGroup &grp, hipStream_t s)
         long first, count;
         ckq_grid_chunk(a0.ntok, per, c, &first, &count);
         GemvArgs a = a0;
-        a.X = a0.X + (size_t)first * (size_t)a0.xrow;
+        a.X = a0.X + (size_t)first * (XQ ? (size_t)a0.npos * 256 : (size_t)a0.xrow);
         a.y = a0.y ? a0.y + (size_t)first * (size_t)a0.ldy : nullptr;
         a.ntok = (int)count;
         dim3 grid((nr + rows_per_block - 1) / rows_per_block, (a.ntok + MT - 1) / MT, 1);
-        hipLaunchKernelGGL((gemv_kernel<F, LPR, PPL, MT, RPI, DUMP, WPB, LDSX>), grid, dim3(64 * WPB), lds, s,
+        hipLaunchKernelGGL((gemv_kernel<F, LPR, PPL, MT, RPI, DUMP, WPB, LDSX, false, XQ>), grid, dim3(64 * WPB), lds, s,
                            a.W, a.X, a.wrow, a.xrow, a.row0, a.row1, a.npos, a.ntok, a.y, a.bias, a.ldy, a.sub,
                            a.nsub_row, a.nrows, grp);
         const int rc = (int)hipGetLastError();
@@ -277,6 +297,12 @@ template <class F, int LPR, int PPL, int MT, int RPI, int WPB>
 static int launch_tile(const GemvArgs &a, const GemvGroup &grp, hipStream_t s)
 {
     const bool fits = F::xs_lds_bytes((size_t)MT * (size_t)a.xrow) <= 65536;
+    if (a.xq) {
+        if constexpr (F::XBLOCK == 292) {
+            if (fits && !a.sub) return launch_one<F, LPR, PPL, MT, RPI, false, WPB, true, true>(a, grp, s);
+        }
+        return CKQ_EINVAL;
+    }
     if (a.sub) {
         if constexpr (F::TOKEN_TILES) {
             if (fits) return launch_one<F, LPR, PPL, MT, RPI, true, WPB, true>(a, grp, s);

@@ -511,12 +511,13 @@ void ckq_set_parallel_whole(int enabled)
 /* Shapes                                                                    */
 /* ------------------------------------------------------------------------ */
 
-static int fmt_block_elems(int fmt) { return (fmt == CKQ_FMT_Q8_0 || fmt == CKQ_FMT_Q5_0 || fmt == CKQ_KERNEL_Q80_F32) ? 32 : 256; }
+static int fmt_block_elems(int fmt) { fmt &= ~CKQ_ACT_F32_QUANT; return (fmt == CKQ_FMT_Q8_0 || fmt == CKQ_FMT_Q5_0 || fmt == CKQ_KERNEL_Q80_F32) ? 32 : 256; }
 
 static int is_f32act(int fmt) { return fmt == CKQ_KERNEL_Q80_F32 || fmt == CKQ_KERNEL_Q4K_F32 || fmt == CKQ_KERNEL_Q6K_F32; }
 
 static int weight_fmt(int fmt)
 {
+    fmt &= ~CKQ_ACT_F32_QUANT;
     return fmt == CKQ_KERNEL_Q80_F32 ? CKQ_FMT_Q8_0 : fmt == CKQ_KERNEL_Q4K_F32 ? CKQ_FMT_Q4_K
          : fmt == CKQ_KERNEL_Q6K_F32 ? CKQ_FMT_Q6_K : fmt;
 }
@@ -528,7 +529,7 @@ static size_t weight_row_bytes(int fmt, int K)
 
 static size_t act_row_bytes(int fmt, int K)
 {
-    if (is_f32act(fmt)) return (size_t)K * 4;
+    if (is_f32act(fmt) || (fmt & CKQ_ACT_F32_QUANT)) return (size_t)K * 4;
     if (fmt == CKQ_FMT_Q8_0 || fmt == CKQ_FMT_Q5_0) return ckq_row_bytes(CKQ_FMT_Q8_0, K);
     return ckq_row_bytes(CKQ_FMT_Q8_K, K);
 }
@@ -1099,8 +1100,10 @@ int ckq_quantize_q8_0_dev(const float *x, void *y, int num_rows, int k, void *st
 int ckq_gemm_nt_dev(int fmt, const void *A_q8, const void *B, const float *bias, float *C,
                     int M, int N, int K, long ldc, void *stream)
 {
-    if (fmt != CKQ_FMT_Q4_K && fmt != CKQ_FMT_Q5_K && fmt != CKQ_FMT_Q6_K && fmt != CKQ_FMT_Q8_0 && fmt != CKQ_FMT_Q5_0)
+    const int wf = fmt & ~CKQ_ACT_F32_QUANT;
+    if (wf != CKQ_FMT_Q4_K && wf != CKQ_FMT_Q5_K && wf != CKQ_FMT_Q6_K && wf != CKQ_FMT_Q8_0 && wf != CKQ_FMT_Q5_0)
         return CKQ_EFORMAT;
+    if (fmt != wf && (wf == CKQ_FMT_Q8_0 || wf == CKQ_FMT_Q5_0)) return CKQ_EFORMAT;
     return ckq_launch_gemv(fmt, C, B, A_q8, bias, N, K, M, ldc, 0, N, NULL, stream);
 }
 

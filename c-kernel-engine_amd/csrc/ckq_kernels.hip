@@ -244,7 +244,7 @@ extern "C" int ckq_launch_gemv_group(int fmt, int n, float *const *y, const void
     /* Every grouped kernel stages its token tile in LDS.  A tile that does not
      * fit (the tile is the token count rounded up to 1, 2, 4 or 8 rows of
      * activations) goes out as n separate launches, which stream it instead. */
-    if (n == 1 || !group_tile_fits_lds(fmt, K, ntok)) {
+    if (n == 1 || !group_tile_fits_lds(fmt & ~CKQ_ACT_F32_QUANT, K, ntok)) {
         if (subdots) return CKQ_EINVAL;
         for (int i = 0; i < n; ++i) {
             const int rc = ckq_launch_gemv(fmt, y[i], W[i], X[i], bias ? bias[i] : nullptr, rows[i], K, ntok, ldys[i], 0,
@@ -268,8 +268,9 @@ extern "C" int ckq_launch_gemv_group(int fmt, int n, float *const *y, const void
     return launch_gemv_args(fmt, a, grp, K, stream);
 }
 
-static int launch_gemv_args(int fmt, GemvArgs &a, const GemvGroup &grp, int K, void *stream, const GemmOpts &opts)
+static int launch_gemv_args(int fmt_flags, GemvArgs &a, const GemvGroup &grp, int K, void *stream, const GemmOpts &opts)
 {
+    int fmt = fmt_flags;
     float *const y = a.y;
     const void *const W = a.W, *const X = a.X;
     const float *const bias = a.bias;
@@ -277,7 +278,12 @@ static int launch_gemv_args(int fmt, GemvArgs &a, const GemvGroup &grp, int K, v
     const long ldy = a.ldy;
     hipStream_t s = (hipStream_t)stream;
     const bool dump = a.sub != nullptr;
-    const bool whole = !dump && grp.n == 1 && row0 == 0 && row1 == nrows;   /* what a matrix-core GEMM can take */
+    const bool xq = (fmt & CKQ_ACT_F32_QUANT) != 0;
+    fmt &= ~CKQ_ACT_F32_QUANT;
+    if (xq && (dump || ntok > CKQ_STREAM_TOKENS || (fmt != CKQ_FMT_Q4_K && fmt != CKQ_FMT_Q5_K && fmt != CKQ_FMT_Q6_K)))
+        return CKQ_EINVAL;
+    a.xq = xq;
+    const bool whole = !xq && !dump && grp.n == 1 && row0 == 0 && row1 == nrows;   /* what a matrix-core GEMM can take */
     switch (fmt) {
     case CKQ_FMT_Q4_K:
         if (K % 256) return CKQ_ESHAPE;
@@ -410,21 +416,6 @@ extern "C" int ckq_launch_gemm_block_sums(int fmt, const void *A, const void *B,
 /* Activation quantizers                                                      */
 /* ========================================================================= */
 
-/* x86 cvtps2dq + saturating packs: round to nearest even, NaN -> -128. */
-__device__ __forceinline__ int rne_sat_i8(float p)
-{
-    if (p != p) return -128;
-    const float r = __builtin_rintf(p);
-    return (int)fminf(fmaxf(r, -128.0f), 127.0f);
-}
-
-/*
- * fp32 -> Q8_K, one wave per 256-element block, lane l owns elements
- * 4l..4l+3 (reference: quantize_row_q8_k_sse.c:22-82).  The scale comes from
- * the FIRST element with the largest magnitude, sign kept; iscale = -127/max
- * with IEEE division; each product is rounded to fp32 and then to the nearest
- * even integer; d = 1/iscale.
- */
 /* SiLU(g) * u as the reference's fused prefill MLP forms it
  * (fused/prefill_fused_gemm.c:904-906, 1034-1040): g / (1 + expf(-g)), then
  * the product, each operation rounded to fp32.  exp is evaluated in double
@@ -437,8 +428,10 @@ __device__ __forceinline__ float swiglu_value(float g, float u)
     return s * u;
 }
 
-/* SWIGLU: the quantizer's input is SiLU(x) * up instead of x.  Rows of the
- * input are ldx floats apart, bpr blocks of 256 per row. */
+/* fp32 -> Q8_K, one wave per 256-element block, lane l owns elements 4l..4l+3
+ * (q8k_quantize_block holds the reference's rules).  SWIGLU: the quantizer's
+ * input is SiLU(x) * up instead of x.  Rows of the input are ldx floats apart,
+ * bpr blocks of 256 per row. */
 template <bool SWIGLU>
 __global__ void __launch_bounds__(256) quantize_q8_k_kernel(const float *__restrict__ x, const float *__restrict__ up,
                                                             uint8_t *__restrict__ y, long nblocks, int bpr, long ldx)
@@ -455,40 +448,7 @@ __global__ void __launch_bounds__(256) quantize_q8_k_kernel(const float *__restr
         e[2] = swiglu_value(e[2], w.z); e[3] = swiglu_value(e[3], w.w);
     }
 
-    /* first-largest |x| inside the lane, then across lanes (lower index wins ties) */
-    float amax = 0.0f, smax = 0.0f;
-    int idx = 4 * lane;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const float ax = fabsf(e[i]);
-        if (ax > amax) { amax = ax; smax = e[i]; idx = 4 * lane + i; }
-    }
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const float oa = __shfl_xor(amax, off), os = __shfl_xor(smax, off);
-        const int   oi = __shfl_xor(idx, off);
-        if (oa > amax || (oa == amax && oi < idx)) { amax = oa; smax = os; idx = oi; }
-    }
-
-    uint8_t *out = y + blk * 292;
-    if (amax == 0.0f) {
-        /* 292 bytes of zeros: d, qs, bsums */
-        reinterpret_cast<u32 *>(out)[lane] = 0;
-        if (lane < 9) reinterpret_cast<u32 *>(out)[64 + lane] = 0;
-        return;
-    }
-    const float iscale = -127.0f / smax;
-    int q[4], s = 0;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        q[i] = rne_sat_i8(__fmul_rn(e[i], iscale));
-        s += q[i];
-    }
-    const u32 packed = (u32)(q[0] & 0xff) | ((u32)(q[1] & 0xff) << 8) | ((u32)(q[2] & 0xff) << 16) | ((u32)(q[3] & 0xff) << 24);
-    reinterpret_cast<u32 *>(out + 4)[lane] = packed;
-    s = group_sum<4>(s);                       /* 16 consecutive elements = 4 lanes */
-    if ((lane & 3) == 3) reinterpret_cast<int16_t *>(out + 260)[lane >> 2] = (int16_t)s;
-    if (lane == 0) *reinterpret_cast<float *>(out) = 1.0f / iscale;
+    q8k_quantize_block(e, lane, y + blk * 292);
 }
 
 /*

@@ -25,6 +25,13 @@ extern "C" {
 #define CKQ_KERNEL_Q80_F32 16
 #define CKQ_KERNEL_Q4K_F32 17
 #define CKQ_KERNEL_Q6K_F32 18
+/* Added to CKQ_FMT_Q4_K / _Q5_K / _Q6_K in the streaming launches (at most
+ * eight tokens): X is ntok contiguous rows of K floats that the kernel
+ * quantizes to Q8_K while it stages them, with the bits of
+ * ckq_launch_quantize_q8_k; CKQ_EINVAL when the tile does not fit in LDS. */
+#ifndef CKQ_ACT_F32_QUANT
+#define CKQ_ACT_F32_QUANT 0x100
+#endif
 
 /*
  * y[t*ldy + row] = dot(W[row], X[t]) (+ bias[row]) for row < nrows, t < ntok.

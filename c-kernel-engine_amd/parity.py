@@ -143,11 +143,20 @@ def dev_quantize(x_t, fmt="q8_k", rows=1):
     return out
 
 
+ACT_F32_QUANT = 0x100
+
+
+def fmt_tag(name):
+    """Weight-format tag; "<fmt>+f32q" adds CKQ_ACT_F32_QUANT (fp32 activations
+    quantized to Q8_K inside the consumer)."""
+    return FMT[name[:-5]] | ACT_F32_QUANT if name.endswith("+f32q") else FMT[name]
+
+
 def dev_gemm_nt(fmt, A_t, B_t, bias_t, M, N, K, out=None):
     """C[M,N] on the device; M = 1 is the GEMV."""
     import torch
     c = out if out is not None else torch.empty(M * N, dtype=torch.float32, device=B_t.device)
-    check(lib().ckq_gemm_nt_dev(FMT[fmt], _dp(A_t), _dp(B_t), _dp(bias_t), _dp(c), M, N, K, N, _stream()),
+    check(lib().ckq_gemm_nt_dev(fmt_tag(fmt), _dp(A_t), _dp(B_t), _dp(bias_t), _dp(c), M, N, K, N, _stream()),
           "ckq_gemm_nt_dev")
     return c.view(M, N)
 
@@ -251,6 +260,6 @@ def dev_matmul_sequence(ops, repeat=1):
                               None, C_t.data_ptr(), eps)
         else:
             fmt, A_t, B_t, bias_t, C_t, M, N, K = op
-            arr[i] = MatmulOp(FMT[fmt], M, N, K, N, A_t.data_ptr(), B_t.data_ptr(),
+            arr[i] = MatmulOp(fmt_tag(fmt), M, N, K, N, A_t.data_ptr(), B_t.data_ptr(),
                               bias_t.data_ptr() if bias_t is not None else None, C_t.data_ptr(), 0.0)
     check(lib().ckq_matmul_sequence_dev(ctypes.cast(arr, _vp), len(ops), repeat, _stream()), "ckq_matmul_sequence_dev")

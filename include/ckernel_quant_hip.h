@@ -218,7 +218,14 @@ int ckq_quantize_q8_0_dev(const float *x, void *y, int num_rows, int k, void *st
 
 /* Generic form: fmt is a ckq_format weight tag (activations Q8_0 for
  * CKQ_FMT_Q8_0, Q8_K otherwise).  C[m*ldc + n] = dot(B[n], A[m]) (+bias[n]),
- * m < M tokens, n < N rows.  M = 1 with ldc = N is the GEMV. */
+ * m < M tokens, n < N rows.  M = 1 with ldc = N is the GEMV.
+ * fmt | CKQ_ACT_F32_QUANT (CKQ_FMT_Q4_K, _Q5_K, _Q6_K; M <= 8): A_q8 is M
+ * contiguous rows of K floats (16-byte aligned) instead, which the kernel
+ * quantizes to Q8_K while it stages them - the bits of ckq_quantize_q8_k_dev
+ * followed by the plain call, one launch less; CKQ_EINVAL for more tokens or
+ * when the token tile (M rounded up to 1, 2, 4 or 8 rows of K/256 * 292
+ * bytes) exceeds the 64 KB of LDS a block stages it in. */
+#define CKQ_ACT_F32_QUANT 0x100
 int ckq_gemm_nt_dev(int fmt, const void *A_q8, const void *B, const float *bias, float *C,
                     int M, int N, int K, long ldc, void *stream);
 
@@ -289,7 +296,8 @@ int ckq_gemm_nt_f32act_dev(int fmt, const float *A, const void *B, const float *
  *                           apart (0 = K), gamma at B, epsilon in eps (rmsnorm_q8_k_fused)
  *   CKQ_STEP_SWIGLU_Q8_K    C = Q8_K(SiLU(gate) * up): gate at A_q8, up at B, M rows of K floats, rows
  *                           ldc floats apart (0 = K) (ckq_swiglu_q8_k_dev)
- * N and bias are unused by producer entries; C is the block buffer. */
+ * N and bias are unused by producer entries; C is the block buffer.  A matmul
+ * entry may carry CKQ_ACT_F32_QUANT as in ckq_gemm_nt_dev. */
 #define CKQ_STEP_QUANTIZE_Q8_K 32
 #define CKQ_STEP_QUANTIZE_Q8_0 33
 #define CKQ_STEP_RMSNORM_Q8_K  34

@@ -381,6 +381,60 @@ def test_sequence_with_producer_steps():
     assert T.norm_err(one["y"].cpu().numpy(), T.oracle_gemv("q6_k", Wd, one["hq"].cpu().numpy(), D, F)) <= TOL
 
 
+# ---- activations quantized inside the consumer -----------------------------------------------------------
+
+@pytest.mark.parametrize("fmt", ["q4_k", "q5_k", "q6_k"])
+def test_quantize_in_consumer_prologue(fmt):
+    """fmt | CKQ_ACT_F32_QUANT: the streaming kernel takes fp32 rows and quantizes
+    them to Q8_K while it stages them.  Its outputs have the bits of
+    ckq_quantize_q8_k_dev followed by the plain call, for every token tile and
+    lane mapping, with zero blocks, ties for the largest magnitude and a
+    partial last tile; the quantizer itself is bit-exact with the oracle
+    elsewhere.  More than eight tokens are refused."""
+    import torch
+    for (N, K), Ms in (((70, 256), (1, 3)), ((300, 1024), (1, 2)), ((129, 2048), (1, 5)), ((512, 4096), (1, 2, 4, 8)),
+                       ((96, 11008), (1, 2, 3)), ((9000, 512), (1,)), ((2100, 4096), (1,)), ((40, 14336), (1, 2))):
+        W = P.to_device(T.synth_weights(fmt, N, K, seed=N + K))
+        for M in Ms:
+            say(f"prologue quantizer {fmt} {N}x{K} M={M}")
+            x = T.normal(M * K, 0.0, 1.0, seed=3 * N + M)
+            x[:256] = 0.0                                  # an all-zero block
+            if K >= 512:
+                x[256:512] = np.where(np.arange(256) % 2 == 0, 0.75, -0.75)   # every element ties for the maximum
+            x_t = P.to_device(x)
+            want = P.dev_gemm_nt(fmt, P.dev_quantize(x_t, "q8_k", rows=M), W, None, M, N, K)
+            got = P.dev_gemm_nt(fmt + "+f32q", x_t, W, None, M, N, K)
+            torch.cuda.synchronize()
+            assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+    one = ctypes.c_void_p(256)
+    assert ckq.lib().ckq_gemm_nt_dev(P.fmt_tag(fmt + "+f32q"), one, one, None, one, 9, 64, 256, 64, None) == -1
+    # a tile of eight 11008-wide rows (100 KB of Q8_K blocks) does not fit in LDS
+    assert ckq.lib().ckq_gemm_nt_dev(P.fmt_tag(fmt + "+f32q"), one, one, None, one, 7, 64, 11008, 64, None) == -1
+    assert ckq.lib().ckq_gemm_nt_dev(P.FMT["q8_0"] | P.ACT_F32_QUANT, one, one, None, one, 1, 64, 256, 64, None) == -3
+
+
+def test_sequence_with_quantizing_consumers():
+    """Q/K/V and gate/up as grouped launches whose members quantize the shared
+    fp32 row themselves: the bits of the quantizer step followed by the plain
+    grouped launch."""
+    import torch
+    D, F, KV = 1024, 2816, 256
+    for M in (1, 3):
+        x = P.to_device(T.normal(M * D, 0.0, 1.0, 191 + M))
+        Ws = [P.to_device(T.synth_weights("q4_k", n, D, seed=194 + i)) for i, n in enumerate((D, KV, KV, F, F))]
+        rows = (D, KV, KV, F, F)
+        f32 = lambda n: torch.zeros(M * n, dtype=torch.float32, device="cuda")
+        a, b = [f32(n) for n in rows], [f32(n) for n in rows]
+        xq = torch.zeros(M * T.row_bytes("q8_k", D), dtype=torch.uint8, device="cuda")
+        say(f"grouped launches with quantizing consumers M={M}")
+        P.dev_matmul_sequence([("quantize_q8_k", x, None, xq, M, D)] +
+                              [("q4_k", xq, Ws[i], None, a[i], M, rows[i], D) for i in range(5)])
+        P.dev_matmul_sequence([("q4_k+f32q", x, Ws[i], None, b[i], M, rows[i], D) for i in range(5)])
+        torch.cuda.synchronize()
+        for i in range(5):
+            assert torch.equal(a[i], b[i]), i
+
+
 # ---- host-pointer paths with the weight cache off, long contexts ---------------------------------------
 
 def test_host_paths_with_weight_cache_off():
