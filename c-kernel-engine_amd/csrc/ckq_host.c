@@ -60,6 +60,18 @@ static int          g_cache_on = 1;
 static int          g_parallel_whole = CKQ_PARALLEL_WHOLE_DEFAULT;
 static hipStream_t  g_stream = NULL;
 static dev_buf      g_buf[BUF_COUNT];
+/* Pinned host twins of the staging buffers.  Small transfers (a decode step's
+ * activation vector up, its outputs down) go through them: a copy between
+ * pageable memory and the device makes the runtime stage and wait inside each
+ * hipMemcpyAsync, a copy from or to pinned memory is one enqueue.  Every
+ * host-pointer call ends in a stream synchronisation, so a twin is free again
+ * when the next call starts. */
+enum { PIN_MAX_BYTES = 1 << 20 };
+typedef struct {
+    void  *host;
+    size_t cap;
+} pin_buf;
+static pin_buf      g_pin[BUF_COUNT];
 static weight_entry *g_w = NULL;
 static size_t       g_nw = 0, g_capw = 0;
 static size_t       g_cache_max_bytes = (size_t)64 << 30;   /* bound on unpinned resident weights */
@@ -203,8 +215,27 @@ static int buf_reserve(int which, size_t bytes, void **out)
     return 0;
 }
 
+/* Pinned twin of staging buffer `which`, at least `bytes` large (bytes <=
+ * PIN_MAX_BYTES).  Nothing is in flight on a twin when this is called. */
+static int pin_reserve(int which, size_t bytes, void **out)
+{
+    pin_buf *b = &g_pin[which];
+    if (b->cap < bytes) {
+        if (b->host) {
+            HIP_TRY(hipHostFree(b->host));
+            b->host = NULL;
+            b->cap = 0;
+        }
+        size_t cap = bytes < 65536 ? 65536 : bytes + bytes / 4;
+        HIP_TRY(hipHostMalloc(&b->host, cap, hipHostMallocDefault));
+        b->cap = cap;
+    }
+    *out = b->host;
+    return 0;
+}
+
 /* Device view of an input: device pointers pass through, host memory is
- * copied into staging buffer `which`. */
+ * copied into staging buffer `which` (small inputs by way of its pinned twin). */
 static int stage_in(int which, const void *p, size_t bytes, const void **out)
 {
     if (is_device_ptr(p)) {
@@ -214,8 +245,42 @@ static int stage_in(int which, const void *p, size_t bytes, const void **out)
     void *d = NULL;
     int rc = buf_reserve(which, bytes, &d);
     if (rc) return rc;
-    HIP_TRY(hipMemcpyAsync(d, p, bytes, hipMemcpyHostToDevice, g_stream));
+    const void *src = p;
+    if (bytes <= PIN_MAX_BYTES) {
+        void *h = NULL;
+        rc = pin_reserve(which, bytes, &h);
+        if (rc) return rc;
+        memcpy(h, p, bytes);
+        src = h;
+    }
+    HIP_TRY(hipMemcpyAsync(d, src, bytes, hipMemcpyHostToDevice, g_stream));
     *out = d;
+    return 0;
+}
+
+/* The contents of staging buffer `which` back to the host and the stream
+ * drained: `rows` rows of `w` bytes, `src_pitch` apart on the device,
+ * `dst_pitch` apart at `dst`.  Small results come down in one copy into the
+ * pinned twin and are scattered by the CPU after the synchronisation. */
+static int stage_out_sync(int which, void *dst, size_t dst_pitch, size_t src_pitch, size_t w, size_t rows)
+{
+    const uint8_t *dev = (const uint8_t *)g_buf[which].dev;
+    const size_t span = rows ? (rows - 1) * src_pitch + w : 0;
+    if (span && span <= PIN_MAX_BYTES) {
+        void *h = NULL;
+        int rc = pin_reserve(which, span, &h);
+        if (rc) return rc;
+        HIP_TRY(hipMemcpyAsync(h, dev, span, hipMemcpyDeviceToHost, g_stream));
+        HIP_TRY(hipStreamSynchronize(g_stream));
+        for (size_t r = 0; r < rows; ++r) memcpy((uint8_t *)dst + r * dst_pitch, (const uint8_t *)h + r * src_pitch, w);
+        return 0;
+    }
+    if (rows == 1 || (dst_pitch == w && src_pitch == w)) {
+        HIP_TRY(hipMemcpyAsync(dst, dev, rows * w, hipMemcpyDeviceToHost, g_stream));
+    } else {
+        HIP_TRY(hipMemcpy2DAsync(dst, dst_pitch, dev, src_pitch, w, rows, hipMemcpyDeviceToHost, g_stream));
+    }
+    HIP_TRY(hipStreamSynchronize(g_stream));
     return 0;
 }
 
@@ -564,20 +629,12 @@ static void matmul_locked(int fmt, const void *A, const void *B, const float *bi
         int rc = ckq_launch_gemv(fmt, dC, dB, dA, (const float *)dbias, nrows, K, ntok, ld, row0, row1, NULL, g_stream);
         if (rc) { fail(rc, "ckq_launch_gemv"); break; }
         if (!c_on_dev) {
-            hipError_t e = hipSuccess;
-            const size_t w = (size_t)(row1 - row0) * sizeof(float);
-            if (ldc == ld || ntok == 1) {
-                for (int t = 0; t < ntok && e == hipSuccess; ++t)
-                    e = hipMemcpyAsync(C + (size_t)t * ldc + row0, (float *)g_buf[BUF_Y].dev + (size_t)t * ld, w,
-                                       hipMemcpyDeviceToHost, g_stream);
-            } else {
-                e = hipMemcpy2DAsync(C + row0, (size_t)ldc * sizeof(float), g_buf[BUF_Y].dev, (size_t)ld * sizeof(float),
-                                     w, (size_t)ntok, hipMemcpyDeviceToHost, g_stream);
-            }
-            if (e != hipSuccess) { fail((int)e, "copy result to host"); break; }
+            if (stage_out_sync(BUF_Y, C + row0, (size_t)ldc * sizeof(float), (size_t)ld * sizeof(float),
+                               (size_t)(row1 - row0) * sizeof(float), (size_t)ntok)) break;
+        } else {
+            hipError_t e = hipStreamSynchronize(g_stream);
+            if (e != hipSuccess) { fail((int)e, "hipStreamSynchronize"); break; }
         }
-        hipError_t e = hipStreamSynchronize(g_stream);
-        if (e != hipSuccess) fail((int)e, "hipStreamSynchronize");
         done = 1;
     } while (0);
     if (!done) drain_after_error();
@@ -641,11 +698,11 @@ static void host_quantize(int q8k, const float *x, void *y, int rows, int k)
                      : ckq_launch_quantize_q8_0((const float *)dx, dy, rows, k, g_stream);
         if (rc) { fail(rc, "quantize launch"); break; }
         if (!y_on_dev) {
-            hipError_t e = hipMemcpyAsync(y, dy, out_bytes, hipMemcpyDeviceToHost, g_stream);
-            if (e != hipSuccess) { fail((int)e, "copy result to host"); break; }
+            if (stage_out_sync(BUF_Y, y, out_bytes, out_bytes, out_bytes, 1)) break;
+        } else {
+            hipError_t e = hipStreamSynchronize(g_stream);
+            if (e != hipSuccess) { fail((int)e, "hipStreamSynchronize"); break; }
         }
-        hipError_t e = hipStreamSynchronize(g_stream);
-        if (e != hipSuccess) fail((int)e, "hipStreamSynchronize");
         done = 1;
     } while (0);
     if (!done) drain_after_error();
@@ -820,11 +877,11 @@ static void host_dequant_rows(int fmt, const void *table, size_t table_rows, con
                                          (float *)dout, n_valid, n_row, tokens, n_out_rows, g_stream);
         if (rc) { fail(rc, "ckq_launch_dequant_rows"); break; }
         if (!on_dev) {
-            hipError_t e = hipMemcpyAsync(out, dout, out_bytes, hipMemcpyDeviceToHost, g_stream);
-            if (e != hipSuccess) { fail((int)e, "copy result to host"); break; }
+            if (stage_out_sync(BUF_Y, out, out_bytes, out_bytes, out_bytes, 1)) break;
+        } else {
+            hipError_t e = hipStreamSynchronize(g_stream);
+            if (e != hipSuccess) { fail((int)e, "hipStreamSynchronize"); break; }
         }
-        hipError_t e = hipStreamSynchronize(g_stream);
-        if (e != hipSuccess) fail((int)e, "hipStreamSynchronize");
         done = 1;
     } while (0);
     if (!done) drain_after_error();
@@ -885,11 +942,11 @@ void rmsnorm_q8_k_fused(const float *input, const float *gamma, void *vy, int to
                                                aligned_embed_dim, eps, g_stream);
         if (rc) { fail(rc, "rmsnorm_q8_k_fused launch"); break; }
         if (!y_on_dev) {
-            hipError_t e = hipMemcpyAsync(vy, dy, out_bytes, hipMemcpyDeviceToHost, g_stream);
-            if (e != hipSuccess) { fail((int)e, "copy result to host"); break; }
+            if (stage_out_sync(BUF_Y, vy, out_bytes, out_bytes, out_bytes, 1)) break;
+        } else {
+            hipError_t e = hipStreamSynchronize(g_stream);
+            if (e != hipSuccess) { fail((int)e, "hipStreamSynchronize"); break; }
         }
-        hipError_t e = hipStreamSynchronize(g_stream);
-        if (e != hipSuccess) fail((int)e, "hipStreamSynchronize");
         done = 1;
     } while (0);
     if (!done) drain_after_error();
@@ -961,11 +1018,11 @@ void fused_mlp_swiglu_prefill_w1w2_quant(const float *x, const void *W1, const f
         rc = ckq_launch_gemv(fmt2, (float *)dout, dW2, dh, (const float *)dB2, E, I, seq_len, (long)E, 0, E, NULL, g_stream);
         if (rc) { fail(rc, "down GEMM launch"); break; }
         if (!out_on_dev) {
-            hipError_t e = hipMemcpyAsync(output, dout, out_bytes, hipMemcpyDeviceToHost, g_stream);
-            if (e != hipSuccess) { fail((int)e, "copy result to host"); break; }
+            if (stage_out_sync(BUF_Y, output, out_bytes, out_bytes, out_bytes, 1)) break;
+        } else {
+            hipError_t e = hipStreamSynchronize(g_stream);
+            if (e != hipSuccess) { fail((int)e, "hipStreamSynchronize"); break; }
         }
-        hipError_t e = hipStreamSynchronize(g_stream);
-        if (e != hipSuccess) fail((int)e, "hipStreamSynchronize");
         done = 1;
     } while (0);
     if (!done) drain_after_error();
