@@ -18,6 +18,7 @@
 #include <pthread.h>
 #include <stdlib.h>
 #include <string.h>
+#include <time.h>
 
 /* ------------------------------------------------------------------------ */
 /* fp16                                                                      */
@@ -972,6 +973,58 @@ void orc_gemv_threads(int fmt, float *y, const void *W, const void *x_q8, int M,
     }
     thr_main(&arg[0]);
     for (int t = 1; t < nth; ++t) pthread_join(tid[t], NULL);
+}
+
+/* Timing harness for the CPU baseline: `nth` persistent threads (the caller is
+ * thread 0) run fn(y, W, x, M, K, ith, nth) `iters` times, every round between
+ * two barriers, as the reference's thread pool runs a split GEMV
+ * (src/ck_threadpool.c:289-349: wake the workers, every thread takes its `ith`,
+ * barrier).  seconds[i] is the wall time of round i as thread 0 sees it.  The
+ * kernel is the caller's: the compiled reference's *_parallel_simd entry point,
+ * or this file's restatement. */
+typedef struct {
+    orc_split_gemv_fn fn;
+    float *y;
+    const void *W, *x;
+    int M, K, ith, nth, iters;
+    pthread_barrier_t *bar;
+} time_arg;
+
+static void *time_main(void *p)
+{
+    time_arg *a = (time_arg *)p;
+    for (int i = 0; i < a->iters; ++i) {
+        pthread_barrier_wait(a->bar);
+        a->fn(a->y, a->W, a->x, a->M, a->K, a->ith, a->nth);
+        pthread_barrier_wait(a->bar);
+    }
+    return NULL;
+}
+
+int orc_time_split_gemv(orc_split_gemv_fn fn, float *y, const void *W, const void *x_q8, int M, int K, int nth, int iters,
+                        double *seconds)
+{
+    if (!fn || !y || !W || !x_q8 || !seconds || M <= 0 || K <= 0 || nth < 1 || nth > 256 || iters < 1) return -1;
+    pthread_barrier_t bar;
+    if (pthread_barrier_init(&bar, NULL, (unsigned)nth)) return -1;
+    pthread_t tid[256];
+    time_arg  arg[256];
+    for (int t = 1; t < nth; ++t) {
+        arg[t] = (time_arg){fn, y, W, x_q8, M, K, t, nth, iters, &bar};
+        if (pthread_create(&tid[t], NULL, time_main, &arg[t])) return -1;   /* a thread short: the barrier would never open */
+    }
+    for (int i = 0; i < iters; ++i) {
+        struct timespec t0, t1;
+        pthread_barrier_wait(&bar);
+        clock_gettime(CLOCK_MONOTONIC, &t0);
+        fn(y, W, x_q8, M, K, 0, nth);
+        pthread_barrier_wait(&bar);
+        clock_gettime(CLOCK_MONOTONIC, &t1);
+        seconds[i] = (double)(t1.tv_sec - t0.tv_sec) + 1e-9 * (double)(t1.tv_nsec - t0.tv_nsec);
+    }
+    for (int t = 1; t < nth; ++t) pthread_join(tid[t], NULL);
+    pthread_barrier_destroy(&bar);
+    return 0;
 }
 
 /* fp32-activation GEMMs: a token loop over the GEMV, then the bias

@@ -57,6 +57,10 @@ void orc_subdots_q8_0_q8_0(const void *w_row, const void *x_q8, int K, int32_t *
 
 /* ---- GEMV: y[M] = W[M x K] . x ----------------------------------------- */
 void orc_gemv_q4_k_q8_k(float *y, const void *W, const void *x_q8, int M, int K);      /* gemm_kernels_q4k_q8k.c:121-200 */
+/* CPU-baseline timing: persistent threads, one barrier-bracketed round per call of a split GEMV. */
+typedef void (*orc_split_gemv_fn)(float *y, const void *W, const void *x_q8, int M, int K, int ith, int nth);
+int orc_time_split_gemv(orc_split_gemv_fn fn, float *y, const void *W, const void *x_q8, int M, int K, int nth, int iters,
+                        double *seconds);
 void orc_gemv_q4_k_q8_k_parallel(float *y, const void *W, const void *x_q8, int M, int K, int ith, int nth); /* :212-243 */
 void orc_gemv_q5_k_q8_k(float *y, const void *W, const void *x_q8, int M, int K);      /* gemm_kernels_q5_k.c:130-208,305-329 */
 void orc_gemv_q5_k(float *y, const void *W, const float *x, int M, int K);             /* gemm_kernels_q5_k.c:369-391 (K%256==0 branch) */
