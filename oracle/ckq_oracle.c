@@ -983,20 +983,32 @@ void orc_gemv_threads(int fmt, float *y, const void *W, const void *x_q8, int M,
  * kernel is the caller's: the compiled reference's *_parallel_simd entry point,
  * or this file's restatement. */
 typedef struct {
+    pthread_mutex_t   mu;
+    pthread_cond_t    cv;
+    int               go;      /* 0 wait, 1 run, -1 give up (a thread could not be created) */
+    pthread_barrier_t bar;
+} time_gate;
+
+typedef struct {
     orc_split_gemv_fn fn;
     float *y;
     const void *W, *x;
     int M, K, ith, nth, iters;
-    pthread_barrier_t *bar;
+    time_gate *gate;
 } time_arg;
 
 static void *time_main(void *p)
 {
     time_arg *a = (time_arg *)p;
+    pthread_mutex_lock(&a->gate->mu);
+    while (a->gate->go == 0) pthread_cond_wait(&a->gate->cv, &a->gate->mu);
+    const int go = a->gate->go;
+    pthread_mutex_unlock(&a->gate->mu);
+    if (go < 0) return NULL;
     for (int i = 0; i < a->iters; ++i) {
-        pthread_barrier_wait(a->bar);
+        pthread_barrier_wait(&a->gate->bar);
         a->fn(a->y, a->W, a->x, a->M, a->K, a->ith, a->nth);
-        pthread_barrier_wait(a->bar);
+        pthread_barrier_wait(&a->gate->bar);
     }
     return NULL;
 }
@@ -1005,26 +1017,37 @@ int orc_time_split_gemv(orc_split_gemv_fn fn, float *y, const void *W, const voi
                         double *seconds)
 {
     if (!fn || !y || !W || !x_q8 || !seconds || M <= 0 || K <= 0 || nth < 1 || nth > 256 || iters < 1) return -1;
-    pthread_barrier_t bar;
-    if (pthread_barrier_init(&bar, NULL, (unsigned)nth)) return -1;
+    time_gate gate;
+    if (pthread_barrier_init(&gate.bar, NULL, (unsigned)nth)) return -1;
+    pthread_mutex_init(&gate.mu, NULL);
+    pthread_cond_init(&gate.cv, NULL);
+    gate.go = 0;
     pthread_t tid[256];
     time_arg  arg[256];
-    for (int t = 1; t < nth; ++t) {
-        arg[t] = (time_arg){fn, y, W, x_q8, M, K, t, nth, iters, &bar};
-        if (pthread_create(&tid[t], NULL, time_main, &arg[t])) return -1;   /* a thread short: the barrier would never open */
+    int made = 1;
+    for (; made < nth; ++made) {
+        arg[made] = (time_arg){fn, y, W, x_q8, M, K, made, nth, iters, &gate};
+        if (pthread_create(&tid[made], NULL, time_main, &arg[made])) break;
     }
-    for (int i = 0; i < iters; ++i) {
+    const int ok = made == nth;      /* a thread short: the barrier would never open, so nobody enters it */
+    pthread_mutex_lock(&gate.mu);
+    gate.go = ok ? 1 : -1;
+    pthread_cond_broadcast(&gate.cv);
+    pthread_mutex_unlock(&gate.mu);
+    for (int i = 0; ok && i < iters; ++i) {
         struct timespec t0, t1;
-        pthread_barrier_wait(&bar);
+        pthread_barrier_wait(&gate.bar);
         clock_gettime(CLOCK_MONOTONIC, &t0);
         fn(y, W, x_q8, M, K, 0, nth);
-        pthread_barrier_wait(&bar);
+        pthread_barrier_wait(&gate.bar);
         clock_gettime(CLOCK_MONOTONIC, &t1);
         seconds[i] = (double)(t1.tv_sec - t0.tv_sec) + 1e-9 * (double)(t1.tv_nsec - t0.tv_nsec);
     }
-    for (int t = 1; t < nth; ++t) pthread_join(tid[t], NULL);
-    pthread_barrier_destroy(&bar);
-    return 0;
+    for (int t = 1; t < made; ++t) pthread_join(tid[t], NULL);
+    pthread_barrier_destroy(&gate.bar);
+    pthread_cond_destroy(&gate.cv);
+    pthread_mutex_destroy(&gate.mu);
+    return ok ? 0 : -1;
 }
 
 /* fp32-activation GEMMs: a token loop over the GEMV, then the bias

@@ -490,3 +490,24 @@ def test_encoders_round_trip():
     out = np.zeros(T.row_bytes("q4_k", len(w)), np.uint8)
     S.ckq_synth_quantize(T.FMT["q4_k"], ptr(w), ptr(out), ctypes.c_size_t(len(w)))
     assert np.all(T.np_decode_q4_k(out)["dmin"] > 0)
+
+
+def test_cpu_timing_harness_computes_what_it_times():
+    """The CPU-baseline harness (persistent threads, one barrier-bracketed round
+    per call) runs the split kernel it is handed: the output of its rounds is the
+    serial GEMV's, every round is timed, bad arguments are refused."""
+    import ctypes
+    M, K, nth, iters = 203, 512, 3, 4
+    W = T.synth_weights("q4_k", M, K, seed=77)
+    xq = T.oracle_quantize(T.normal(K, seed=78), "q8_k")
+    orc = T.oracle()
+    orc.orc_time_split_gemv.restype = ctypes.c_int
+    orc.orc_time_split_gemv.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 4 + [ctypes.c_void_p]
+    fn = ctypes.cast(orc.orc_gemv_q4_k_q8_k_parallel, ctypes.c_void_p)
+    y = np.full(M, np.nan, np.float32)
+    sec = np.zeros(iters, np.float64)
+    assert orc.orc_time_split_gemv(fn, T.ptr(y), T.ptr(W), T.ptr(xq), M, K, nth, iters, T.ptr(sec)) == 0
+    assert np.array_equal(y, T.oracle_gemv("q4_k", W, xq, M, K))
+    assert np.all(sec > 0)
+    assert orc.orc_time_split_gemv(fn, T.ptr(y), T.ptr(W), T.ptr(xq), M, K, 0, iters, T.ptr(sec)) == -1
+    assert orc.orc_time_split_gemv(None, T.ptr(y), T.ptr(W), T.ptr(xq), M, K, nth, iters, T.ptr(sec)) == -1
