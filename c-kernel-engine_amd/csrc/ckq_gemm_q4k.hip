@@ -242,22 +242,26 @@ __global__ void __launch_bounds__(256 * KG, KG == 2 ? 1 : WPE) gemm_q4k_mfma_ker
     /* copies of block b into stage buf: the side loads (into registers) first,
      * then nine global->LDS instructions that copy_one(i) issues one at a
      * time so they can be spread over the MFMA steps */
-    const uint8_t *cp_w = wbase, *cp_x = xbase;
+    /* the copies address their source as buffer (uniform base in SGPRs) + per-lane
+     * 32-bit offset + uniform K offset: no address arithmetic in the loop */
+    const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc((void *)wbase, 0, 0x7fffffff, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rs_x = __builtin_amdgcn_make_buffer_rsrc((void *)xbase, 0, 0x7fffffff, 0x00020000);
+    int cp_w = 0, cp_x = 0;
     int cp_buf = 0;
     auto copy_begin = [&](int b, int buf) {
         ld8<4>(nbs, st_src + (u32)b * 292u + 260 + 8 * st_q);
         nd = __builtin_bit_cast(float, ld4<4>(st_src + (u32)b * 292u));
-        cp_w = wbase + (u32)b * 144u;
-        cp_x = xbase + (u32)b * 292u;
+        cp_w = b * 144;
+        cp_x = b * 292;
         cp_buf = buf;
     };
     auto copy_one = [&](int i) {
         if (i < NWI)      /* weight slots past 17 repeat slot 17: same bytes, no branch */
-            __builtin_amdgcn_global_load_lds((ckq_glb_void *)(cp_w + wofs_g[i]),
-                                             (ckq_lds_void *)(stage[cp_buf].w + 1024 * min(wave + 4 * i, 17)), 16, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (ckq_lds_void *)(stage[cp_buf].w + 1024 * min(wave + 4 * i, 17)), 16,
+                                                     (int)wofs_g[i], cp_w, 0, 0);
         else
-            __builtin_amdgcn_global_load_lds((ckq_glb_void *)(cp_x + qofs_g[i - NWI]),
-                                             (ckq_lds_void *)(stage[cp_buf].q + 1024 * (wave + 4 * (i - NWI))), 16, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, (ckq_lds_void *)(stage[cp_buf].q + 1024 * (wave + 4 * (i - NWI))), 16,
+                                                     (int)qofs_g[i - NWI], cp_x, 0, 0);
     };
     static_assert(NWI + NQI == 9, "the pipelined block issues nine copies");
     auto side_store = [&](int buf) {

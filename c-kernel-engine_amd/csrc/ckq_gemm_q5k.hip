@@ -221,25 +221,27 @@ __global__ void __launch_bounds__(256, 1) gemm_q5k_mfma_kernel(GemmArgs a)
         bofs_g = (u32)min(e >> 1, a.M - 1 - t0) * xstride + 260u + 16u * (u32)(e & 1);
     }
 
-    const uint8_t *cp_w = wbase, *cp_x = xbase;
+    /* the copies address their source as buffer (uniform base in SGPRs) + per-lane
+     * 32-bit offset + uniform K offset: no address arithmetic in the loop */
+    const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc((void *)wbase, 0, 0x7fffffff, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rs_x = __builtin_amdgcn_make_buffer_rsrc((void *)xbase, 0, 0x7fffffff, 0x00020000);
+    int cp_w = 0, cp_x = 0;
     int cp_buf = 0;
     auto copy_begin = [&](int b, int buf) {
-        cp_w = wbase + (u32)b * 176u;
-        cp_x = xbase + (u32)b * 292u;
+        cp_w = b * 176;
+        cp_x = b * 292;
         cp_buf = buf;
     };
     auto copy_one = [&](int i) {
         if (i < NWI)
-            __builtin_amdgcn_global_load_lds((ckq_glb_void *)(cp_w + wofs_g[i]),
-                                             (ckq_lds_void *)(stage[cp_buf].w + 1024 * min(wave + 4 * i, 21)), 16, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (ckq_lds_void *)(stage[cp_buf].w + 1024 * min(wave + 4 * i, 21)), 16, (int)(wofs_g[i]), cp_w, 0, 0);
         else if (i < NWI + NQI)
-            __builtin_amdgcn_global_load_lds((ckq_glb_void *)(cp_x + qofs_g[i - NWI]),
-                                             (ckq_lds_void *)(stage[cp_buf].q + 1024 * (wave + 4 * (i - NWI))), 16, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, (ckq_lds_void *)(stage[cp_buf].q + 1024 * (wave + 4 * (i - NWI))), 16,
+                                                     (int)qofs_g[i - NWI], cp_x, 0, 0);
         else if (i == NWI + NQI)
-            __builtin_amdgcn_global_load_lds((ckq_glb_void *)(cp_x + dofs_g), (ckq_lds_void *)(stage[cp_buf].d), 4, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, (ckq_lds_void *)(stage[cp_buf].d), 4, (int)(dofs_g), cp_x, 0, 0);
         else
-            __builtin_amdgcn_global_load_lds((ckq_glb_void *)(cp_x + bofs_g),
-                                             (ckq_lds_void *)(stage[cp_buf].b + 1024 * (wave & 1)), 16, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, (ckq_lds_void *)(stage[cp_buf].b + 1024 * (wave & 1)), 16, (int)(bofs_g), cp_x, 0, 0);
     };
 
     /* read-side offsets of this lane */

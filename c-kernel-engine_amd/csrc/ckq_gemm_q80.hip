@@ -107,11 +107,14 @@ __global__ void __launch_bounds__(256, 2) gemm_q80_mfma_kernel(GemmArgs a)
         xd_g[0] = (u32)min(e & 63, a.M - 1 - t0) * stride;
     }
 
-    const uint8_t *cp_w = wbase, *cp_x = xbase;
+    /* the copies address their source as buffer (uniform base in SGPRs) + per-lane
+     * 32-bit offset + uniform K offset */
+    const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc((void *)wbase, 0, 0x7fffffff, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rs_x = __builtin_amdgcn_make_buffer_rsrc((void *)xbase, 0, 0x7fffffff, 0x00020000);
+    int cp_k = 0;
     int cp_buf = 0, cp_valid = KB;
     auto copy_begin = [&](int it, int buf) {
-        cp_w = wbase + (u32)it * (KB * 34u);
-        cp_x = xbase + (u32)it * (KB * 34u);
+        cp_k = it * (KB * 34);
         cp_valid = min(KB, nblk - it * KB);
         cp_buf = buf;
     };
@@ -119,17 +122,17 @@ __global__ void __launch_bounds__(256, 2) gemm_q80_mfma_kernel(GemmArgs a)
     auto blk_ofs = [&](u32 j) { return ((int)j < cp_valid ? j : 0u) * 34u; };
     auto copy_one = [&](int i) {
         if (i < NWQ)
-            __builtin_amdgcn_global_load_lds((ckq_glb_void *)(cp_w + (wq_g[i] + blk_ofs(wq_blk[i]))),
-                                             (ckq_lds_void *)(stage[cp_buf].wq + 1024 * (wave + 4 * i)), 16, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (ckq_lds_void *)(stage[cp_buf].wq + 1024 * (wave + 4 * i)), 16,
+                                                     (int)(wq_g[i] + blk_ofs(wq_blk[i])), cp_k, 0, 0);
         else if (i < NWQ + NXQ)
-            __builtin_amdgcn_global_load_lds((ckq_glb_void *)(cp_x + (xq_g[i - NWQ] + blk_ofs(xq_blk[i - NWQ]))),
-                                             (ckq_lds_void *)(stage[cp_buf].xq + 1024 * (wave + 4 * (i - NWQ))), 16, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, (ckq_lds_void *)(stage[cp_buf].xq + 1024 * (wave + 4 * (i - NWQ))), 16,
+                                                     (int)(xq_g[i - NWQ] + blk_ofs(xq_blk[i - NWQ])), cp_k, 0, 0);
         else if (i < NWQ + NXQ + NWD)   /* 2-byte loads land zero-extended, one dword per lane */
-            __builtin_amdgcn_global_load_lds((ckq_glb_void *)(cp_w + (wd_g[i - NWQ - NXQ] + blk_ofs(wd_blk[i - NWQ - NXQ]))),
-                                             (ckq_lds_void *)(stage[cp_buf].wd + 64 * (wave + 4 * (i - NWQ - NXQ))), 2, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (ckq_lds_void *)(stage[cp_buf].wd + 64 * (wave + 4 * (i - NWQ - NXQ))), 2,
+                                                     (int)(wd_g[i - NWQ - NXQ] + blk_ofs(wd_blk[i - NWQ - NXQ])), cp_k, 0, 0);
         else
-            __builtin_amdgcn_global_load_lds((ckq_glb_void *)(cp_x + (xd_g[0] + blk_ofs(xd_blk[0]))),
-                                             (ckq_lds_void *)(stage[cp_buf].xd + 64 * wave), 2, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, (ckq_lds_void *)(stage[cp_buf].xd + 64 * wave), 2,
+                                                     (int)(xd_g[0] + blk_ofs(xd_blk[0])), cp_k, 0, 0);
     };
 
     /* read-side offsets of this lane */
