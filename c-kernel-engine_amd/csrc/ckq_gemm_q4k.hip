@@ -38,6 +38,7 @@
  * each see a weight tile once.
  */
 #include "ckq_gemm_common.cuh"
+#include <type_traits>
 
 #ifndef CKQ_GEMM_WPE
 #define CKQ_GEMM_WPE 2          /* waves per SIMD the register budget is sized for */
@@ -50,8 +51,12 @@ __device__ __forceinline__ int mul_bytes(u32 v, u32 s16x2)
     return __builtin_bit_cast(int, (ckq_v2u16)(a * b));
 }
 
-/* small non-negative / signed integer (|v| < 2^8 significant bits) -> bf16 bits */
-__device__ __forceinline__ u32 bf16_bits(float f) { return __builtin_bit_cast(u32, f) >> 16; }
+/* two floats whose low 16 bits are zero (integers of at most 8 significant
+ * bits) -> their bf16 forms in one dword, lo in the low half: one v_perm_b32 */
+__device__ __forceinline__ u32 bf16_pair(float lo, float hi)
+{
+    return __builtin_amdgcn_perm(__builtin_bit_cast(u32, hi), __builtin_bit_cast(u32, lo), 0x07060302u);
+}
 
 constexpr int GEMM_BM = 64;     /* tokens per tile */
 constexpr int GEMM_BN = GEMM_TILE_ROWS;    /* weight rows per tile */
@@ -94,12 +99,17 @@ __device__ __forceinline__ void gemm_block_pipe(const GemmStage &st, u32 wofs, c
     const u32 sc47 = (h3 & 0x0f0f0f0fu) | (((h1 >> 6) & 0x03030303u) << 4);
     const float dw = h2f(h0 & 0xffff), dmin = h2f(h0 >> 16);
 
+    /* the two 3-bit halves of the eight scales, four per word; byte k of a word
+     * becomes the u16 pair {k-th, k-th} a plane is multiplied by with one v_perm_b32
+     * (selector 0x0c yields a zero byte) */
+    const u32 schi03 = (sc03 >> 3) & 0x07070707u, sclo03 = sc03 & 0x07070707u;
+    const u32 schi47 = (sc47 >> 3) & 0x07070707u, sclo47 = sc47 & 0x07070707u;
+    auto pair_of_byte = [](u32 w, int k) { return __builtin_amdgcn_perm(0u, w, 0x0c000c00u | (u32)k | ((u32)k << 16)); };
+
     ckq_v4i bH[8], bL[8];
     auto decode = [&](int j) {
         const int g = j >> 1, hi = j & 1;
-        const u32 scw = j < 4 ? sc03 : sc47;
-        const u32 sc = (scw >> (8 * (j & 3))) & 0xff;
-        const u32 mh = (sc >> 3) * 0x00010001u, ml = (sc & 7) * 0x00010001u;
+        const u32 mh = pair_of_byte(j < 4 ? schi03 : schi47, j & 3), ml = pair_of_byte(j < 4 ? sclo03 : sclo47, j & 3);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const u32 v = (u32)qv[g][i];
@@ -161,7 +171,7 @@ __device__ __forceinline__ void gemm_block_pipe(const GemmStage &st, u32 wofs, c
             for (int i = 0; i < 4; ++i) {
                 const u32 src = i < 2 ? mn03 : mn47;
                 const u32 m0 = (src >> (16 * (i & 1))) & 0xff, m1 = (src >> (16 * (i & 1) + 8)) & 0xff;
-                m[i] = bf16_bits((float)m0) | (bf16_bits((float)m1) << 16);
+                m[i] = bf16_pair((float)m0, (float)m1);
             }
             const ckq_v4i t = {(int)m[0], (int)m[1], (int)m[2], (int)m[3]};
             bm = __builtin_bit_cast(ckq_v8bf, t);
@@ -270,8 +280,8 @@ __global__ void __launch_bounds__(256 * KG, KG == 2 ? 1 : WPE) gemm_q4k_mfma_ker
         const int b0 = (int)(int16_t)(nbs[0] & 0xffff) + (int)(int16_t)(nbs[0] >> 16);
         const int b1 = (int)(int16_t)(nbs[1] & 0xffff) + (int)(int16_t)(nbs[1] >> 16);
         u32 *bd = reinterpret_cast<u32 *>(&stage[buf].b[st_tok * 16]);
-        bd[st_q]     = bf16_bits((float)(b0 & 63)) | (bf16_bits((float)(b1 & 63)) << 16);
-        bd[4 + st_q] = bf16_bits((float)(64 * (b0 >> 6))) | (bf16_bits((float)(64 * (b1 >> 6))) << 16);
+        bd[st_q]     = bf16_pair((float)(b0 & 63), (float)(b1 & 63));
+        bd[4 + st_q] = bf16_pair((float)(64 * (b0 >> 6)), (float)(64 * (b1 >> 6)));
     };
 
     /* read-side offsets of this lane */
@@ -296,8 +306,12 @@ __global__ void __launch_bounds__(256 * KG, KG == 2 ? 1 : WPE) gemm_q4k_mfma_ker
     /* both groups run the same number of iterations (the barrier is the
      * block's); a group without a block in the last one only keeps step */
     const int niter = (b1 - b0 + KG - 1) / KG;
-    for (int it = 0; it < niter; ++it) {
-        const int b = b0 + grp + KG * it, cur = it & 1;
+    /* One K-block.  The stage it reads is a compile-time constant (the loop
+     * below is unrolled by the two stages), so every LDS address of the block is
+     * a per-lane register set up once plus an immediate offset. */
+    auto kstep = [&](int it, auto curc) {
+        constexpr int cur = decltype(curc)::value;
+        const int b = b0 + grp + KG * it;
         copy_begin(min(b + KG, last), cur ^ 1);
         __builtin_amdgcn_sched_barrier(0);
         GemmDumpLane dl = {};
@@ -313,6 +327,10 @@ __global__ void __launch_bounds__(256 * KG, KG == 2 ? 1 : WPE) gemm_q4k_mfma_ker
         side_store(cur ^ 1);
         __builtin_amdgcn_s_waitcnt(0x0070);
         __syncthreads();
+    };
+    for (int it = 0; it < niter; it += 2) {
+        kstep(it, std::integral_constant<int, 0>{});
+        if (it + 1 < niter) kstep(it + 1, std::integral_constant<int, 1>{});
     }
 
     if constexpr (KG == 2) {
