@@ -30,6 +30,7 @@
  * Block = 4 waves = 64 tokens x 128 weight rows; wave w owns rows 32w..32w+31.
  */
 #include "ckq_gemm_common.cuh"
+#include <type_traits>
 
 constexpr int GEMM5_BM = 64, GEMM5_BN = 128, GEMM5_ROW = 176;
 
@@ -268,8 +269,11 @@ __global__ void __launch_bounds__(256, 1) gemm_q5k_mfma_kernel(GemmArgs a)
     /* Block b+1 has landed when only the copies issued during this iteration
      * are still in flight; the block's waves exchange data only through those
      * copies, so a bare s_barrier follows. */
-    int cur = 0, pf = NST - 1;
-    for (int b = b0; b < b1; ++b) {
+    /* One K-block; the stage it reads and the one it fills are compile-time
+     * constants (the loop is unrolled over the stages), so LDS addresses are
+     * per-lane registers set up once plus immediates. */
+    auto kstep = [&](int b, auto curc) {
+        constexpr int cur = decltype(curc)::value, pf = (cur + NST - 1) % NST;
         copy_begin(min(b + NST - 1, last), pf);
         __builtin_amdgcn_sched_barrier(0);
         GemmDumpLane dl = {};
@@ -284,8 +288,12 @@ __global__ void __launch_bounds__(256, 1) gemm_q5k_mfma_kernel(GemmArgs a)
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_waitcnt(0x0070 | (NCOPY & 15) | ((NCOPY >> 4) << 14));
         __builtin_amdgcn_s_barrier();
-        cur = cur + 1 == NST ? 0 : cur + 1;
-        pf = pf + 1 == NST ? 0 : pf + 1;
+    };
+    static_assert(NST == 3, "the loop is unrolled over three stages");
+    for (int b = b0; b < b1; b += 3) {
+        kstep(b, std::integral_constant<int, 0>{});
+        if (b + 1 < b1) kstep(b + 1, std::integral_constant<int, 1>{});
+        if (b + 2 < b1) kstep(b + 2, std::integral_constant<int, 2>{});
     }
 
     const GemmOut o = work.out;

@@ -31,6 +31,7 @@
  *   enough to fill the chip with them.
  */
 #include "ckq_gemm_common.cuh"
+#include <type_traits>
 
 constexpr int GEMM6_BN  = 128;   /* weight rows per tile */
 constexpr int GEMM6_ROW = 224;   /* LDS bytes per staged weight block: 14 chunks */
@@ -264,10 +265,14 @@ __global__ void __launch_bounds__(256, 1) gemm_q6k_mfma_kernel(GemmArgs a)
      * the copies issued during this iteration (three stages) or none (two) are
      * still in flight.  A bare s_barrier: the block's waves exchange data only
      * through those copies. */
-    int cur = 0, pf = NST - 1;
     Gemm6Head<TH> head;
     gemm6_head_read<TH>(stage[0], wrow, aofs[0], half, head);
-    for (int b = b0; b < b1; ++b) {
+    /* One K-block.  With three stages the stage it reads (and the one it fills)
+     * is a compile-time constant - the loop below is unrolled over the stages -
+     * so the LDS addresses of a block are per-lane registers set up once plus
+     * immediates. */
+    auto kstep = [&](int b, auto curc) {
+        const int cur = curc, pf = cur == 0 ? NST - 1 : cur - 1, nxt = cur + 1 == NST ? 0 : cur + 1;
         copy_begin(min(b + NST - 1, last), pf);
         __builtin_amdgcn_sched_barrier(0);
         Gemm6Sums<TH> sums;
@@ -284,21 +289,29 @@ __global__ void __launch_bounds__(256, 1) gemm_q6k_mfma_kernel(GemmArgs a)
         if constexpr (NST == 3) __builtin_amdgcn_s_waitcnt(0x0070 | (NCOPY & 15) | ((NCOPY >> 4) << 14));
         else                    __builtin_amdgcn_s_waitcnt(0x0070);
         __builtin_amdgcn_s_barrier();
-        cur = cur + 1 == NST ? 0 : cur + 1;
-        pf = pf + 1 == NST ? 0 : pf + 1;
         /* The next block's first reads, then this block's fp32 combine under
          * them (after the last block the stage holds that block again: unused).
          * The 128-token tile has no registers to spare for that overlap. */
         if constexpr (TH == 2) {
-            gemm6_head_read<TH>(stage[cur], wrow, aofs[0], half, head);
+            gemm6_head_read<TH>(stage[nxt], wrow, aofs[0], half, head);
             __builtin_amdgcn_sched_barrier(0);
             gemm6_combine<TH, DUMP>(sums, acc, dl);
         } else {
             gemm6_combine<TH, DUMP>(sums, acc, dl);
             __builtin_amdgcn_sched_barrier(0);
-            gemm6_head_read<TH>(stage[cur], wrow, aofs[0], half, head);
+            gemm6_head_read<TH>(stage[nxt], wrow, aofs[0], half, head);
         }
         __builtin_amdgcn_sched_barrier(0);
+    };
+    if constexpr (NST == 3) {
+        for (int b = b0; b < b1; b += 3) {
+            kstep(b, std::integral_constant<int, 0>{});
+            if (b + 1 < b1) kstep(b + 1, std::integral_constant<int, 1>{});
+            if (b + 2 < b1) kstep(b + 2, std::integral_constant<int, 2>{});
+        }
+    } else {            /* the 128-token tile has no registers to spare for constant-stage addressing */
+        int cur = 0;
+        for (int b = b0; b < b1; ++b, cur ^= 1) kstep(b, cur);
     }
 
     const GemmOut o = work.out;

@@ -31,6 +31,7 @@
  * Block = 4 waves = 64 tokens x 128 weight rows; wave w owns rows 32w..32w+31.
  */
 #include "ckq_gemm_common.cuh"
+#include <type_traits>
 
 constexpr int GEMM8_BM = 64, GEMM8_BN = 128, GEMM8_KB = 4;   /* tokens, rows, 32-blocks per iteration */
 
@@ -162,8 +163,11 @@ __global__ void __launch_bounds__(256, 2) gemm_q80_mfma_kernel(GemmArgs a)
     auto lds16 = [&](const void *p) { return *reinterpret_cast<const ckq_v4i *>(p); };
     const ckq_v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 
-    int cur = 0;
-    for (int it = it0; it < niter; ++it) {
+    /* One iteration (KB blocks); the stage it reads is a compile-time constant
+     * (the loop below is unrolled over the two stages): LDS addresses are
+     * per-lane registers set up once plus immediates. */
+    auto kstep = [&](int it, auto curc) {
+        constexpr int cur = decltype(curc)::value;
         const Gemm8Stage &st = stage[cur];
         const int valid = min(KB, nblk - it * KB);
         /* Operands of block j (read one block ahead of their use, through the
@@ -218,7 +222,10 @@ __global__ void __launch_bounds__(256, 2) gemm_q80_mfma_kernel(GemmArgs a)
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_waitcnt(0x0070);                /* vmcnt(0): the next iteration has landed */
         __builtin_amdgcn_s_barrier();
-        cur ^= 1;
+    };
+    for (int it = it0; it < niter; it += 2) {
+        kstep(it, std::integral_constant<int, 0>{});
+        if (it + 1 < niter) kstep(it + 1, std::integral_constant<int, 1>{});
     }
 
     /* lane: token t0 + col + 32 ts, rows n0 + 32 wave + 8 q + 4 half + (0..3) */
