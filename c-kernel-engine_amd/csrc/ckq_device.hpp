@@ -1,5 +1,5 @@
 /*
- * ckq_device.cuh - gfx950 device helpers shared by the quantized kernels:
+ * ckq_device.hpp - gfx950 device helpers shared by the quantized kernels:
  * unaligned 128-bit loads, packed int8 dot, wave64 DPP reductions.
  */
 #pragma once

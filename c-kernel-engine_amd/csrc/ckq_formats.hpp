@@ -1,5 +1,5 @@
 /*
- * ckq_formats.cuh - per-format traits for the dequant-dot kernels.
+ * ckq_formats.hpp - per-format traits for the dequant-dot kernels.
  *
  * A weight row is cut into "positions": the unit of work of one lane.
  *   Q4_K / Q5_K : one 64-element group of a super-block (header + 32 B of
@@ -27,7 +27,7 @@
  *   Q8_0 x fp32  gemm_kernels_q8_0.c:254-277      sum d*q*x
  */
 #pragma once
-#include "ckq_device.cuh"
+#include "ckq_device.hpp"
 
 /* 6-bit scale/min pair of sub-blocks (2g, 2g+1) from the 12 packed bytes
  * (layout: reference include/ckernel_quant.h:227-251).  u0,u1,u2 are the

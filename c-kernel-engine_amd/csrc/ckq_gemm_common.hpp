@@ -1,11 +1,11 @@
 /*
- * ckq_gemm_common.cuh - what the four matrix-core GEMM kernels share: operand
+ * ckq_gemm_common.hpp - what the four matrix-core GEMM kernels share: operand
  * vector types, the launch arguments, the K-split bookkeeping and the entry
  * points of each kernel's translation unit.
  */
 #pragma once
 #include <mutex>
-#include "ckq_device.cuh"
+#include "ckq_device.hpp"
 #include "ckq_launch.h"
 
 typedef int   ckq_v4i  __attribute__((ext_vector_type(4)));

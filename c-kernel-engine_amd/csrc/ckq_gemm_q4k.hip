@@ -37,7 +37,7 @@
  * 32w..32w+31.  Grid: token tiles fastest inside an XCD so the eight XCD L2s
  * each see a weight tile once.
  */
-#include "ckq_gemm_common.cuh"
+#include "ckq_gemm_common.hpp"
 #include <type_traits>
 
 #ifndef CKQ_GEMM_WPE

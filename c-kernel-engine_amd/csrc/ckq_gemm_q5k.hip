@@ -29,7 +29,7 @@
  *
  * Block = 4 waves = 64 tokens x 128 weight rows; wave w owns rows 32w..32w+31.
  */
-#include "ckq_gemm_common.cuh"
+#include "ckq_gemm_common.hpp"
 #include <type_traits>
 
 constexpr int GEMM5_BM = 64, GEMM5_BN = 128, GEMM5_ROW = 176;

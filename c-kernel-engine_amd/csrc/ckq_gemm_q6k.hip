@@ -30,7 +30,7 @@
  *   slab s and larger token tiles (TH = 4) amortise it where the grid is big
  *   enough to fill the chip with them.
  */
-#include "ckq_gemm_common.cuh"
+#include "ckq_gemm_common.hpp"
 #include <type_traits>
 
 constexpr int GEMM6_BN  = 128;   /* weight rows per tile */

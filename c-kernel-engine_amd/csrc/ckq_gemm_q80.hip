@@ -30,7 +30,7 @@
  *
  * Block = 4 waves = 64 tokens x 128 weight rows; wave w owns rows 32w..32w+31.
  */
-#include "ckq_gemm_common.cuh"
+#include "ckq_gemm_common.hpp"
 #include <type_traits>
 
 constexpr int GEMM8_BM = 64, GEMM8_BN = 128, GEMM8_KB = 4;   /* tokens, rows, 32-blocks per iteration */

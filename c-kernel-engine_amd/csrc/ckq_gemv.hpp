@@ -1,7 +1,7 @@
 /*
- * ckq_gemv.cuh - the weight-streaming dequant-dot kernel (decode GEMV and token
+ * ckq_gemv.hpp - the weight-streaming dequant-dot kernel (decode GEMV and token
  * tiles of up to eight activation rows) and its launch-shape selection, as
- * templates over the per-format traits of ckq_formats.cuh.  Each format is
+ * templates over the per-format traits of ckq_formats.hpp.  Each format is
  * instantiated in a translation unit of its own (ckq_gemv_<fmt>.hip).
  */
 #pragma once
@@ -9,7 +9,7 @@
 #include <stdint.h>
 
 #include "ckq_blocks.h"
-#include "ckq_formats.cuh"
+#include "ckq_formats.hpp"
 #include "ckq_launch.h"
 
 constexpr int CKQ_GROUP_MAX = 4;   /* independent matmuls of one shape in one launch */

@@ -19,7 +19,7 @@
 #include <stdint.h>
 
 #include "ckq_blocks.h"
-#include "ckq_formats.cuh"
+#include "ckq_formats.hpp"
 #include "ckq_launch.h"
 
 /* ========================================================================= */
@@ -71,8 +71,8 @@ static bool gemm_on_matrix_cores(int ntok, size_t weight_bytes, size_t budget_mb
     return passes * per > (budget_mb << 20);
 }
 
-#include "ckq_gemv.cuh"
-#include "ckq_gemm_common.cuh"
+#include "ckq_gemv.hpp"
+#include "ckq_gemm_common.hpp"
 
 /* C = bias + partial 0 + partial 1 + ... in that order: the result does not
  * depend on which block finished first.  One thread per output. */
@@ -91,7 +91,7 @@ __global__ void __launch_bounds__(256) gemm_splitk_reduce_kernel(float *__restri
 static std::recursive_mutex g_split_mu;
 std::recursive_mutex &gemm_split_mutex() { return g_split_mu; }
 
-/* Grow-only device scratch per (stream, kind); see ckq_gemm_common.cuh. */
+/* Grow-only device scratch per (stream, kind); see ckq_gemm_common.hpp. */
 /* kind 0: partial tiles of a K split; kind 1: weights rewritten for another kernel */
 int gemm_workspace(int kind, hipStream_t s, size_t bytes, float **out)
 {
