@@ -88,6 +88,8 @@ _SIGS = {
     "gemm_q8_0": (None, [_vp, _vp, _vp, _i, _i, _i]),
     "gemm_nt_q8_0": (None, [_vp, _vp, _vp, _vp, _i, _i, _i]),
     "ck_test_quantize_q8_k": (None, [_vp, _vp, _i]),
+    "ck_test_dequant_q4_k": (None, [_vp, _vp, _i]),
+    "ck_test_dequant_q6_k": (None, [_vp, _vp, _i]),
     "ck_test_gemv_q4_k": (None, [_vp, _vp, _vp, _i]),
     "ck_test_gemv_q6_k": (None, [_vp, _vp, _vp, _i]),
     "ck_test_gemv_q8_0": (None, [_vp, _vp, _vp, _i, _i]),
@@ -133,6 +135,8 @@ _SIGS = {
     "ckq_weights_invalidate": (None, [_vp]),
     "ckq_weights_clear": (None, []),
     "ckq_weights_set_cache": (None, [_i]),
+    "ckq_weights_set_limit": (None, [_c.c_size_t]),
+    "ckq_release_stream": (_i, [_vp]),
     "ckq_set_parallel_whole": (None, [_i]),
     "ckq_set_gemm_policy": (None, [_i]),
     "ckq_last_error": (_i, []),

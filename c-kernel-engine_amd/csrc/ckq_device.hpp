@@ -84,10 +84,13 @@ __device__ __forceinline__ T group_sum(T v)
     return v;
 }
 
-/* x86 cvtps2dq + saturating packs: round to nearest even, NaN -> -128. */
+/* x86 cvtps2dq + saturating packs (quantize_row_q8_k_sse.c:61-68): round to
+ * nearest even; NaN, +-inf and anything outside int32 convert to INT_MIN, which
+ * the packs saturate to -128 - also for +inf and for values >= 2^31 (a block of
+ * magnitudes below 127/FLT_MAX has an infinite inverse scale). */
 __device__ __forceinline__ int rne_sat_i8(float p)
 {
-    if (p != p) return -128;
+    if (!(p < 2147483648.0f)) return -128;     /* NaN, +inf, >= 2^31 */
     const float r = __builtin_rintf(p);
     return (int)fminf(fmaxf(r, -128.0f), 127.0f);
 }

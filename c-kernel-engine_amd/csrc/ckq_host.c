@@ -56,7 +56,7 @@ static int          g_cache_on = 1;
 /* Thread-split entry points: 1 = the ith == 0 call computes all rows in one
  * launch and the other threads return (through the reference's 16-thread pool:
  * 53 us per GEMV against 480 us when each thread runs its own row range). */
-#define CKQ_PARALLEL_WHOLE_DEFAULT 1
+#define CKQ_PARALLEL_WHOLE_DEFAULT 0
 static int          g_parallel_whole = CKQ_PARALLEL_WHOLE_DEFAULT;
 static hipStream_t  g_stream = NULL;
 static dev_buf      g_buf[BUF_COUNT];
@@ -320,6 +320,10 @@ static uint64_t fingerprint(const void *p, size_t bytes)
  * evicted. */
 enum { CACHE_MAX_ENTRIES = 4096 };
 static uint64_t g_use_clock = 0;
+/* g_use_clock when the current call resolved its first weight operand: entries
+ * used later than this belong to the call and must stay until its kernels are
+ * enqueued (the fused MLP holds W1 while it resolves W2). */
+static uint64_t g_call_epoch = 0;
 
 static size_t cache_unpinned_bytes(void)
 {
@@ -331,23 +335,28 @@ static size_t cache_unpinned_bytes(void)
 
 static void drop_entry(size_t i);
 
-/* Make room for a new unpinned entry of `bytes`. */
-static void cache_evict_for(size_t bytes)
+/* Make room for a new unpinned entry of `bytes`: least recently used entries go
+ * first, entries of the current call never.  Returns 0 when the bound cannot
+ * be met (the caller then serves the operand without caching it). */
+static int cache_evict_for(size_t bytes)
 {
     for (;;) {
         size_t n_unpinned = 0, lru = (size_t)-1;
         for (size_t i = 0; i < g_nw; ++i) {
             if (g_w[i].pinned) continue;
             ++n_unpinned;
+            if (g_w[i].last_use > g_call_epoch) continue;      /* held by this call */
             if (lru == (size_t)-1 || g_w[i].last_use < g_w[lru].last_use) lru = i;
         }
-        if (lru == (size_t)-1) return;
-        if (n_unpinned < CACHE_MAX_ENTRIES && cache_unpinned_bytes() + bytes <= g_cache_max_bytes) return;
+        if (n_unpinned < CACHE_MAX_ENTRIES && cache_unpinned_bytes() + bytes <= g_cache_max_bytes) return 1;
+        if (lru == (size_t)-1) return 0;
         drop_entry(lru);
     }
 }
 
-static int weights_lookup(const void *W, size_t bytes, const void **out)
+static int weights_uncached(int slot, const void *W, size_t bytes, const void **out);
+
+static int weights_lookup(int slot, const void *W, size_t bytes, const void **out)
 {
     if (is_device_ptr(W)) {
         *out = W;
@@ -377,7 +386,10 @@ static int weights_lookup(const void *W, size_t bytes, const void **out)
             return 0;
         }
     }
-    cache_evict_for(bytes);
+    if (!cache_evict_for(bytes)) {
+        if (slot < 0) return fail((int)hipErrorOutOfMemory, "registering weights beyond the cache bound");
+        return weights_uncached(slot, W, bytes, out);
+    }
     if (g_nw == g_capw) {
         size_t nc = g_capw ? g_capw * 2 : 64;
         weight_entry *nw = (weight_entry *)realloc(g_w, nc * sizeof(*nw));
@@ -440,6 +452,7 @@ static int in_registered_region(const void *W, size_t bytes)
 /* Device view of weight operand number `slot` (0 or 1) of the current call. */
 static int weights_resolve(int slot, const void *W, size_t bytes, const void **out)
 {
+    if (slot == 0) g_call_epoch = g_use_clock;       /* the first operand opens a call */
     if (is_device_ptr(W)) {
         *out = W;
         return 0;
@@ -449,13 +462,14 @@ static int weights_resolve(int slot, const void *W, size_t bytes, const void **o
      * harness's scratch matrix) are cheaper to copy than to track: a per-row
      * loop over a large matrix would otherwise leave one allocation per row. */
     if (bytes < CACHE_MIN_BYTES && !in_registered_region(W, bytes)) return weights_uncached(slot, W, bytes, out);
-    return weights_lookup(W, bytes, out);
+    return weights_lookup(slot, W, bytes, out);
 }
 
 static int register_locked(const void *W, size_t bytes)
 {
     const void *d;
-    int rc = weights_lookup(W, bytes, &d);
+    g_call_epoch = g_use_clock;
+    int rc = weights_lookup(-1, W, bytes, &d);
     if (rc) return rc;
     for (size_t i = 0; i < g_nw; ++i)
         if (g_w[i].host == W && g_w[i].bytes == bytes) g_w[i].pinned = 1;
@@ -561,6 +575,17 @@ void ckq_weights_clear(void)
     pthread_mutex_unlock(&g_mu);
 }
 
+void ckq_weights_set_limit(size_t bytes)
+{
+    pthread_mutex_lock(&g_mu);
+    g_cache_max_bytes = bytes ? bytes : (size_t)64 << 30;
+    g_call_epoch = g_use_clock;
+    (void)cache_evict_for(0);
+    pthread_mutex_unlock(&g_mu);
+}
+
+int ckq_release_stream(void *stream) { return ckq_launch_release_stream(stream); }
+
 void ckq_weights_set_cache(int enabled)
 {
     pthread_mutex_lock(&g_mu);
@@ -575,9 +600,9 @@ void ckq_set_parallel_whole(int enabled)
     pthread_mutex_lock(&g_mu);
     if (enabled < 0) {                       /* back to the default (CKQ_PARALLEL_MODE or the built-in one) */
         const char *p = getenv("CKQ_PARALLEL_MODE");
-        g_parallel_whole = p ? strcmp(p, "whole") == 0 : CKQ_PARALLEL_WHOLE_DEFAULT;
+        __atomic_store_n(&g_parallel_whole, p ? strcmp(p, "whole") == 0 : CKQ_PARALLEL_WHOLE_DEFAULT, __ATOMIC_RELAXED);
     } else {
-        g_parallel_whole = enabled != 0;
+        __atomic_store_n(&g_parallel_whole, enabled != 0, __ATOMIC_RELAXED);
     }
     pthread_mutex_unlock(&g_mu);
 }
@@ -634,7 +659,9 @@ static void matmul_locked(int fmt, const void *A, const void *B, const float *bi
             void *t;
             ld = row1 - row0; /* compact staging: only the computed rows */
             if (buf_reserve(BUF_Y, (size_t)ntok * (size_t)ld * sizeof(float), &t)) break;
-            dC = (float *)t - row0; /* kernel indexes with absolute rows */
+            /* the kernel indexes with absolute rows: bias the base by row0 in integer
+             * arithmetic (a pointer in front of its allocation must not be formed) */
+            dC = (float *)((uintptr_t)t - (uintptr_t)row0 * sizeof(float));
         }
         int rc = ckq_launch_gemv(fmt, dC, dB, dA, (const float *)dbias, nrows, K, ntok, ld, row0, row1, NULL, g_stream);
         if (rc) { fail(rc, "ckq_launch_gemv"); break; }
@@ -667,7 +694,7 @@ static void host_matmul(int fmt, const void *A, const void *B, const float *bias
 static int split_rows(int M, int ith, int nth, int *r0, int *r1)
 {
     if (ith < 0 || nth <= 0 || ith >= nth) return 0;
-    if (g_parallel_whole) {
+    if (__atomic_load_n(&g_parallel_whole, __ATOMIC_RELAXED)) {
         if (ith != 0) return 0;
         *r0 = 0;
         *r1 = M;
@@ -1104,6 +1131,8 @@ void gemm_nt_q8_0(const float *A, const void *B, const float *bias, float *C, in
 
 /* Parity-test wrappers (reference: src/ck_parity_api.c). */
 void ck_test_quantize_q8_k(const float *src, void *dst, int n) { quantize_row_q8_k(src, dst, n); }
+void ck_test_dequant_q4_k(const void *src, float *dst, int n) { if (n > 0) dequant_q4_k_row(src, dst, (size_t)n); }
+void ck_test_dequant_q6_k(const void *src, float *dst, int n) { if (n > 0) dequant_q6_k_row(src, dst, (size_t)n); }
 
 void ck_test_gemv_q4_k(const void *w, const float *in, float *out, int cols)
 {

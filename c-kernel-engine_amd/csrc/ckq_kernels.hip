@@ -91,29 +91,96 @@ __global__ void __launch_bounds__(256) gemm_splitk_reduce_kernel(float *__restri
 static std::recursive_mutex g_split_mu;
 std::recursive_mutex &gemm_split_mutex() { return g_split_mu; }
 
-/* Grow-only device scratch per (stream, kind); see ckq_gemm_common.hpp. */
-/* kind 0: partial tiles of a K split; kind 1: weights rewritten for another kernel */
+/* Slot bookkeeping of gemm_workspace, free of HIP calls so that it can be tested on
+ * the CPU: the slot whose key equals `key`, else the first free one (key 0), else the
+ * least recently used one (smallest last_use), which the caller recycles. */
+extern "C" int ckq_workspace_pick(const uint64_t *keys, const uint64_t *last_use, int n, uint64_t key)
+{
+    int free_slot = -1, lru = 0;
+    for (int i = 0; i < n; ++i) {
+        if (keys[i] == key) return i;
+        if (keys[i] == 0 && free_slot < 0) free_slot = i;
+        if (last_use[i] < last_use[lru]) lru = i;
+    }
+    return free_slot >= 0 ? free_slot : lru;
+}
+
+/* Grow-only device scratch per (device, stream, kind); see ckq_gemm_common.hpp.
+ * kind 0: partial tiles of a K split; kind 1: weights rewritten for another kernel.
+ * When all slots are taken the least recently used one is recycled: the device is
+ * synchronised (its stream may no longer exist), its buffer freed.  A destroyed
+ * stream whose handle value is given out again finds the old stream's slot: harmless,
+ * that stream's work has ended and the buffer is still this device's memory.
+ * ckq_launch_release_stream gives a stream's slots back explicitly. */
+namespace {
+constexpr int WS_SLOTS = 32;
+struct WsSlot { hipStream_t s; int kind, dev; void *p; size_t cap; };
+WsSlot   g_ws[WS_SLOTS];
+uint64_t g_ws_key[WS_SLOTS], g_ws_use[WS_SLOTS], g_ws_clock = 0;
+uint64_t ws_key(int dev, hipStream_t s, int kind)
+{
+    /* lossless for user-space handles (below 2^56), 32 devices and two kinds; never 0 */
+    return (1ull << 63) | ((uint64_t)(kind & 1) << 61) | ((uint64_t)(dev & 31) << 56) | ((uint64_t)(uintptr_t)s & ((1ull << 56) - 1));
+}
+}
+
 int gemm_workspace(int kind, hipStream_t s, size_t bytes, float **out)
 {
-    struct Slot { hipStream_t s; int kind; void *p; size_t cap; bool used; };
-    static Slot slots[32];
-    Slot *sl = nullptr;
-    for (auto &c : slots) if (c.used && c.s == s && c.kind == kind) { sl = &c; break; }
-    if (!sl) for (auto &c : slots) if (!c.used) { sl = &c; c.used = true; c.s = s; c.kind = kind; c.p = nullptr; c.cap = 0; break; }
-    if (!sl) return (int)hipErrorOutOfMemory;
+    std::lock_guard<std::recursive_mutex> lock(g_split_mu);
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    const uint64_t key = ws_key(dev, s, kind);
+    int i = ckq_workspace_pick(g_ws_key, g_ws_use, WS_SLOTS, key);
+    WsSlot *sl = &g_ws[i];
+    if (g_ws_key[i] != key) {
+        if (g_ws_key[i] != 0 && sl->p) {                 /* recycle */
+            int cur = dev;
+            if (sl->dev != cur) (void)hipSetDevice(sl->dev);
+            e = hipDeviceSynchronize();
+            if (e == hipSuccess) e = hipFree(sl->p);
+            if (sl->dev != cur) (void)hipSetDevice(cur);
+            if (e != hipSuccess) return (int)e;
+        }
+        g_ws_key[i] = key;
+        *sl = {s, kind, dev, nullptr, 0};
+    }
+    g_ws_use[i] = ++g_ws_clock;
     if (sl->cap < bytes) {
         if (sl->p) {
-            hipError_t e = hipStreamSynchronize(s);
+            e = hipStreamSynchronize(s);
             if (e != hipSuccess) return (int)e;
             (void)hipFree(sl->p);
             sl->p = nullptr; sl->cap = 0;
         }
         const size_t cap = bytes + bytes / 2;
-        hipError_t e = hipMalloc(&sl->p, cap);
+        e = hipMalloc(&sl->p, cap);
         if (e != hipSuccess) return (int)e;
         sl->cap = cap;
     }
     *out = (float *)sl->p;
+    return 0;
+}
+
+/* Frees the scratch held for `stream` on the current device (call before the
+ * stream is destroyed, after its work has been synchronised). */
+extern "C" int ckq_launch_release_stream(void *stream)
+{
+    std::lock_guard<std::recursive_mutex> lock(g_split_mu);
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    for (int i = 0; i < WS_SLOTS; ++i) {
+        if (g_ws_key[i] == 0 || g_ws[i].s != (hipStream_t)stream || g_ws[i].dev != dev) continue;
+        if (g_ws[i].p) {
+            e = hipStreamSynchronize((hipStream_t)stream);
+            if (e != hipSuccess) return (int)e;
+            (void)hipFree(g_ws[i].p);
+        }
+        g_ws_key[i] = 0;
+        g_ws_use[i] = 0;
+        g_ws[i] = {};
+    }
     return 0;
 }
 
@@ -386,6 +453,19 @@ extern "C" int ckq_launch_gemv_noalloc(int fmt, float *y, const void *W, const v
     if (fmt != CKQ_FMT_Q4_K && fmt != CKQ_FMT_Q5_K && fmt != CKQ_FMT_Q6_K && fmt != CKQ_FMT_Q8_0) return CKQ_EFORMAT;
     if (!y || !W || !X || nrows <= 0 || K <= 0 || ntok <= 0 || ldy < nrows) return CKQ_EINVAL;
     void *p = nullptr;
+    {
+        /* The scratch address of this device is normally resolved by ckq_init().  Resolving it
+         * here, on a first call, may load the code object, which is not legal while the stream
+         * is being captured: such a call is refused instead. */
+        int dev = 0;
+        if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < CKQ_MAX_DEVICES &&
+            !g_scratch_ptr[dev].load(std::memory_order_acquire)) {
+            hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+            if (hipStreamIsCapturing((hipStream_t)stream, &st) == hipSuccess && st != hipStreamCaptureStatusNone)
+                return (int)hipErrorStreamCaptureUnsupported;
+            (void)hipGetLastError();
+        }
+    }
     const int rc = noalloc_scratch(&p);
     if (rc) return rc;
     GemvArgs a = {};
@@ -599,13 +679,11 @@ extern "C" int ckq_launch_rmsnorm_q8_k_fused(const float *input, const float *ga
     const size_t lds = (size_t)d_model * 4 + 32;
     if (lds > 160 * 1024) return CKQ_ESHAPE;               /* the row is staged in LDS */
     if (lds > 64 * 1024) {
-        static bool raised = false;                        /* opt in to more than 64 KB of dynamic LDS once */
-        if (!raised) {
-            hipError_t e = hipFuncSetAttribute((const void *)rmsnorm_q8_k_fused_kernel,
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-            if (e != hipSuccess) return (int)e;
-            raised = true;
-        }
+        /* more than 64 KB of dynamic LDS is an opt-in per function and per device: set on every
+         * such call for the device that is current (rows this long are rare; the call is cheap) */
+        hipError_t e = hipFuncSetAttribute((const void *)rmsnorm_q8_k_fused_kernel,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return (int)e;
     }
     hipLaunchKernelGGL(rmsnorm_q8_k_fused_kernel, dim3((unsigned)tokens), dim3(256), lds, (hipStream_t)stream,
                        input, gamma, (uint8_t *)y, d_model, (long)aligned_embed_dim, eps);

@@ -96,6 +96,10 @@ int ckq_launch_dequant_rows(int fmt, const void *table, const int32_t *ids, int 
  * device (once per device; also done by the first call on a device). */
 #define CKQ_NOALLOC_SCRATCH_BYTES ((size_t)4 << 20)
 int ckq_launch_noalloc_setup(void);
+/* Frees the K-split / rewrite scratch held for `stream` on the current device. */
+int ckq_launch_release_stream(void *stream);
+/* Slot choice of that scratch table (no HIP calls; unit-tested on the CPU). */
+int ckq_workspace_pick(const uint64_t *keys, const uint64_t *last_use, int n, uint64_t key);
 int ckq_launch_gemv_noalloc(int fmt, float *y, const void *W, const void *X, const float *bias,
                             int nrows, int K, int ntok, long ldy, void *stream);
 

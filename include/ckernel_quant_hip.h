@@ -187,10 +187,13 @@ void fused_mlp_swiglu_prefill_w1w2_quant(const float *x, const void *W1, const f
 size_t fused_mlp_swiglu_prefill_w1w2_quant_scratch_size(int aligned_embed_dim, int aligned_intermediate_dim);
 
 /* Parity-test wrappers: fp32 input is quantized, then the kernel runs.
- * Replace src/ck_parity_api.c:207-210 (quantize), :217-258 (gemv q4_k/q6_k),
+ * Replace src/ck_parity_api.c:189-197 (dequant), :207-210 (quantize), :217-258 (gemv q4_k/q6_k),
  * :288-360 (gemv q8_0), :397-400 (vec_dot), :411-503 (gemm) and the size
  * getters of include/ck_parity_api.h:614-629. */
 void ck_test_quantize_q8_k(const float *src, void *dst, int n);
+/* include/ck_parity_api.h:48-53, src/ck_parity_api.c:189-197: the row dequantizers under their parity names */
+void ck_test_dequant_q4_k(const void *src, float *dst, int n);
+void ck_test_dequant_q6_k(const void *src, float *dst, int n);
 void ck_test_gemv_q4_k(const void *weight_q4k, const float *input_f32, float *output, int cols);
 void ck_test_gemv_q6_k(const void *weight_q6k, const float *input_f32, float *output, int cols);
 void ck_test_gemv_q8_0(const void *weight_q8_0, const float *input_f32, float *output, int rows, int cols);
@@ -242,7 +245,10 @@ int ckq_gemm_nt_dev(int fmt, const void *A_q8, const void *B, const float *bias,
  * frees or synchronizes.  Every call on a GPU shares that GPU's array: calls
  * that overlap on one GPU (two streams, two threads) race.  The array's
  * address is resolved once per device, by ckq_init() or by the first call on
- * that device. */
+ * that device; resolving it may load the library's code object, so call
+ * ckq_init() on the device BEFORE a region that must not allocate, and before
+ * stream capture begins: a first call on a capturing stream with the address
+ * still unresolved returns hipErrorStreamCaptureUnsupported. */
 int ckq_gemm_nt_noalloc_dev(int fmt, const void *A_q8, const void *B, const float *bias, float *C,
                             int M, int N, int K, long ldc, void *stream);
 
@@ -386,13 +392,25 @@ int  ckq_weights_resident(size_t *bytes);
 void ckq_weights_invalidate(const void *W);
 void ckq_weights_clear(void);
 void ckq_weights_set_cache(int enabled);
-/* Thread-split entry points (*_parallel, *_parallel_simd): 1 (default; also
- * CKQ_PARALLEL_MODE=whole) = the ith == 0 call computes all rows in one launch
- * and the other threads return at once, which is what a thread pool that calls
- * every ith wants (one upload, launch and download instead of nth serialized
- * ones); 0 (CKQ_PARALLEL_MODE=rows) = every call computes exactly its own row
- * range, for callers that invoke single ith values; a negative value restores
- * the default. */
+/* Bound on the bytes of resident weights that are not registered (0 = the
+ * default of 64 GiB; CKQ_WEIGHT_CACHE_MB sets it from the environment).  The
+ * least recently used entries are dropped first, never one the running call
+ * uses; an operand that does not fit beside those is uploaded for the call
+ * and not kept. */
+void ckq_weights_set_limit(size_t bytes);
+/* Frees the device scratch the library keeps for `stream` (a hipStream_t) on
+ * the current device: the partial tiles of K-split GEMMs and rewritten Q5_0
+ * weights.  Call it before destroying a stream that ran ckq_*_dev calls. */
+int  ckq_release_stream(void *stream);
+/* Thread-split entry points (*_parallel, *_parallel_simd): 0 (the default;
+ * CKQ_PARALLEL_MODE=rows) = every call computes exactly the row range of its
+ * ith, as the reference does (gemm_kernels_q4k_q8k.c:212-231), so a caller
+ * that invokes single ith values or reads its rows before a barrier is served;
+ * 1 (CKQ_PARALLEL_MODE=whole) = the ith == 0 call computes all rows in one
+ * launch and the other threads return at once - for a thread pool that calls
+ * every ith and joins at a barrier, like the reference's (one upload, launch
+ * and download instead of nth serialized ones: 5 to 9 times faster per
+ * dispatch); a negative value restores the default. */
 void ckq_set_parallel_whole(int enabled);
 /* Which kernel serves a matmul of more than eight tokens (up to eight always
  * take the weight-streaming kernel, one pass over the weights).  AUTO, the

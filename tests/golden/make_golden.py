@@ -91,6 +91,26 @@ def q8k_edge_inputs():
     rows.append(a)
     a = np.linspace(-1.0, 1.0, 256).astype(np.float32)      # both extremes equal magnitude
     rows.append(a)
+    # magnitudes below 127/FLT_MAX: the inverse scale is infinite, products are +-inf
+    # or NaN (0 * inf), and cvtps2dq turns all of them into INT_MIN -> -128
+    a = (np.where(np.arange(256) % 3 == 0, -1.0, 1.0) * np.geomspace(1e-38, 1e-41, 256)).astype(np.float32)
+    rows.append(a)                                          # mixed signs, 1e-38 .. 1e-41
+    a = np.full(256, -2e-39, np.float32); a[100] = 1e-40    # a single +tiny among -tiny
+    rows.append(a)
+    a = z.copy(); a[3] = 3e-38; a[77] = -1e-39              # zeros beside an infinite inverse scale
+    rows.append(a)
+    return np.concatenate(rows)
+
+
+def q80_edge_inputs():
+    """32-element blocks whose inverse scale 127/amax overflows to +inf."""
+    rows = []
+    a = (np.where(np.arange(32) % 2 == 0, 1.0, -1.0) * np.geomspace(1e-38, 1e-41, 32)).astype(np.float32)
+    rows.append(a)                                          # mixed signs
+    a = np.full(32, -2e-39, np.float32); a[5] = 1e-40       # a single +tiny among -tiny
+    rows.append(a)
+    a = np.zeros(32, np.float32); a[9] = 2e-38              # zeros: 0 * inf = NaN
+    rows.append(a)
     return np.concatenate(rows)
 
 
@@ -120,7 +140,8 @@ def main():
     x_0 = np.concatenate([normal(S, 96 * 32, 0.0, 1.0, 111), np.zeros(32, np.float32),
                           np.full(32, 2.5, np.float32), normal(S, 16 * 32, 0.0, 1e-6, 112),
                           normal(S, 16 * 32, 0.0, 1e4, 113),
-                          (np.arange(32, dtype=np.float32) - 16.0) / 2.0 * (127.0 / 127.0)])
+                          (np.arange(32, dtype=np.float32) - 16.0) / 2.0 * (127.0 / 127.0),
+                          q80_edge_inputs()])
     G["q80_in"] = x_0
     outs = {}
     for tag, L in libs.items():

@@ -38,6 +38,10 @@ def test_reference_symbol_names_present(L):
               "gemv_q6_k_q8_k", "gemv_q6_k_q8_k_parallel_simd", "gemm_nt_q6_k_q8_k", "gemv_q8_0_q8_0",
               "gemv_q8_0", "gemm_nt_q8_0_q8_0", "vec_dot_q6_k_q8_k", "vec_dot_q8_0_q8_0"]:
         assert hasattr(L, n)
+    # the parity scripts' wrappers (reference include/ck_parity_api.h:42-56, 193-201)
+    for n in ["ck_test_dequant_q4_k", "ck_test_dequant_q6_k", "ck_test_quantize_q8_k", "ck_test_gemv_q4_k",
+              "ck_test_gemv_q6_k", "ck_test_gemm_q4_k", "ck_test_gemm_q6_k", "ck_test_gemm_q8_0"]:
+        assert hasattr(L, n)
 
 
 def test_block_size_getters(L):
@@ -147,6 +151,41 @@ def test_grid_chunk_index_arithmetic(L):
             covered += count.value
             c += 1
         assert covered == total and c == -(-total // per)
+
+
+def test_workspace_slot_bookkeeping(L):
+    """Slot choice of the per-(device, stream, kind) scratch table of the K-split
+    GEMMs: a known key finds its slot, a new key takes the first free slot, and
+    with every slot taken the least recently used one is handed out for
+    recycling - more distinct streams than slots must not fail."""
+    n = 8
+    U64 = ctypes.c_uint64 * n
+    L.ckq_workspace_pick.restype = ctypes.c_int
+    L.ckq_workspace_pick.argtypes = [U64, U64, ctypes.c_int, ctypes.c_uint64]
+    keys, use = U64(), U64()
+    clock = 0
+    where = {}
+    for k in range(1, 3 * n + 1):                    # 24 distinct "streams" through 8 slots
+        key = (1 << 63) | (0x7f0000001000 + 64 * k)
+        i = L.ckq_workspace_pick(keys, use, n, key)
+        assert 0 <= i < n
+        if k <= n:
+            assert keys[i] == 0 and i == k - 1       # first free slot, in order
+        else:
+            assert use[i] == min(use)                # least recently used
+            where = {kk: ii for kk, ii in where.items() if ii != i}
+        keys[i] = key
+        clock += 1
+        use[i] = clock
+        where[key] = i
+        # a key that is present is found again, whatever its age
+        for kk, ii in where.items():
+            assert L.ckq_workspace_pick(keys, use, n, kk) == ii
+    # touching an old entry protects it from being the next victim
+    oldest = min(range(n), key=lambda j: use[j])
+    clock += 1
+    use[oldest] = clock
+    assert L.ckq_workspace_pick(keys, use, n, (1 << 63) | 0x1234) != oldest
 
 
 def test_no_device_fails_loudly():

@@ -123,8 +123,10 @@ def np_block_sums(fmt, W, A, M, N, K):
 
 GEMM_DUMP_SHAPES = {
     "q4_k": [(70, 200, 1024), (130, 384, 2048), (33, 128, 256), (64, 130, 4096), (520, 260, 512)],
-    "q5_k": [(70, 200, 1024), (66, 96, 512), (130, 333, 2048)],
-    "q6_k": [(70, 200, 1024), (130, 1100, 512), (33, 128, 256), (140, 384, 2048)],   # 64- and 128-token tiles
+    # K = 768 and 1536: 3 and 6 K-blocks, the exit of the three-stage K loops after a whole round of stages
+    "q5_k": [(70, 200, 1024), (66, 96, 512), (130, 333, 2048), (40, 160, 768), (70, 130, 1536)],
+    "q6_k": [(70, 200, 1024), (130, 1100, 512), (33, 128, 256), (140, 384, 2048),    # 64- and 128-token tiles
+             (40, 160, 768), (140, 130, 1536), (70, 96, 2304)],
     "q8_0": [(70, 200, 896), (130, 333, 160), (33, 128, 32), (64, 96, 1024)],
 }
 
@@ -469,6 +471,46 @@ def test_host_paths_with_weight_cache_off():
         assert L.ckq_weights_resident(None) == 0
     finally:
         L.ckq_weights_set_cache(1)
+
+
+def test_weight_cache_eviction_under_a_small_limit():
+    """A bound on resident weights smaller than W1 + W2 of a fused MLP: the
+    lookup of W2 must not drop W1, which the same call still holds (it is
+    served uncached instead), alternating GEMVs evict each other, results stay
+    those of the oracle and the resident bytes stay within the bound."""
+    L = ckq.lib()
+    L.ckq_weights_clear()
+    seq, E, I = 70, 256, 1024
+    x = T.normal(seq * E, 0.0, 1.0, 71)
+    W1 = T.synth_weights("q8_0", 2 * I, E, seed=72, std=0.25)       # 557 056 bytes
+    W2 = T.synth_weights("q4_k", E, I, seed=73)                     # 147 456 bytes
+    Wa = T.synth_weights("q4_k", 600, 1024, seed=74)                # 345 600 bytes
+    Wb = T.synth_weights("q6_k", 500, 1024, seed=75)                # 420 000 bytes
+    xq = T.oracle_quantize(T.normal(1024, 0.0, 1.0, 76), "q8_k")
+    limit = 600 * 1024
+    assert W1.nbytes < limit < W1.nbytes + W2.nbytes and Wa.nbytes + Wb.nbytes > limit
+    L.ckq_weights_set_limit(limit)
+    try:
+        want = T.oracle_fused_mlp(x, W1, None, W2, None, "q4_k", seq, E, E, I, I)
+        for rep in range(2):
+            say("fused MLP under a cache limit, call", rep)
+            got = P.fused_mlp_swiglu_prefill_w1w2_quant(x, W1, None, "q8_0", W2, None, "q4_k", seq, E, E, I, I)
+            assert np.mean(np.abs(got - want) <= 1e-4 * np.abs(want).max()) >= 0.98
+            assert np.abs(got - want).max() <= 5e-3 * np.abs(want).max()
+            nbytes = ctypes.c_size_t(0)
+            L.ckq_weights_resident(ctypes.byref(nbytes))
+            assert nbytes.value <= limit
+        ya, yb = T.oracle_gemv("q4_k", Wa, xq, 600, 1024), T.oracle_gemv("q6_k", Wb, xq, 500, 1024)
+        for rep in range(3):
+            say("alternating GEMVs under a cache limit, round", rep)
+            assert T.norm_err(P.gemv("q4_k", Wa, xq, 600, 1024), ya) <= TOL
+            assert T.norm_err(P.gemv("q6_k", Wb, xq, 500, 1024), yb) <= TOL
+            nbytes = ctypes.c_size_t(0)
+            n = L.ckq_weights_resident(ctypes.byref(nbytes))
+            assert n >= 1 and nbytes.value <= limit
+    finally:
+        L.ckq_weights_set_limit(0)
+        L.ckq_weights_clear()
 
 
 def test_embedding_context_window_beyond_grid_y():

@@ -193,10 +193,8 @@ def test_parallel_union_equals_serial(fmt):
     rows, K = 301, 1024
     W, _, xq = make_case(fmt, rows, K, "rand", 5)
     serial = P.gemv(fmt, W, xq, rows, K)
-    # default ("whole") mode: the union over ith is the serial result, computed by the ith == 0 call
-    y = P.gemv_parallel(fmt, W, xq, rows, K, 8, True)
-    assert np.array_equal(y, serial)
-    ckq.lib().ckq_set_parallel_whole(0)             # "rows" mode: every call computes its own range
+    # default ("rows", the reference's semantics): every call computes exactly its own range
+    ckq.lib().ckq_set_parallel_whole(-1)
     for nth in (1, 3, 8, 64):
         for simd in (False, True):
             say("parallel", fmt, "nth", nth, "simd", simd)
@@ -209,9 +207,10 @@ def test_parallel_union_equals_serial(fmt):
         dr = (rows + 3) // 4
         assert np.all(y[:dr] == -5.0) and np.all(y[2 * dr:] == -5.0)
         assert np.array_equal(y[dr:2 * dr], serial[dr:2 * dr])
-    # "whole" mode: ith 0 computes everything, the rest return
+    # "whole" mode: ith 0 computes everything, the rest return; the union is still the serial result
     ckq.lib().ckq_set_parallel_whole(1)
     try:
+        assert np.array_equal(P.gemv_parallel(fmt, W, xq, rows, K, 8, True), serial)
         y = np.zeros(rows, np.float32)
         fn = getattr(ckq.lib(), P._GEMV[fmt] + "_parallel_simd")
         fn(T.ptr(y), T.ptr(W), T.ptr(xq), rows, K, 0, 8)
@@ -432,6 +431,11 @@ def test_dequant_rows_bit_exact(fmt):
     w, want = G["deq_%s_w" % fmt], G["deq_%s_out" % fmt]
     say("dequant row golden", fmt)
     assert np.array_equal(P.dequant_row(fmt, w, len(want)).view(np.uint32), want.view(np.uint32))
+    if fmt != "q8_0":
+        # the parity scripts' name for the same routine (reference src/ck_parity_api.c:189-197)
+        out = np.zeros(len(want), np.float32)
+        getattr(ckq.lib(), "ck_test_dequant_" + fmt)(T.ptr(w), T.ptr(out), len(want))
+        assert np.array_equal(out.view(np.uint32), want.view(np.uint32))
     # larger, against the oracle
     n = 64 * 1024
     W = T.random_blocks(fmt, n // T.ELEMS[fmt], 91)

@@ -76,6 +76,42 @@ def test_noalloc_entry_point_matches_allocating_one(fmt):
         L.ckq_set_gemm_policy(0)
 
 
+def test_noalloc_entry_point_leaves_device_memory_untouched():
+    """The free device memory the driver reports is the same before and after
+    the calls (operands and output allocated beforehand, ckq_init() done): a
+    K-split matrix-core GEMM and a streaming call, several times each."""
+    import torch
+    L = ckq.lib()
+    assert L.ckq_init() == 0
+    cases = [("q4_k", 64, 1536, 11008), ("q6_k", 128, 2048, 4096), ("q4_k", 3, 500, 1024)]
+    bufs = []
+    for i, (fmt, M, N, K) in enumerate(cases):
+        W = T.synth_weights(fmt, N, K, seed=350 + i)
+        A = T.oracle_quantize(T.normal(M * K, 0.0, 1.0, 360 + i), T.act_fmt(fmt), rows=M)
+        bufs.append((fmt, M, N, K, P.to_device(A), P.to_device(W), torch.zeros(M * N, dtype=torch.float32, device="cuda")))
+    stream = P._stream()
+    torch.cuda.synchronize()
+    L.ckq_set_gemm_policy(1)
+    try:
+        free0 = torch.cuda.mem_get_info()[0]
+        for rep in range(3):
+            for fmt, M, N, K, Ad, Wd, c in bufs:
+                say("no-alloc call, memory check", fmt, M, N, K, rep)
+                assert L.ckq_gemm_nt_noalloc_dev(FMT[fmt], P._dp(Ad), P._dp(Wd), None, P._dp(c), M, N, K, N, stream) == 0
+        torch.cuda.synchronize()
+        free1 = torch.cuda.mem_get_info()[0]
+    finally:
+        L.ckq_set_gemm_policy(0)
+    assert free1 == free0, (free0, free1)
+    for fmt, M, N, K, Ad, Wd, c in bufs:          # and the results are the allocating entry point's
+        L.ckq_set_gemm_policy(1)
+        try:
+            want = P.dev_gemm_nt(fmt, Ad, Wd, None, M, N, K)
+        finally:
+            L.ckq_set_gemm_policy(0)
+        assert np.array_equal(c.view(M, N).cpu().numpy(), want.cpu().numpy())
+
+
 def test_noalloc_entry_point_rejects_what_does_not_fit():
     """Q4_K, M = 128, N = 4096, K = 11008: four K splits of 2 MiB of partial tiles
     each exceed the 4 MiB static scratch: CKQ_ESCRATCH, nothing enqueued, output
