@@ -550,36 +550,49 @@ def main():
                 ("swiglu_q8_k", g_[4], u_[4], hq_, 1, 11008, 11008),
                 ("q6_k", hq_, d_[2], None, d_[4], 1, 4096, 11008)])
         sc = H.time_sequence(chains, 64, 5)
+        ab = {}
+        for mode, key in ((0, "unfused_us"), (2, "all_fused_us")):      # A/B against the default (1: fuse where it pays)
+            H.L.ckq_set_fused_producers(mode)
+            try:
+                ab[key] = round(H.time_sequence(chains, 64, 5) * 1e6, 2)
+            finally:
+                H.L.ckq_set_fused_producers(1)
         extras["layer_7b_decode_chain_M1"] = {"us": round(sc * 1e6, 2), "matmul_only_us": round(s * 1e6, 2),
-                                              "producers_us": round((sc - s) * 1e6, 2), "launches": 8,
+                                              "producers_us": round((sc - s) * 1e6, 2), "launches": 7,
                                               "gbs_of_weight_bytes": round(lbytes / sc / 1e9, 1),
-                                              "note": "norm->Q8_K, Q+K+V, Q8_K, O, norm->Q8_K, gate+up, SwiGLU->Q8_K, down in one C call"}
-        # the same chain with the plain quantizer step folded into its consumer (the O
-        # projection quantizes the attention output while it stages it): seven launches
-        fused = []
-        for ch in chains:
-            fused.append(ch[:4] + [("q4_k+f32q", ch[4][1], ch[5][2], None, ch[5][4], 1, 4096, 4096)] + ch[6:])
-        sf = H.time_sequence(fused, 64, 5)
-        extras["layer_7b_decode_chain_M1"]["quantizer_in_consumer_us"] = round(sf * 1e6, 2)
-        del layers, keep, chains, fused
+                                              "unfused_us": ab["unfused_us"], "all_fused_us": ab["all_fused_us"],
+                                              "expired_waits": int(H.L.ckq_fused_producer_timeouts(P._stream())),
+                                              "note": "norm->Q8_K | Q+K+V | Q8_K + O (one launch: the quantizer rides at the front "
+                                                      "of the O projection's grid) | norm->Q8_K | gate+up | SwiGLU->Q8_K | down, one C call "
+                                                      "per layer; unfused_us: eight launches; all_fused_us: every producer fused with "
+                                                      "its matmuls (four launches)"}
+        del layers, keep, chains
         torch.cuda.empty_cache()
 
-        # fp32 -> Q8_K as its own launch in front of the GEMV against the same step inside the
-        # GEMV's activation staging (every block of the GEMV then quantizes the row itself)
-        qic = {}
+        # a producer as its own launch in front of the GEMV against the fused launch (producer
+        # blocks at the front of the GEMV's grid; the GEMV blocks stream weights while they run)
+        fpm = {}
         for fmt, r, k in (("q4_k", 4096, 4096), ("q4_k", 11008, 4096), ("q6_k", 4096, 11008)):
             _, cps = H.weight_copies(fmt, r, k, seed=r + k + 7)
             xf = P.to_device(T.normal(k, 0.0, 1.0, seed=51))
+            gk = P.to_device(T.normal(k, 1.0, 0.2, seed=52))
             xq = torch.zeros(T.row_bytes("q8_k", k), dtype=torch.uint8, device="cuda")
             y = torch.zeros(r, dtype=torch.float32, device="cuda")
-            two = H.time_sequence([[("quantize_q8_k", xf, None, xq, 1, k), (fmt, xq, c, None, y, 1, r, k)] for c in cps], 128, 5)
-            one = H.time_sequence([[(fmt + "+f32q", xf, c, None, y, 1, r, k)] for c in cps], 128, 5)
-            alone = H.time_sequence([[(fmt, xq, c, None, y, 1, r, k)] for c in cps], 128, 5)
-            qic["%s_%dx%d" % (fmt, r, k)] = {"quantizer_then_gemv_us": round(two * 1e6, 2), "quantizer_in_gemv_us": round(one * 1e6, 2),
-                                             "gemv_alone_us": round(alone * 1e6, 2)}
+            ent = {"gemv_alone_us": round(H.time_sequence([[(fmt, xq, c, None, y, 1, r, k)] for c in cps], 128, 5) * 1e6, 2)}
+            for pname, pstep in (("quantize", ("quantize_q8_k", xf, None, xq, 1, k)),
+                                 ("rmsnorm", ("rmsnorm_q8_k", xf, gk, xq, 1, k, k, 1e-5))):
+                seqs = [[pstep, (fmt, xq, c, None, y, 1, r, k)] for c in cps]
+                H.L.ckq_set_fused_producers(2)
+                ent[pname + "_fused_us"] = round(H.time_sequence(seqs, 128, 5) * 1e6, 2)
+                H.L.ckq_set_fused_producers(0)
+                try:
+                    ent[pname + "_then_gemv_us"] = round(H.time_sequence(seqs, 128, 5) * 1e6, 2)
+                finally:
+                    H.L.ckq_set_fused_producers(1)
+            fpm["%s_%dx%d" % (fmt, r, k)] = ent
             del cps
             torch.cuda.empty_cache()
-        extras["quantizer_in_consumer_M1"] = qic
+        extras["fused_producer_M1"] = fpm
 
         # small-model batched decode (Qwen2-0.5B-like: hidden 896 padded to K=1024, Q5_K
         # projections, Q8_0 LM head 151936x896), M tokens per step

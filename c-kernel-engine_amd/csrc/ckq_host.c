@@ -28,6 +28,7 @@
 
 #include "ckernel_quant_hip.h"
 #include "ckq_launch.h"
+#include "ckq_pure.h"
 
 /* ------------------------------------------------------------------------ */
 /* State                                                                     */
@@ -188,16 +189,32 @@ int ckq_synchronize(void)
     return rc;
 }
 
+/* A host-pointer call classifies its operands (x, W, y) on every call, and the
+ * same buffers come back token after token.  Addresses the runtime has
+ * reported as plain host memory are remembered (a small direct-mapped table),
+ * so the steady state asks the runtime nothing.  Only "host" is remembered,
+ * never "device": should an address change hands, the stale answer makes the
+ * CPU copy from it (at worst a host fault), never a kernel dereference it.
+ * ckq_weights_clear() and ckq_weights_invalidate() empty the table. */
+enum { PTR_CACHE = 64 };
+static const void *g_host_ptr[PTR_CACHE];
+static void ptr_cache_clear(void) { memset(g_host_ptr, 0, sizeof g_host_ptr); }
+
 static int is_device_ptr(const void *p)
 {
+    const size_t slot = ((uintptr_t)p >> 6) % PTR_CACHE;
+    if (p && g_host_ptr[slot] == p) return 0;
     hipPointerAttribute_t at;
     memset(&at, 0, sizeof(at));
     hipError_t e = hipPointerGetAttributes(&at, p);
     if (e != hipSuccess) {
         (void)hipGetLastError(); /* plain host memory: clear the sticky error */
+        g_host_ptr[slot] = p;
         return 0;
     }
-    return at.type == hipMemoryTypeDevice || at.type == hipMemoryTypeManaged;
+    if (at.type == hipMemoryTypeDevice || at.type == hipMemoryTypeManaged) return 1;
+    if (at.type == hipMemoryTypeUnregistered) g_host_ptr[slot] = p;
+    return 0;
 }
 
 static int buf_reserve(int which, size_t bytes, void **out)
@@ -298,21 +315,7 @@ static int stage_out_sync(int which, void *dst, size_t dst_pitch, size_t src_pit
 /* Weight residency                                                          */
 /* ------------------------------------------------------------------------ */
 
-static uint64_t fingerprint(const void *p, size_t bytes)
-{
-    /* FNV-1a over 64 samples of 64 bytes spread across the matrix. */
-    const uint8_t *b = (const uint8_t *)p;
-    uint64_t h = 0xcbf29ce484222325ull ^ bytes;
-    const size_t chunk = 64, n = 64;
-    const size_t step = bytes > chunk * n ? (bytes - chunk) / (n - 1) : chunk;
-    for (size_t i = 0; i < n; ++i) {
-        size_t off = i * step;
-        if (off >= bytes) break;
-        size_t len = bytes - off < chunk ? bytes - off : chunk;
-        for (size_t j = 0; j < len; ++j) h = (h ^ b[off + j]) * 0x100000001b3ull;
-    }
-    return h;
-}
+static uint64_t fingerprint(const void *p, size_t bytes) { return ckq_fingerprint(p, bytes); }
 
 /* The table of unpinned entries is bounded: beyond CACHE_MAX_ENTRIES entries
  * or g_cache_max_bytes bytes (CKQ_WEIGHT_CACHE_MB, default 64 GiB) the least
@@ -500,28 +503,13 @@ int ckq_weights_register_manifest(const void *base, const char *manifest_path)
     if (!base || !manifest_path) return CKQ_EINVAL;
     FILE *mf = fopen(manifest_path, "r");
     if (!mf) return CKQ_EINVAL;
-    static const char *const quant[] = {"q4_k", "q4k", "q5_k", "q5k", "q6_k", "q6k", "q8_0", "q80", "q5_0", "q50"};
     char line[4096];
     int n = 0, rc = 0, inited = 0;
     while (rc == 0 && fgets(line, sizeof line, mf)) {
-        char *p = line;
-        while (*p == ' ' || *p == '\t') ++p;
-        if (*p == '#' || *p == '\n' || *p == '\r' || *p == 0) continue;
-        char *f[5];
-        int nf = 0;
-        for (char *q = p; nf < 5; ++nf) {
-            f[nf] = q;
-            char *bar = strchr(q, '|');
-            if (!bar) { ++nf; break; }
-            *bar = 0;
-            q = bar + 1;
-        }
-        if (nf < 5) { rc = CKQ_EINVAL; break; }        /* malformed line */
-        int is_quant = 0;
-        for (size_t i = 0; i < sizeof quant / sizeof quant[0]; ++i) is_quant |= strcasecmp(f[1], quant[i]) == 0;
-        if (!is_quant) continue;
-        const unsigned long long size = strtoull(f[3], NULL, 0), off = strtoull(f[4], NULL, 0);
-        if (size == 0) continue;
+        unsigned long long size = 0, off = 0;
+        const int kind = ckq_manifest_parse_line(line, &size, &off);
+        if (kind < 0) { rc = CKQ_EINVAL; break; }      /* malformed line */
+        if (kind == 0) continue;
         pthread_mutex_lock(&g_mu);
         if (!inited) { rc = init_locked(); inited = 1; }
         if (rc == 0) rc = register_locked((const uint8_t *)base + off, (size_t)size);
@@ -561,6 +549,7 @@ static void drop_entry(size_t i)
 void ckq_weights_invalidate(const void *W)
 {
     pthread_mutex_lock(&g_mu);
+    ptr_cache_clear();
     for (size_t i = 0; i < g_nw;) {
         if (g_w[i].host == W) drop_entry(i);
         else ++i;
@@ -571,6 +560,7 @@ void ckq_weights_invalidate(const void *W)
 void ckq_weights_clear(void)
 {
     pthread_mutex_lock(&g_mu);
+    ptr_cache_clear();
     while (g_nw) drop_entry(g_nw - 1);
     pthread_mutex_unlock(&g_mu);
 }
@@ -611,13 +601,12 @@ void ckq_set_parallel_whole(int enabled)
 /* Shapes                                                                    */
 /* ------------------------------------------------------------------------ */
 
-static int fmt_block_elems(int fmt) { fmt &= ~CKQ_ACT_F32_QUANT; return (fmt == CKQ_FMT_Q8_0 || fmt == CKQ_FMT_Q5_0 || fmt == CKQ_KERNEL_Q80_F32) ? 32 : 256; }
+static int fmt_block_elems(int fmt) { return (fmt == CKQ_FMT_Q8_0 || fmt == CKQ_FMT_Q5_0 || fmt == CKQ_KERNEL_Q80_F32) ? 32 : 256; }
 
 static int is_f32act(int fmt) { return fmt == CKQ_KERNEL_Q80_F32 || fmt == CKQ_KERNEL_Q4K_F32 || fmt == CKQ_KERNEL_Q6K_F32; }
 
 static int weight_fmt(int fmt)
 {
-    fmt &= ~CKQ_ACT_F32_QUANT;
     return fmt == CKQ_KERNEL_Q80_F32 ? CKQ_FMT_Q8_0 : fmt == CKQ_KERNEL_Q4K_F32 ? CKQ_FMT_Q4_K
          : fmt == CKQ_KERNEL_Q6K_F32 ? CKQ_FMT_Q6_K : fmt;
 }
@@ -629,7 +618,7 @@ static size_t weight_row_bytes(int fmt, int K)
 
 static size_t act_row_bytes(int fmt, int K)
 {
-    if (is_f32act(fmt) || (fmt & CKQ_ACT_F32_QUANT)) return (size_t)K * 4;
+    if (is_f32act(fmt)) return (size_t)K * 4;
     if (fmt == CKQ_FMT_Q8_0 || fmt == CKQ_FMT_Q5_0) return ckq_row_bytes(CKQ_FMT_Q8_0, K);
     return ckq_row_bytes(CKQ_FMT_Q8_K, K);
 }
@@ -655,17 +644,27 @@ static void matmul_locked(int fmt, const void *A, const void *B, const float *bi
         const int c_on_dev = is_device_ptr(C);
         float *dC = C;
         long   ld = ldc;
+        void  *ypin = NULL;      /* small results are written by the kernel straight into the pinned twin */
         if (!c_on_dev) {
             void *t;
             ld = row1 - row0; /* compact staging: only the computed rows */
-            if (buf_reserve(BUF_Y, (size_t)ntok * (size_t)ld * sizeof(float), &t)) break;
+            const size_t ybytes = (size_t)ntok * (size_t)ld * sizeof(float);
+            if (ybytes <= PIN_MAX_BYTES) {
+                if (pin_reserve(BUF_Y, round16(ybytes), &ypin)) break;
+                t = g_pin[BUF_Y].dev;
+            } else if (buf_reserve(BUF_Y, ybytes, &t)) break;
             /* the kernel indexes with absolute rows: bias the base by row0 in integer
              * arithmetic (a pointer in front of its allocation must not be formed) */
             dC = (float *)((uintptr_t)t - (uintptr_t)row0 * sizeof(float));
         }
         int rc = ckq_launch_gemv(fmt, dC, dB, dA, (const float *)dbias, nrows, K, ntok, ld, row0, row1, NULL, g_stream);
         if (rc) { fail(rc, "ckq_launch_gemv"); break; }
-        if (!c_on_dev) {
+        if (ypin) {
+            hipError_t e = hipStreamSynchronize(g_stream);
+            if (e != hipSuccess) { fail((int)e, "hipStreamSynchronize"); break; }
+            const size_t w = (size_t)(row1 - row0) * sizeof(float);
+            for (int t = 0; t < ntok; ++t) memcpy(C + (size_t)t * ldc + row0, (const uint8_t *)ypin + (size_t)t * w, w);
+        } else if (!c_on_dev) {
             if (stage_out_sync(BUF_Y, C + row0, (size_t)ldc * sizeof(float), (size_t)ld * sizeof(float),
                                (size_t)(row1 - row0) * sizeof(float), (size_t)ntok)) break;
         } else {
@@ -693,17 +692,7 @@ static void host_matmul(int fmt, const void *A, const void *B, const float *bias
 /* Row range of thread ith of nth (reference: gemm_kernels_q4k_q8k.c:226-231). */
 static int split_rows(int M, int ith, int nth, int *r0, int *r1)
 {
-    if (ith < 0 || nth <= 0 || ith >= nth) return 0;
-    if (__atomic_load_n(&g_parallel_whole, __ATOMIC_RELAXED)) {
-        if (ith != 0) return 0;
-        *r0 = 0;
-        *r1 = M;
-        return 1;
-    }
-    const int dr = (M + nth - 1) / nth;
-    *r0 = dr * ith;
-    *r1 = (*r0 + dr < M) ? *r0 + dr : M;
-    return *r0 < M;
+    return ckq_split_rows(M, ith, nth, __atomic_load_n(&g_parallel_whole, __ATOMIC_RELAXED), r0, r1);
 }
 
 static void host_gemv_split(int fmt, float *y, const void *W, const void *x, int M, int K, int ith, int nth)
@@ -1196,10 +1185,8 @@ int ckq_quantize_q8_0_dev(const float *x, void *y, int num_rows, int k, void *st
 int ckq_gemm_nt_dev(int fmt, const void *A_q8, const void *B, const float *bias, float *C,
                     int M, int N, int K, long ldc, void *stream)
 {
-    const int wf = fmt & ~CKQ_ACT_F32_QUANT;
-    if (wf != CKQ_FMT_Q4_K && wf != CKQ_FMT_Q5_K && wf != CKQ_FMT_Q6_K && wf != CKQ_FMT_Q8_0 && wf != CKQ_FMT_Q5_0)
+    if (fmt != CKQ_FMT_Q4_K && fmt != CKQ_FMT_Q5_K && fmt != CKQ_FMT_Q6_K && fmt != CKQ_FMT_Q8_0 && fmt != CKQ_FMT_Q5_0)
         return CKQ_EFORMAT;
-    if (fmt != wf && (wf == CKQ_FMT_Q8_0 || wf == CKQ_FMT_Q5_0)) return CKQ_EFORMAT;
     return ckq_launch_gemv(fmt, C, B, A_q8, bias, N, K, M, ldc, 0, N, NULL, stream);
 }
 
@@ -1256,11 +1243,7 @@ int ckq_gemm_nt_f32act_dev(int fmt, const float *A, const void *B, const float *
     return ckq_launch_gemv(k, C, B, A, bias, N, K, M, ldc, 0, N, NULL, stream);
 }
 
-static int ranges_overlap(const void *a, size_t na, const void *b, size_t nb)
-{
-    const uintptr_t a0 = (uintptr_t)a, b0 = (uintptr_t)b;
-    return a0 < b0 + nb && b0 < a0 + na;
-}
+static int ranges_overlap(const void *a, size_t na, const void *b, size_t nb) { return ckq_ranges_overlap(a, na, b, nb); }
 
 /* Entries i and j of a sequence can share a launch when they have one format,
  * input width and token count (their row counts may differ: K and V are
@@ -1299,6 +1282,91 @@ static int issue_producer(const ckq_matmul_op *o, void *stream)
     }
 }
 
+/* 0 = never, 1 = where it was measured to pay (below), 2 = wherever a fused form exists */
+static int g_fuse_producers = 1;
+void ckq_set_fused_producers(int mode) { __atomic_store_n(&g_fuse_producers, mode < 0 || mode > 2 ? 1 : mode, __ATOMIC_RELAXED); }
+/* Weight bytes of the matmuls up to which a fused launch beats two launches.
+ * Measured at one token (us; producer + matmul as two launches -> fused):
+ * fp32 -> Q8_K or SiLU*up -> Q8_K in front of Q4_K 1024x4096 11.0 -> 8.7,
+ * 4096x4096 8.1 -> 6.8; 11008x4096 8.2 -> 10.2 and Q6_K 4096x11008 11.8 -> 13.6
+ * lose: the handover (the producers' write-back, the counter, the first
+ * poll) is four round trips through memory, which cost what a launch
+ * boundary costs once the matmul is long enough to hide the next dispatch.
+ * RMSNorm in front loses at every size (4096x4096 8.8 -> 11.2): as a
+ * four-wave producer block its serial chains are slower than in the
+ * sixteen-wave kernel. */
+enum { FUSE_MAX_WEIGHT_BYTES = 12 << 20 };
+
+int ckq_fused_producer_timeouts(void *stream)
+{
+    unsigned n = 0;
+    const int rc = ckq_launch_pro_timeouts(stream, &n);
+    return rc ? (rc > 0 ? -rc : rc) : (int)n;
+}
+
+/* Number of consecutive matmul entries from ops[i] on that can share a launch (1..4). */
+static int group_length(const ckq_matmul_op *ops, int i, int nops)
+{
+    enum { GROUP_MAX = 4 };
+    const ckq_matmul_op *o = &ops[i];
+    int n = 1;
+    const int groupable = o->A_q8 && o->B && o->C && o->M >= 1 && o->M <= 8 && o->N > 0 && o->K > 0 &&
+                          o->ldc >= o->N && !is_f32act(o->fmt) && o->K % fmt_block_elems(o->fmt) == 0;
+    while (groupable && n < GROUP_MAX && i + n < nops) {
+        if (ops[i + n].fmt >= CKQ_STEP_QUANTIZE_Q8_K && ops[i + n].fmt <= CKQ_STEP_SWIGLU_Q8_K) break;
+        int ok = 1;
+        for (int j = 0; j < n && ok; ++j) ok = ops_independent(&ops[i + j], &ops[i + n]);
+        if (!ok) break;
+        ++n;
+    }
+    return n;
+}
+
+/* Producer entry p followed by the n matmul entries m[0..n): one fused launch
+ * when every one of them reads the producer's output and nothing else of the
+ * producer's memory is written by them.  Returns CKQ_EUNFUSED when the steps
+ * have to go out one by one. */
+static int issue_fused(const ckq_matmul_op *p, const ckq_matmul_op *m, int n, void *stream)
+{
+    const int mode = __atomic_load_n(&g_fuse_producers, __ATOMIC_RELAXED);
+    if (!mode) return CKQ_EUNFUSED;
+    const int kind = p->fmt == CKQ_STEP_QUANTIZE_Q8_K ? 1 : p->fmt == CKQ_STEP_RMSNORM_Q8_K ? 2
+                   : p->fmt == CKQ_STEP_SWIGLU_Q8_K ? 3 : 0;
+    if (!kind || !p->A_q8 || !p->C || p->M <= 0 || p->K <= 0) return CKQ_EUNFUSED;
+    if (kind != 1 && !p->B) return CKQ_EUNFUSED;
+    const long pld = p->ldc ? p->ldc : p->K;
+    if (pld < p->K) return CKQ_EUNFUSED;
+    const size_t in_bytes = ((size_t)(p->M - 1) * (size_t)pld + (size_t)p->K) * sizeof(float);
+    float *y[4];
+    const void *W[4], *X[4];
+    const float *b[4];
+    int rows[4];
+    long ld[4];
+    if (mode == 1) {
+        size_t wbytes = 0;
+        for (int j = 0; j < n; ++j) wbytes += (size_t)m[j].N * weight_row_bytes(m[j].fmt, m[j].K);
+        if (kind == 2 || wbytes > FUSE_MAX_WEIGHT_BYTES) return CKQ_EUNFUSED;
+    }
+    for (int j = 0; j < n; ++j) {
+        const ckq_matmul_op *q = &m[j];
+        if (q->fmt != m[0].fmt || q->M != p->M || q->K != p->K || q->A_q8 != (const void *)p->C) return CKQ_EUNFUSED;
+        if (!q->B || !q->C || q->N <= 0 || q->ldc < q->N) return CKQ_EUNFUSED;
+        /* the matmuls run while the producer reads its input: they must not write it */
+        const size_t qc = ((size_t)(q->M - 1) * (size_t)q->ldc + (size_t)q->N) * sizeof(float);
+        if (ranges_overlap(q->C, qc, p->A_q8, in_bytes)) return CKQ_EUNFUSED;
+        if (kind != 1 && ranges_overlap(q->C, qc, p->B, kind == 2 ? (size_t)p->K * sizeof(float) : in_bytes)) return CKQ_EUNFUSED;
+        /* the matmul blocks read their weights (and nothing else of the producer's concern) before the
+         * producer has finished: no cache line of its output may be shared with them */
+        const uintptr_t o0 = (uintptr_t)p->C & ~(uintptr_t)127;
+        const size_t ob = (size_t)p->M * act_row_bytes(q->fmt, q->K);
+        const size_t olen = (((uintptr_t)p->C + ob + 127) & ~(uintptr_t)127) - o0;
+        if (ranges_overlap((const void *)o0, olen, q->B, (size_t)q->N * weight_row_bytes(q->fmt, q->K))) return CKQ_EUNFUSED;
+        y[j] = q->C; W[j] = q->B; X[j] = q->A_q8; b[j] = q->bias; rows[j] = q->N; ld[j] = q->ldc;
+    }
+    return ckq_launch_gemv_pro(m[0].fmt, n, y, W, X, b, rows, ld, m[0].K, m[0].M, kind, (const float *)p->A_q8,
+                               (const float *)p->B, p->C, p->M, p->K, pld, p->eps, stream);
+}
+
 int ckq_matmul_sequence_dev(const ckq_matmul_op *ops, int nops, int repeat, void *stream)
 {
     if (!ops || nops <= 0 || repeat <= 0) return CKQ_EINVAL;
@@ -1307,6 +1375,15 @@ int ckq_matmul_sequence_dev(const ckq_matmul_op *ops, int nops, int repeat, void
         for (int i = 0; i < nops;) {
             const ckq_matmul_op *o = &ops[i];
             if (o->fmt >= CKQ_STEP_QUANTIZE_Q8_K && o->fmt <= CKQ_STEP_SWIGLU_Q8_K) {
+                /* a producer and the matmuls right behind it that read its output: one launch,
+                 * the weights stream while the producer runs */
+                if (i + 1 < nops && !(ops[i + 1].fmt >= CKQ_STEP_QUANTIZE_Q8_K && ops[i + 1].fmt <= CKQ_STEP_SWIGLU_Q8_K) &&
+                    ops[i + 1].M <= 8) {
+                    const int n = group_length(ops, i + 1, nops);
+                    const int rc = issue_fused(o, &ops[i + 1], n, stream);
+                    if (rc == 0) { i += 1 + n; continue; }
+                    if (rc != CKQ_EUNFUSED) return rc;
+                }
                 const int rc = issue_producer(o, stream);
                 if (rc) return rc;
                 ++i;
@@ -1314,15 +1391,7 @@ int ckq_matmul_sequence_dev(const ckq_matmul_op *ops, int nops, int repeat, void
             }
             /* consecutive entries of one shape that do not depend on each other
              * (Q/K/V, gate/up) go out as one launch */
-            int n = 1;
-            const int groupable = o->A_q8 && o->B && o->C && o->M >= 1 && o->M <= 8 && o->N > 0 && o->K > 0 &&
-                                  o->ldc >= o->N && !is_f32act(o->fmt) && o->K % fmt_block_elems(o->fmt) == 0;
-            while (groupable && n < GROUP_MAX && i + n < nops) {
-                int ok = 1;
-                for (int j = 0; j < n && ok; ++j) ok = ops_independent(&ops[i + j], &ops[i + n]);
-                if (!ok) break;
-                ++n;
-            }
+            const int n = group_length(ops, i, nops);
             int rc;
             if (n > 1) {
                 float *y[GROUP_MAX];

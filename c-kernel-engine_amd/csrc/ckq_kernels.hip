@@ -17,10 +17,13 @@
  */
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include "ckq_blocks.h"
 #include "ckq_formats.hpp"
+#include "ckq_producers.hpp"
 #include "ckq_launch.h"
+#include "ckq_pure.h"
 
 /* ========================================================================= */
 /* GEMV                                                                       */
@@ -91,22 +94,9 @@ __global__ void __launch_bounds__(256) gemm_splitk_reduce_kernel(float *__restri
 static std::recursive_mutex g_split_mu;
 std::recursive_mutex &gemm_split_mutex() { return g_split_mu; }
 
-/* Slot bookkeeping of gemm_workspace, free of HIP calls so that it can be tested on
- * the CPU: the slot whose key equals `key`, else the first free one (key 0), else the
- * least recently used one (smallest last_use), which the caller recycles. */
-extern "C" int ckq_workspace_pick(const uint64_t *keys, const uint64_t *last_use, int n, uint64_t key)
-{
-    int free_slot = -1, lru = 0;
-    for (int i = 0; i < n; ++i) {
-        if (keys[i] == key) return i;
-        if (keys[i] == 0 && free_slot < 0) free_slot = i;
-        if (last_use[i] < last_use[lru]) lru = i;
-    }
-    return free_slot >= 0 ? free_slot : lru;
-}
-
 /* Grow-only device scratch per (device, stream, kind); see ckq_gemm_common.hpp.
- * kind 0: partial tiles of a K split; kind 1: weights rewritten for another kernel.
+ * kind 0: partial tiles of a K split; kind 1: weights rewritten for another kernel;
+ * kind 2: the completion counter of fused producer launches (pro_counter below).
  * When all slots are taken the least recently used one is recycled: the device is
  * synchronised (its stream may no longer exist), its buffer freed.  A destroyed
  * stream whose handle value is given out again finds the old stream's slot: harmless,
@@ -114,17 +104,27 @@ extern "C" int ckq_workspace_pick(const uint64_t *keys, const uint64_t *last_use
  * ckq_launch_release_stream gives a stream's slots back explicitly. */
 namespace {
 constexpr int WS_SLOTS = 32;
-struct WsSlot { hipStream_t s; int kind, dev; void *p; size_t cap; };
+struct WsSlot { hipStream_t s; int kind, dev; void *p; size_t cap; unsigned epoch; };
 WsSlot   g_ws[WS_SLOTS];
 uint64_t g_ws_key[WS_SLOTS], g_ws_use[WS_SLOTS], g_ws_clock = 0;
 uint64_t ws_key(int dev, hipStream_t s, int kind)
 {
-    /* lossless for user-space handles (below 2^56), 32 devices and two kinds; never 0 */
-    return (1ull << 63) | ((uint64_t)(kind & 1) << 61) | ((uint64_t)(dev & 31) << 56) | ((uint64_t)(uintptr_t)s & ((1ull << 56) - 1));
+    /* lossless for user-space handles (below 2^56), 32 devices and four kinds; never 0 */
+    return (1ull << 63) | ((uint64_t)(kind & 3) << 61) | ((uint64_t)(dev & 31) << 56) | ((uint64_t)(uintptr_t)s & ((1ull << 56) - 1));
 }
 }
 
+static int workspace_slot(int kind, hipStream_t s, size_t bytes, WsSlot **out, bool *fresh);
+
 int gemm_workspace(int kind, hipStream_t s, size_t bytes, float **out)
+{
+    WsSlot *sl = nullptr;
+    const int rc = workspace_slot(kind, s, bytes, &sl, nullptr);
+    if (rc == 0) *out = (float *)sl->p;
+    return rc;
+}
+
+static int workspace_slot(int kind, hipStream_t s, size_t bytes, WsSlot **out, bool *fresh)
 {
     std::lock_guard<std::recursive_mutex> lock(g_split_mu);
     int dev = 0;
@@ -143,9 +143,10 @@ int gemm_workspace(int kind, hipStream_t s, size_t bytes, float **out)
             if (e != hipSuccess) return (int)e;
         }
         g_ws_key[i] = key;
-        *sl = {s, kind, dev, nullptr, 0};
+        *sl = {s, kind, dev, nullptr, 0, 0u};
     }
     g_ws_use[i] = ++g_ws_clock;
+    if (fresh) *fresh = sl->cap < bytes;
     if (sl->cap < bytes) {
         if (sl->p) {
             e = hipStreamSynchronize(s);
@@ -158,7 +159,7 @@ int gemm_workspace(int kind, hipStream_t s, size_t bytes, float **out)
         if (e != hipSuccess) return (int)e;
         sl->cap = cap;
     }
-    *out = (float *)sl->p;
+    *out = sl;
     return 0;
 }
 
@@ -193,14 +194,6 @@ int gemm_launch_reduce(float *C, long ldc, const float *part, const float *bias,
     return (int)hipGetLastError();
 }
 
-/* Token range [*first, *first + *count) of chunk c of a launch chunked over
- * gridDim.y in pieces of `per` tokens.  Host arithmetic only. */
-extern "C" void ckq_grid_chunk(long total, long per, long c, long *first, long *count)
-{
-    *first = c * per;
-    *count = total - *first < per ? total - *first : per;
-    if (*count < 0) *count = 0;
-}
 
 
 /* Q5_0 block -> Q8_0 block: the scale is kept, the 32 values become int8
@@ -311,7 +304,7 @@ extern "C" int ckq_launch_gemv_group(int fmt, int n, float *const *y, const void
     /* Every grouped kernel stages its token tile in LDS.  A tile that does not
      * fit (the tile is the token count rounded up to 1, 2, 4 or 8 rows of
      * activations) goes out as n separate launches, which stream it instead. */
-    if (n == 1 || !group_tile_fits_lds(fmt & ~CKQ_ACT_F32_QUANT, K, ntok)) {
+    if (n == 1 || !group_tile_fits_lds(fmt, K, ntok)) {
         if (subdots) return CKQ_EINVAL;
         for (int i = 0; i < n; ++i) {
             const int rc = ckq_launch_gemv(fmt, y[i], W[i], X[i], bias ? bias[i] : nullptr, rows[i], K, ntok, ldys[i], 0,
@@ -335,6 +328,102 @@ extern "C" int ckq_launch_gemv_group(int fmt, int n, float *const *y, const void
     return launch_gemv_args(fmt, a, grp, K, stream);
 }
 
+/* The completion counter of fused producer launches on `s`: two dwords of
+ * device memory per (device, stream), zeroed when created, and the value
+ * flag[0] will have once everything enqueued so far has run.  The caller holds
+ * g_split_mu from here until its launch is enqueued and then adds the
+ * launch's producer blocks to *epoch. */
+static int pro_counter(hipStream_t s, unsigned **flag, unsigned **epoch)
+{
+    WsSlot *sl = nullptr;
+    bool fresh = false;
+    int rc = workspace_slot(2, s, 64, &sl, &fresh);
+    if (rc) return rc;
+    if (fresh) {
+        hipError_t e = hipMemsetAsync(sl->p, 0, 64, s);
+        if (e != hipSuccess) return (int)e;
+        sl->epoch = 0;
+    }
+    *flag = (unsigned *)sl->p;
+    *epoch = &sl->epoch;
+    return 0;
+}
+
+static std::atomic<int> g_pro_spin_limit{1 << 20};     /* polls of ~0.5 us each before a matmul block gives up waiting */
+extern "C" void ckq_launch_set_pro_spin_limit(int polls) { g_pro_spin_limit.store(polls > 0 ? polls : 1 << 20); }
+
+/* Expired waits recorded by fused launches on `stream` so far (synchronises the stream). */
+extern "C" int ckq_launch_pro_timeouts(void *stream, unsigned *count)
+{
+    std::lock_guard<std::recursive_mutex> lock(g_split_mu);
+    unsigned *flag, *epoch;
+    int rc = pro_counter((hipStream_t)stream, &flag, &epoch);
+    if (rc) return rc;
+    hipError_t e = hipMemcpyAsync(count, flag + 1, sizeof(unsigned), hipMemcpyDeviceToHost, (hipStream_t)stream);
+    if (e == hipSuccess) e = hipStreamSynchronize((hipStream_t)stream);
+    return (int)e;
+}
+
+/* A producer (CKQ_PRO_*: fp32 rows -> Q8_K blocks at `dst`) and the n (1..4)
+ * matmuls that read `dst` as ONE launch: producer blocks in front, the matmul
+ * blocks start streaming their weights at once and wait for the producer's
+ * count before they touch the activations.  Up to eight tokens, Q4_K / Q5_K /
+ * Q6_K weights.  Returns CKQ_EUNFUSED, with nothing enqueued, when this
+ * combination has no fused form (the caller then issues the steps one by one):
+ * other formats, a token tile or a row too large for LDS, a stream that is
+ * being captured (the counter's expected value is baked into the launch, so a
+ * replay would not wait). */
+extern "C" int ckq_launch_gemv_pro(int fmt, int n, float *const *y, const void *const *W, const void *const *X,
+                                   const float *const *bias, const int *rows, const long *ldys, int K, int ntok,
+                                   int kind, const float *src, const float *src2, void *dst, int pro_rows, int pro_k,
+                                   long pro_ld, float eps, void *stream)
+{
+    if (n < 1 || n > CKQ_GROUP_MAX || !y || !W || !X || !rows || !ldys || K <= 0 || ntok < 1) return CKQ_EINVAL;
+    if (!src || !dst || pro_rows <= 0 || pro_k <= 0 || pro_ld < pro_k) return CKQ_EINVAL;
+    if (fmt != CKQ_FMT_Q4_K && fmt != CKQ_FMT_Q5_K && fmt != CKQ_FMT_Q6_K) return CKQ_EUNFUSED;
+    if (ntok > CKQ_STREAM_TOKENS || K % 256 || pro_k % 256) return CKQ_EUNFUSED;
+    if (kind != CKQ_PRO_QUANT_Q8K && kind != CKQ_PRO_RMSNORM_Q8K && kind != CKQ_PRO_SWIGLU_Q8K) return CKQ_EINVAL;
+    if (kind != CKQ_PRO_QUANT_Q8K && !src2) return CKQ_EINVAL;
+    if (pro_ld % 4 || ((uintptr_t)src | (uintptr_t)src2) % 16) return CKQ_EUNFUSED;
+    if (!group_tile_fits_lds(fmt, K, ntok)) return CKQ_EUNFUSED;
+    if (kind == CKQ_PRO_RMSNORM_Q8K && (size_t)pro_k * 4 + 32 > 65536) return CKQ_EUNFUSED;
+    int nrows = 0;
+    for (int i = 0; i < n; ++i) {
+        if (rows[i] <= 0 || !W[i] || !X[i] || !y[i] || ldys[i] < rows[i] || ldys[i] > 0x7fffffff) return CKQ_EINVAL;
+        if (rows[i] > nrows) nrows = rows[i];
+    }
+    hipStream_t s = (hipStream_t)stream;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &cap) != hipSuccess) { (void)hipGetLastError(); return CKQ_EUNFUSED; }
+    if (cap != hipStreamCaptureStatusNone) return CKQ_EUNFUSED;
+
+    std::lock_guard<std::recursive_mutex> lock(g_split_mu);
+    unsigned *flag, *epoch;
+    int rc = pro_counter(s, &flag, &epoch);
+    if (rc) return rc;
+    GemvPro pro = {};
+    pro.src = src; pro.src2 = src2; pro.dst = (uint8_t *)dst; pro.flag = flag; pro.target = *epoch;
+    pro.spin_limit = g_pro_spin_limit.load(std::memory_order_relaxed);
+    { static const int nap = getenv("CKQ_PRO_NAP") ? atoi(getenv("CKQ_PRO_NAP")) : 1; pro.nap = nap > 0 ? nap : 1; }
+    pro.kind = kind; pro.rows = pro_rows; pro.k = pro_k; pro.ld = pro_ld; pro.eps = eps;
+    int pro_blocks = 0;
+    GemvArgs a = {};
+    GemvGroup grp = k_no_group;
+    a.y = y[0]; a.W = (const uint8_t *)W[0]; a.X = (const uint8_t *)X[0]; a.bias = bias ? bias[0] : nullptr; a.sub = nullptr;
+    a.nrows = nrows; a.ntok = ntok; a.row0 = 0; a.row1 = rows[0]; a.ldy = ldys[0];
+    a.pro = &pro; a.pro_blocks = &pro_blocks;
+    for (int i = 1; i < n; ++i) {
+        grp.y[i - 1] = y[i]; grp.W[i - 1] = (const uint8_t *)W[i]; grp.X[i - 1] = (const uint8_t *)X[i];
+        grp.bias[i - 1] = bias ? bias[i] : nullptr;
+        grp.nrows[i - 1] = rows[i];
+        grp.ldy[i - 1] = (int)ldys[i];
+    }
+    grp.n = n;
+    rc = launch_gemv_args(fmt, a, grp, K, stream);
+    if (rc == 0) *epoch += (unsigned)pro_blocks;
+    return rc;
+}
+
 static int launch_gemv_args(int fmt_flags, GemvArgs &a, const GemvGroup &grp, int K, void *stream, const GemmOpts &opts)
 {
     int fmt = fmt_flags;
@@ -345,12 +434,9 @@ static int launch_gemv_args(int fmt_flags, GemvArgs &a, const GemvGroup &grp, in
     const long ldy = a.ldy;
     hipStream_t s = (hipStream_t)stream;
     const bool dump = a.sub != nullptr;
-    const bool xq = (fmt & CKQ_ACT_F32_QUANT) != 0;
-    fmt &= ~CKQ_ACT_F32_QUANT;
-    if (xq && (dump || ntok > CKQ_STREAM_TOKENS || (fmt != CKQ_FMT_Q4_K && fmt != CKQ_FMT_Q5_K && fmt != CKQ_FMT_Q6_K)))
+    if (a.pro && (dump || ntok > CKQ_STREAM_TOKENS || (fmt != CKQ_FMT_Q4_K && fmt != CKQ_FMT_Q5_K && fmt != CKQ_FMT_Q6_K)))
         return CKQ_EINVAL;
-    a.xq = xq;
-    const bool whole = !xq && !dump && grp.n == 1 && row0 == 0 && row1 == nrows;   /* what a matrix-core GEMM can take */
+    const bool whole = !a.pro && !dump && grp.n == 1 && row0 == 0 && row1 == nrows;   /* what a matrix-core GEMM can take */
     switch (fmt) {
     case CKQ_FMT_Q4_K:
         if (K % 256) return CKQ_ESHAPE;
@@ -496,18 +582,6 @@ extern "C" int ckq_launch_gemm_block_sums(int fmt, const void *A, const void *B,
 /* Activation quantizers                                                      */
 /* ========================================================================= */
 
-/* SiLU(g) * u as the reference's fused prefill MLP forms it
- * (fused/prefill_fused_gemm.c:904-906, 1034-1040): g / (1 + expf(-g)), then
- * the product, each operation rounded to fp32.  exp is evaluated in double
- * and rounded once, which agrees with a correctly rounded expf. */
-__device__ __forceinline__ float swiglu_value(float g, float u)
-{
-#pragma clang fp contract(off)
-    const float e = (float)exp(-(double)g);
-    const float s = g / (1.0f + e);
-    return s * u;
-}
-
 /* fp32 -> Q8_K, one wave per 256-element block, lane l owns elements 4l..4l+3
  * (q8k_quantize_block holds the reference's rules).  SWIGLU: the quantizer's
  * input is SiLU(x) * up instead of x.  Rows of the input are ldx floats apart,
@@ -516,19 +590,9 @@ template <bool SWIGLU>
 __global__ void __launch_bounds__(256) quantize_q8_k_kernel(const float *__restrict__ x, const float *__restrict__ up,
                                                             uint8_t *__restrict__ y, long nblocks, int bpr, long ldx)
 {
-    const int lane = threadIdx.x & 63;
     const long blk = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (blk >= nblocks) return;
-    const long src = (blk / bpr) * ldx + (blk % bpr) * 256;
-    const float4 v = reinterpret_cast<const float4 *>(x + src)[lane];
-    float e[4] = {v.x, v.y, v.z, v.w};
-    if constexpr (SWIGLU) {
-        const float4 w = reinterpret_cast<const float4 *>(up + src)[lane];
-        e[0] = swiglu_value(e[0], w.x); e[1] = swiglu_value(e[1], w.y);
-        e[2] = swiglu_value(e[2], w.z); e[3] = swiglu_value(e[3], w.w);
-    }
-
-    q8k_quantize_block(e, lane, y + blk * 292);
+    pro_quantize_block<SWIGLU>(x, up, y, blk, bpr, ldx, threadIdx.x & 63);
 }
 
 /*
@@ -594,81 +658,19 @@ extern "C" int ckq_launch_quantize_q8_0(const float *x, void *y, int rows, int k
 }
 
 /*
- * Fused producer RMSNorm -> Q8_K, one block per token (reference:
- * src/kernels/fused/rmsnorm_q8_k_fused.c:54-142 as an FMA build compiles it).
- * The sum of squares must be the reference's to the bit, or rstd moves by an
- * ulp and quants flip: eight strided lanes (lane j takes x[8i+j]) each a chain
- * of fused multiply-adds, combined as ((l0+l4)+(l1+l5)) + ((l2+l6)+(l3+l7)).
- * Eight threads walk the chains over the row staged in LDS; every thread then
- * derives the same rstd.  Quantization: n = (x*rstd)*gamma with two roundings,
- * scale from the largest |n| of the block, iscale = -127/max, d = 1/iscale,
- * q = RNE(n*iscale) saturated; one wave per 256-block, lane l owns 4l..4l+3.
+ * Fused producer RMSNorm -> Q8_K, one block of sixteen waves per token (the
+ * arithmetic is rms_row's, ckq_producers.hpp): up to D = 4096 every 256-block of
+ * the row has a wave of its own.
  */
-__global__ void __launch_bounds__(256) rmsnorm_q8_k_fused_kernel(const float *__restrict__ input,
+constexpr int RMS_WAVES = 16;
+__global__ void __launch_bounds__(64 * RMS_WAVES) rmsnorm_q8_k_fused_kernel(const float *__restrict__ input,
                                                                  const float *__restrict__ gamma,
                                                                  uint8_t *__restrict__ y, int d_model, long in_stride,
                                                                  float eps)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    float *xs = reinterpret_cast<float *>(smem);          /* d_model floats, then 8 lane sums */
-    const int tid = threadIdx.x, lane = tid & 63, wave = wave_in_block();
-    const float *x = input + (size_t)blockIdx.x * in_stride;
-    const int D = d_model, nb = D / 256;
-
-    for (int i = tid; i < D / 4; i += 256)
-        reinterpret_cast<float4 *>(xs)[i] = reinterpret_cast<const float4 *>(x)[i];
-    __syncthreads();
-    if (tid < 8) {
-        /* the chain is serial; keep 16 LDS reads in flight ahead of it (D is a multiple of 256) */
-        float acc = 0.0f, cur[16], nxt[16];
-#pragma unroll
-        for (int u = 0; u < 16; ++u) cur[u] = xs[tid + 8 * u];
-        for (int d = 0; d < D; d += 128) {
-            const int dn = d + 128 < D ? d + 128 : d;
-#pragma unroll
-            for (int u = 0; u < 16; ++u) nxt[u] = xs[dn + tid + 8 * u];
-#pragma unroll
-            for (int u = 0; u < 16; ++u) acc = __fmaf_rn(cur[u], cur[u], acc);
-#pragma unroll
-            for (int u = 0; u < 16; ++u) cur[u] = nxt[u];
-        }
-        xs[D + tid] = acc;
-    }
-    __syncthreads();
-    const float s04 = xs[D + 0] + xs[D + 4], s15 = xs[D + 1] + xs[D + 5];
-    const float s26 = xs[D + 2] + xs[D + 6], s37 = xs[D + 3] + xs[D + 7];
-    const float sum_sq = (s04 + s15) + (s26 + s37);
-    /* sqrtf and '/' are the correctly rounded ones (the __fsqrt_rn intrinsic is not) */
-    const float rstd = 1.0f / sqrtf(sum_sq / (float)D + eps);
-
-    for (int b = wave; b < nb; b += 4) {
-        const float4 xv = reinterpret_cast<const float4 *>(xs + 256 * b)[lane];
-        const float4 gv = reinterpret_cast<const float4 *>(gamma + 256 * b)[lane];
-        const float e[4] = {__fmul_rn(__fmul_rn(xv.x, rstd), gv.x), __fmul_rn(__fmul_rn(xv.y, rstd), gv.y),
-                            __fmul_rn(__fmul_rn(xv.z, rstd), gv.z), __fmul_rn(__fmul_rn(xv.w, rstd), gv.w)};
-        float amax = fmaxf(fmaxf(fabsf(e[0]), fabsf(e[1])), fmaxf(fabsf(e[2]), fabsf(e[3])));
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
-
-        uint8_t *out = y + ((size_t)blockIdx.x * nb + b) * 292;
-        if (amax == 0.0f) {
-            reinterpret_cast<u32 *>(out)[lane] = 0;
-            if (lane < 9) reinterpret_cast<u32 *>(out)[64 + lane] = 0;
-            continue;
-        }
-        const float iscale = __fdiv_rn(-127.0f, amax);
-        int q[4], sum = 0;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            q[i] = rne_sat_i8(__fmul_rn(e[i], iscale));
-            sum += q[i];
-        }
-        reinterpret_cast<u32 *>(out + 4)[lane] =
-            (u32)(q[0] & 0xff) | ((u32)(q[1] & 0xff) << 8) | ((u32)(q[2] & 0xff) << 16) | ((u32)(q[3] & 0xff) << 24);
-        sum = group_sum<4>(sum);
-        if ((lane & 3) == 3) reinterpret_cast<int16_t *>(out + 260)[lane >> 2] = (int16_t)sum;
-        if (lane == 0) *reinterpret_cast<float *>(out) = __fdiv_rn(1.0f, iscale);
-    }
+    rms_row<RMS_WAVES, 1>(input + (size_t)blockIdx.x * in_stride, gamma, y + (size_t)blockIdx.x * (d_model / 256) * 292,
+                          d_model, eps, reinterpret_cast<float *>(smem));
 }
 
 extern "C" int ckq_launch_rmsnorm_q8_k_fused(const float *input, const float *gamma, void *y, int tokens, int d_model,
@@ -685,7 +687,7 @@ extern "C" int ckq_launch_rmsnorm_q8_k_fused(const float *input, const float *ga
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return (int)e;
     }
-    hipLaunchKernelGGL(rmsnorm_q8_k_fused_kernel, dim3((unsigned)tokens), dim3(256), lds, (hipStream_t)stream,
+    hipLaunchKernelGGL(rmsnorm_q8_k_fused_kernel, dim3((unsigned)tokens), dim3(64 * RMS_WAVES), lds, (hipStream_t)stream,
                        input, gamma, (uint8_t *)y, d_model, (long)aligned_embed_dim, eps);
     return (int)hipGetLastError();
 }

@@ -143,13 +143,9 @@ def dev_quantize(x_t, fmt="q8_k", rows=1):
     return out
 
 
-ACT_F32_QUANT = 0x100
-
-
 def fmt_tag(name):
-    """Weight-format tag; "<fmt>+f32q" adds CKQ_ACT_F32_QUANT (fp32 activations
-    quantized to Q8_K inside the consumer)."""
-    return FMT[name[:-5]] | ACT_F32_QUANT if name.endswith("+f32q") else FMT[name]
+    """Weight-format tag of a format name."""
+    return FMT[name]
 
 
 def dev_gemm_nt(fmt, A_t, B_t, bias_t, M, N, K, out=None):

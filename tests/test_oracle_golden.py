@@ -2,6 +2,7 @@
 (tests/golden/make_golden.py), hand-computed known answers, closed forms and
 brute force.  Runs on CPU."""
 import ctypes
+import os
 
 import numpy as np
 import pytest
@@ -511,3 +512,18 @@ def test_cpu_timing_harness_computes_what_it_times():
     assert np.all(sec > 0)
     assert orc.orc_time_split_gemv(fn, T.ptr(y), T.ptr(W), T.ptr(xq), M, K, 0, iters, T.ptr(sec)) == -1
     assert orc.orc_time_split_gemv(None, T.ptr(y), T.ptr(W), T.ptr(xq), M, K, nth, iters, T.ptr(sec)) == -1
+
+
+def test_sanitizer_pass_over_cpu_code():
+    """The oracle, the synthetic-data encoders and the library's HIP-free host
+    helpers built with -fsanitize=address,undefined and driven over ragged
+    shapes, extreme inputs and malformed manifest lines (oracle/asan_harness.c):
+    no report, exit status 0."""
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run(["make", "-C", os.path.join(root, "oracle"), "asan"], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
+    r = subprocess.run([os.path.join(root, "oracle", "asan_harness")], capture_output=True, text=True,
+                       env=dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=0", LD_PRELOAD=""))
+    assert r.returncode == 0 and "ok" in r.stdout, (r.stdout + r.stderr)[-3000:]
+    assert "runtime error" not in r.stderr and "AddressSanitizer" not in r.stderr
