@@ -258,10 +258,23 @@ def cpu_baseline(rows, K, seconds_budget=12.0):
     res = {}
     for threads in (1, nth):
         per = max(float(np.median(timed(threads, 5))), 1e-6)
-        iters = int(max(20, min(20000, (seconds_budget / 2) / per)))
+        iters = int(max(20, min(20000, (seconds_budget / 3) / per)))
         ts = timed(threads, iters)
         res[threads] = (float(np.median(ts)), float(ts.mean()), iters)
     bytes_ = gemv_bytes("q4_k", rows, K)
+    # the same call rotating over 22 copies of the weights (558 MB): every round reads its weights from DRAM,
+    # like the GPU figure, which rotates over more weight bytes than the Infinity Cache holds
+    ncopies = 22
+    Wrot = np.tile(W, ncopies)
+    orc.orc_time_split_gemv_rotating.restype = ctypes.c_int
+    orc.orc_time_split_gemv_rotating.argtypes = ([ctypes.c_void_p] * 3 + [ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p] +
+                                                 [ctypes.c_int] * 4 + [ctypes.c_void_p])
+    it_rot = int(max(2 * ncopies, min(4000, (seconds_budget / 3) / max(res[nth][0], 1e-6))))
+    sec = np.zeros(it_rot, np.float64)
+    if orc.orc_time_split_gemv_rotating(fn_addr, p(y), p(Wrot), len(W), ncopies, p(xq), rows, K, nth, it_rot, p(sec)):
+        raise RuntimeError("orc_time_split_gemv_rotating failed")
+    rot_med = float(np.median(sec[ncopies:]))
+    del Wrot
     med, mean, iters = res[nth]
     model = "unknown"
     try:
@@ -276,6 +289,8 @@ def cpu_baseline(rows, K, seconds_budget=12.0):
         "host_cores": os.cpu_count(), "cpu_model": model,
         "median_ms": round(med * 1e3, 4), "mean_ms": round(mean * 1e3, 4),
         "single_thread_gbs": round(bytes_ / res[1][0] / 1e9, 3),
+        "rotated_gbs": round(bytes_ / rot_med / 1e9, 3), "rotated_median_ms": round(rot_med * 1e3, 4),
+        "rotated_sample": "%d calls rotating over %d copies of the weights (%d MB, from DRAM), same threads" % (it_rot, ncopies, ncopies * len(W) >> 20),
         "sample": "%d calls of %s %dx%d M=1 row-split over %d persistent threads, one barrier-bracketed round per call, the same "
                   "25 MB of weights every call (they stay in the host's last-level cache) (median %.2f ms/call, mean %.2f); "
                   "single thread median %.2f ms/call" % (iters, fn_name, rows, K, nth, med * 1e3, mean * 1e3, res[1][0] * 1e3),
@@ -407,6 +422,13 @@ def main():
         extras["gemm_q4_k_q8_k_M512"] = {"tops": round(ops / sg / 1e12, 2), "ms": round(sg * 1e3, 4),
                                          "frac_int8_peak": round(ops / sg / 1e12 / INT8_PEAK_TOPS, 4),
                                          "ops_per_call": ops, "kernel": "two-plane int8 MFMA (v_mfma_i32_32x32x32_i8) + bf16 MFMA min term"}
+        # a longer prompt: four times the tokens against the same weights
+        xg2 = P.dev_quantize(P.to_device(T.normal(2048 * K, seed=98)), "q8_k", rows=2048)
+        sg2, _, _ = H.time_gemv("q4_k", rows, K, 2048, copies[:2], xg2, 8, GEMM_REPS)
+        extras["gemm_q4_k_q8_k_M2048"] = {"tops": round(2.0 * 2048 * rows * K / sg2 / 1e12, 2), "ms": round(sg2 * 1e3, 4),
+                                          "frac_int8_peak": round(2.0 * 2048 * rows * K / sg2 / 1e12 / INT8_PEAK_TOPS, 4),
+                                          "ops_per_call": 2.0 * 2048 * rows * K}
+        del xg2
         # the same prefill step for the down projection of a Q4_K_M model: Q6_K weights, K = 11008
         r6, k6 = 4096, 11008
         _, cps6 = H.weight_copies("q6_k", r6, k6, seed=66, min_total=1)
@@ -465,21 +487,11 @@ def main():
         # fp32-activation entry point (gemv_q4_k: weights dequantized on the fly, nothing quantized)
         xf_d = P.to_device(xf)
         outf = torch.empty(rows, dtype=torch.float32, device="cuda")
-        for c in copies[:4]:
-            P.dev_gemm_nt_f32act("q4_k", xf_d, c, None, 1, rows, K, out=outf)
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        nf = 64 * len(copies)
-        e0.record()
-        for i in range(nf):
-            P.dev_gemm_nt_f32act("q4_k", xf_d, copies[i % len(copies)], None, 1, rows, K, out=outf)
-        e1.record()
-        torch.cuda.synchronize()
-        sf = e0.elapsed_time(e1) * 1e-3 / nf
+        sf = H.time_sequence([[("q4_k+f32", xf_d, c, None, outf, 1, rows, K)] for c in copies], 128, 5)
         bf = len(W) + 4 * K + 4 * rows
         extras["gemv_q4_k_f32act_11008x4096"] = {"gbs": round(bf / sf / 1e9, 1), "us": round(sf * 1e6, 2),
                                                  "frac_hbm": round(bf / sf / 1e9 / HBM_PEAK_GBS, 4),
-                                                 "note": "launched from Python one call at a time"}
+                                                 "note": "fp32 activations, weights dequantized on the fly; back-to-back launches of one C call"}
 
         # fused producer rmsnorm -> Q8_K next to the plain quantizer (launch-bound at one token)
         gam_d = P.to_device(T.normal(K, 1.0, 0.2, seed=55))
@@ -550,49 +562,12 @@ def main():
                 ("swiglu_q8_k", g_[4], u_[4], hq_, 1, 11008, 11008),
                 ("q6_k", hq_, d_[2], None, d_[4], 1, 4096, 11008)])
         sc = H.time_sequence(chains, 64, 5)
-        ab = {}
-        for mode, key in ((0, "unfused_us"), (2, "all_fused_us")):      # A/B against the default (1: fuse where it pays)
-            H.L.ckq_set_fused_producers(mode)
-            try:
-                ab[key] = round(H.time_sequence(chains, 64, 5) * 1e6, 2)
-            finally:
-                H.L.ckq_set_fused_producers(1)
         extras["layer_7b_decode_chain_M1"] = {"us": round(sc * 1e6, 2), "matmul_only_us": round(s * 1e6, 2),
-                                              "producers_us": round((sc - s) * 1e6, 2), "launches": 7,
+                                              "producers_us": round((sc - s) * 1e6, 2), "launches": 8,
                                               "gbs_of_weight_bytes": round(lbytes / sc / 1e9, 1),
-                                              "unfused_us": ab["unfused_us"], "all_fused_us": ab["all_fused_us"],
-                                              "expired_waits": int(H.L.ckq_fused_producer_timeouts(P._stream())),
-                                              "note": "norm->Q8_K | Q+K+V | Q8_K + O (one launch: the quantizer rides at the front "
-                                                      "of the O projection's grid) | norm->Q8_K | gate+up | SwiGLU->Q8_K | down, one C call "
-                                                      "per layer; unfused_us: eight launches; all_fused_us: every producer fused with "
-                                                      "its matmuls (four launches)"}
+                                              "note": "norm->Q8_K, Q+K+V, Q8_K, O, norm->Q8_K, gate+up, SwiGLU->Q8_K, down in one C call"}
         del layers, keep, chains
         torch.cuda.empty_cache()
-
-        # a producer as its own launch in front of the GEMV against the fused launch (producer
-        # blocks at the front of the GEMV's grid; the GEMV blocks stream weights while they run)
-        fpm = {}
-        for fmt, r, k in (("q4_k", 4096, 4096), ("q4_k", 11008, 4096), ("q6_k", 4096, 11008)):
-            _, cps = H.weight_copies(fmt, r, k, seed=r + k + 7)
-            xf = P.to_device(T.normal(k, 0.0, 1.0, seed=51))
-            gk = P.to_device(T.normal(k, 1.0, 0.2, seed=52))
-            xq = torch.zeros(T.row_bytes("q8_k", k), dtype=torch.uint8, device="cuda")
-            y = torch.zeros(r, dtype=torch.float32, device="cuda")
-            ent = {"gemv_alone_us": round(H.time_sequence([[(fmt, xq, c, None, y, 1, r, k)] for c in cps], 128, 5) * 1e6, 2)}
-            for pname, pstep in (("quantize", ("quantize_q8_k", xf, None, xq, 1, k)),
-                                 ("rmsnorm", ("rmsnorm_q8_k", xf, gk, xq, 1, k, k, 1e-5))):
-                seqs = [[pstep, (fmt, xq, c, None, y, 1, r, k)] for c in cps]
-                H.L.ckq_set_fused_producers(2)
-                ent[pname + "_fused_us"] = round(H.time_sequence(seqs, 128, 5) * 1e6, 2)
-                H.L.ckq_set_fused_producers(0)
-                try:
-                    ent[pname + "_then_gemv_us"] = round(H.time_sequence(seqs, 128, 5) * 1e6, 2)
-                finally:
-                    H.L.ckq_set_fused_producers(1)
-            fpm["%s_%dx%d" % (fmt, r, k)] = ent
-            del cps
-            torch.cuda.empty_cache()
-        extras["fused_producer_M1"] = fpm
 
         # small-model batched decode (Qwen2-0.5B-like: hidden 896 padded to K=1024, Q5_K
         # projections, Q8_0 LM head 151936x896), M tokens per step

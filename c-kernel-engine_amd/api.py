@@ -137,8 +137,6 @@ _SIGS = {
     "ckq_weights_set_cache": (None, [_i]),
     "ckq_weights_set_limit": (None, [_c.c_size_t]),
     "ckq_release_stream": (_i, [_vp]),
-    "ckq_set_fused_producers": (None, [_i]),
-    "ckq_fused_producer_timeouts": (_i, [_vp]),
     "ckq_set_parallel_whole": (None, [_i]),
     "ckq_set_gemm_policy": (None, [_i]),
     "ckq_last_error": (_i, []),

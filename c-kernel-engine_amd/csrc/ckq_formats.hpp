@@ -48,7 +48,6 @@ __device__ __forceinline__ void k4_scale_pair(u32 u0, u32 u1, u32 u2, int g, u32
 struct FmtQ4K {
     static constexpr int POS_PER_BLOCK = 4, WBLOCK = 144, XBLOCK = 292, NSUB = 2;
     static constexpr int OCC1 = 8, OCC2 = 6;   /* waves per SIMD the one-token kernel is held to: one row, two rows per wave */
-    static constexpr int OCC1_PRO = 8, OCC2_PRO = 6;   /* the same for the fused launch (producer blocks in front) */
     static constexpr bool TOKEN_TILES = true; /* tiles of 2, 4 and 8 tokens exist */
     struct Wt  { u32 hdr[4]; u32 qs[8]; };
     struct Act { int q[16]; float d; int b_lo, b_hi; };
@@ -129,7 +128,6 @@ struct FmtQ4K {
 struct FmtQ5K {
     static constexpr int POS_PER_BLOCK = 4, WBLOCK = 176, XBLOCK = 292, NSUB = 2;
     static constexpr int OCC1 = 8, OCC2 = 5;            /* waves per SIMD the one-token kernel is held to */
-    static constexpr int OCC1_PRO = 7, OCC2_PRO = 5;    /* the same for the fused launch (producer blocks in front) */
     static constexpr bool TOKEN_TILES = true; /* tiles of 2, 4 and 8 tokens exist */
     struct Wt  { u32 hdr[4]; u32 qh[8]; u32 qs[8]; };
     typedef FmtQ4K::Act Act;
@@ -192,7 +190,6 @@ struct FmtQ5K {
 struct FmtQ6K {
     static constexpr int POS_PER_BLOCK = 4, WBLOCK = 210, XBLOCK = 292, NSUB = 4;
     static constexpr int OCC1 = 8, OCC2 = 6;   /* waves per SIMD the one-token kernel is held to: one row, two rows per wave */
-    static constexpr int OCC1_PRO = 7, OCC2_PRO = 5;   /* the same for the fused launch (producer blocks in front) */
     static constexpr bool TOKEN_TILES = true; /* tiles of 2, 4 and 8 tokens exist */
     struct Wt  { u32 ql0[4], ql1[4], qh[4]; u32 sc[2]; u32 d; };
     struct Act { int q[16]; float d; int a32[4]; };      /* a32[r] = 32 * sum of the run's 16 quants */

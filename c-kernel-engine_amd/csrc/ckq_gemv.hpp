@@ -10,7 +10,6 @@
 
 #include "ckq_blocks.h"
 #include "ckq_formats.hpp"
-#include "ckq_producers.hpp"
 #include "ckq_launch.h"
 
 constexpr int CKQ_GROUP_MAX = 4;   /* independent matmuls of one shape in one launch */
@@ -23,8 +22,6 @@ struct GemvArgs {
     int32_t       *sub;
     int  nrows, npos, ntok, row0, row1, nsub_row;
     long wrow, xrow, ldy;
-    const GemvPro *pro;   /* host side only: producer blocks in front of the launch (fused launch), or NULL */
-    int  *pro_blocks;     /* host side only: receives the number of producer blocks a fused launch ran */
 };
 
 /* Problems 1..3 of a grouped launch (blockIdx.z = g > 0); problem 0 is in GemvArgs. */
@@ -49,9 +46,10 @@ struct GemvGroup {
  * summed over the LPR lanes with a fixed DPP tree; the last lane of the group
  * stores.
  */
-template <class F, int LPR, int PPL, int MT, int RPI, bool DUMP, int WPB, bool LDSX, bool GRP, bool PRO>
-__device__ __forceinline__ void gemv_body(const uint8_t *W, const uint8_t *X, long wrow, long xrow, int row0, int row1, int npos, int ntok,
-            float *y, const float *bias, long ldy, int32_t *sub, int nsub_row, int nrows, const GemvGroup &grp, const GemvPro &pro)
+template <class F, int LPR, int PPL, int MT, int RPI, bool DUMP, int WPB, bool LDSX, bool GRP = false>
+__global__ void __launch_bounds__(64 * WPB) __attribute__((amdgpu_waves_per_eu(DUMP ? 1 : MT == 1 && PPL == 1 && RPI == 1 ? F::OCC1 : MT == 1 && PPL == 1 && RPI == 2 && LPR == 64 ? F::OCC2 : MT >= 4 && PPL == 1 ? 4 : 1)))
+gemv_kernel(const uint8_t *W, const uint8_t *X, long wrow, long xrow, int row0, int row1, int npos, int ntok,
+            float *y, const float *bias, long ldy, int32_t *sub, int nsub_row, int nrows, GemvGroup grp)
 {
     /* The arguments are scalars, those the first loads need in front: the
      * first fourteen registers' worth arrive preloaded with the wave (build
@@ -72,17 +70,7 @@ __device__ __forceinline__ void gemv_body(const uint8_t *W, const uint8_t *X, lo
     const float *const   gbias = g == 0 ? a.bias : grp.bias[g - 1];
     const int lane = threadIdx.x & 63, wave = wave_in_block();
     const int slot = lane / LPR, l = lane % LPR;
-    /* fused launch: the first pro.nblocks blocks of grid x are the producer's (those of the
-     * first token tile of the first problem run it), the matmul blocks follow */
-    int bx = (int)blockIdx.x;
-    if constexpr (PRO) {
-        if (bx < pro.nblocks) {
-            if (blockIdx.y == 0 && blockIdx.z == 0) pro_block<WPB>(pro, bx, xs);
-            return;
-        }
-        bx -= pro.nblocks;
-    }
-    const int wave_row = a.row0 + (bx * WPB + wave) * (SLOTS * RPI);   /* uniform */
+    const int wave_row = a.row0 + (blockIdx.x * WPB + wave) * (SLOTS * RPI);   /* uniform */
     const bool live = wave_row < a.row1;
     if (!LDSX && !live) return;
     const int wrow_c = min(wave_row, a.row1 - 1);
@@ -102,12 +90,6 @@ __device__ __forceinline__ void gemv_body(const uint8_t *W, const uint8_t *X, lo
     const int xbytes = (int)((long)mt_live * a.xrow), xn = xbytes / F::XS_SRC;   /* staging units */
     const u32 xcap = (u32)((long)MT * a.xrow / F::XS_SRC);                                     /* units of a full tile */
     u32 xv[XU][F::XS_REGS];
-    /* fused launch: the block is resident and waits here, before it has a single load in
-     * flight, until the producer blocks have counted.  (Streaming the weights during the wait
-     * was measured and lost: with every matmul block's loads queued, the producer's few loads,
-     * its counter update, each poll and the activation loads are all round trips at LOADED
-     * latency - 11.3 us against 9.2 for quantizer + 11008x4096 as two launches.) */
-    if constexpr (PRO) pro_wait(pro);
     if (LDSX) {
 #pragma unroll
         for (int u = 0; u < XU; ++u) {
@@ -248,28 +230,6 @@ __device__ __forceinline__ void gemv_body(const uint8_t *W, const uint8_t *X, lo
         }
 }
 
-#define CKQ_GEMV_OCC (DUMP ? 1 : MT == 1 && PPL == 1 && RPI == 1 ? F::OCC1 : MT == 1 && PPL == 1 && RPI == 2 && LPR == 64 ? F::OCC2 : MT >= 4 && PPL == 1 ? 4 : 1)
-
-template <class F, int LPR, int PPL, int MT, int RPI, bool DUMP, int WPB, bool LDSX, bool GRP = false>
-__global__ void __launch_bounds__(64 * WPB) __attribute__((amdgpu_waves_per_eu(CKQ_GEMV_OCC)))
-gemv_kernel(const uint8_t *W, const uint8_t *X, long wrow, long xrow, int row0, int row1, int npos, int ntok,
-            float *y, const float *bias, long ldy, int32_t *sub, int nsub_row, int nrows, GemvGroup grp)
-{
-    gemv_body<F, LPR, PPL, MT, RPI, DUMP, WPB, LDSX, GRP, false>(W, X, wrow, xrow, row0, row1, npos, ntok, y, bias, ldy, sub,
-                                                                 nsub_row, nrows, grp, GemvPro{});
-}
-
-/* The fused launch: producer blocks in front (ckq_producers.hpp), the matmul
- * blocks behind them; activations always staged in LDS. */
-template <class F, int LPR, int PPL, int MT, int RPI, int WPB, bool GRP>
-__global__ void __launch_bounds__(64 * WPB) __attribute__((amdgpu_waves_per_eu(MT == 1 && PPL == 1 && RPI == 1 ? (LPR == 64 ? F::OCC1_PRO : 7) : MT == 1 && PPL == 1 && RPI == 2 && LPR == 64 ? F::OCC2_PRO : MT >= 4 && PPL == 1 ? 4 : 1)))
-gemv_pro_kernel(const uint8_t *W, const uint8_t *X, long wrow, long xrow, int row0, int row1, int npos, int ntok,
-                float *y, const float *bias, long ldy, int32_t *sub, int nsub_row, int nrows, GemvGroup grp, GemvPro pro)
-{
-    gemv_body<F, LPR, PPL, MT, RPI, false, WPB, true, GRP, true>(W, X, wrow, xrow, row0, row1, npos, ntok, y, bias, ldy, sub,
-                                                                 nsub_row, nrows, grp, pro);
-}
-
 /* Rows the grid has to cover: the computed range, or the largest problem of a group. */
 static int launch_rows(const GemvArgs &a, const GemvGroup &grp) { return grp.n > 1 ? a.nrows : a.row1 - a.row0; }
 
@@ -312,52 +272,12 @@ static int launch_one(const GemvArgs &a0, const GemvGroup &grp, hipStream_t s)
     return 0;
 }
 
-/* LDS a fused launch needs: the staged token tile or the producer's row, whichever is larger. */
-static size_t pro_lds_bytes(const GemvPro &pro, size_t tile_bytes)
-{
-    const size_t p = pro.kind == CKQ_PRO_RMSNORM_Q8K ? (size_t)pro.k * 4 + 32 : 0;
-    return p > tile_bytes ? p : tile_bytes;
-}
-
-/* The fused launch of the same shape: pro.nblocks producer blocks (of WPB
- * waves) in front of the matmul blocks.  One token tile (ntok <= MT). */
-template <class F, int LPR, int PPL, int MT, int RPI, int WPB>
-static int launch_one_pro(const GemvArgs &a0, const GemvGroup &grp, hipStream_t s)
-{
-    constexpr int rows_per_block = WPB * (64 / LPR) * RPI;
-    if (a0.ntok > MT || a0.sub) return CKQ_EINVAL;
-    GemvPro pro = *a0.pro;
-    pro.nblocks = pro_block_count(pro.kind, pro.rows, pro.k, WPB);
-    pro.target += (unsigned)pro.nblocks;               /* host: the counter's value before this launch */
-    const int nr = launch_rows(a0, grp);
-    const size_t lds = pro_lds_bytes(pro, F::xs_lds_bytes((size_t)MT * (size_t)a0.xrow));
-    dim3 grid((unsigned)(pro.nblocks + (nr + rows_per_block - 1) / rows_per_block), 1, (unsigned)grp.n);
-    if (grp.n > 1)
-        hipLaunchKernelGGL((gemv_pro_kernel<F, LPR, PPL, MT, RPI, WPB, true>), grid, dim3(64 * WPB), lds, s,
-                           a0.W, a0.X, a0.wrow, a0.xrow, a0.row0, a0.row1, a0.npos, a0.ntok, a0.y, a0.bias, a0.ldy, a0.sub,
-                           a0.nsub_row, a0.nrows, grp, pro);
-    else
-        hipLaunchKernelGGL((gemv_pro_kernel<F, LPR, PPL, MT, RPI, WPB, false>), grid, dim3(64 * WPB), lds, s,
-                           a0.W, a0.X, a0.wrow, a0.xrow, a0.row0, a0.row1, a0.npos, a0.ntok, a0.y, a0.bias, a0.ldy, a0.sub,
-                           a0.nsub_row, a0.nrows, grp, pro);
-    const int rc = (int)hipGetLastError();
-    if (rc == 0) *a0.pro_blocks = pro.nblocks;
-    return rc;
-}
-
 /* Activation rows are staged in LDS when the token tile fits in 64 KB.  The
  * dump build of an instantiation exists for the staged form only. */
 template <class F, int LPR, int PPL, int MT, int RPI, int WPB>
 static int launch_tile(const GemvArgs &a, const GemvGroup &grp, hipStream_t s)
 {
     const bool fits = F::xs_lds_bytes((size_t)MT * (size_t)a.xrow) <= 65536;
-    if (a.pro) {
-        if constexpr (F::XBLOCK == 292 && F::TOKEN_TILES) {
-            if (pro_lds_bytes(*a.pro, F::xs_lds_bytes((size_t)MT * (size_t)a.xrow)) <= 65536)
-                return launch_one_pro<F, LPR, PPL, MT, RPI, WPB>(a, grp, s);
-        }
-        return CKQ_EINVAL;
-    }
     if (a.sub) {
         if constexpr (F::TOKEN_TILES) {
             if (fits) return launch_one<F, LPR, PPL, MT, RPI, true, WPB, true>(a, grp, s);

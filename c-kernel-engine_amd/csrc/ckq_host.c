@@ -25,6 +25,7 @@
 #include <stdlib.h>
 #include <string.h>
 #include <strings.h>
+#include <time.h>
 
 #include "ckernel_quant_hip.h"
 #include "ckq_launch.h"
@@ -76,6 +77,16 @@ typedef struct {
     size_t cap;
 } pin_buf;
 static pin_buf      g_pin[BUF_COUNT];
+/* Completion word of the host-pointer calls: a dword of pinned memory that the
+ * stream writes (hipStreamWriteValue32) once everything enqueued before it has
+ * finished.  The caller spins on it for a bounded time instead of entering
+ * hipStreamSynchronize, whose wake-up costs several microseconds on a call that
+ * is a few tens long; when the word does not arrive in time, or the write cannot
+ * be enqueued, the synchronisation call takes over. */
+static volatile uint32_t *g_done_host = NULL;
+static void              *g_done_dev = NULL;
+static uint32_t           g_done_seq = 0;
+static int                g_done_ok = 1;       /* cleared for good when the stream write is not available */
 static weight_entry *g_w = NULL;
 static size_t       g_nw = 0, g_capw = 0;
 static size_t       g_cache_max_bytes = (size_t)64 << 30;   /* bound on unpinned resident weights */
@@ -217,6 +228,41 @@ static int is_device_ptr(const void *p)
     return 0;
 }
 
+/* Waits for the work enqueued on the library's stream so far. */
+static int stream_wait(void)
+{
+    if (g_done_ok && !g_done_host) {
+        void *h = NULL;
+        if (hipHostMalloc(&h, 64, hipHostMallocDefault) == hipSuccess && hipHostGetDevicePointer(&g_done_dev, h, 0) == hipSuccess) {
+            g_done_host = (volatile uint32_t *)h;
+            *g_done_host = 0;
+        } else {
+            (void)hipGetLastError();
+            g_done_ok = 0;
+        }
+    }
+    if (g_done_ok) {
+        const uint32_t seq = ++g_done_seq;
+        if (hipStreamWriteValue32(g_stream, g_done_dev, seq, 0) == hipSuccess) {
+            struct timespec t0, t1;
+            clock_gettime(CLOCK_MONOTONIC, &t0);
+            for (unsigned spins = 0;; ++spins) {
+                if (*g_done_host == seq) return 0;
+                __builtin_ia32_pause();
+                if ((spins & 1023) == 1023) {
+                    clock_gettime(CLOCK_MONOTONIC, &t1);
+                    if ((t1.tv_sec - t0.tv_sec) * 1000000000L + (t1.tv_nsec - t0.tv_nsec) > 200000L) break;   /* 0.2 ms: a long job */
+                }
+            }
+        } else {
+            (void)hipGetLastError();
+            g_done_ok = 0;
+        }
+    }
+    HIP_TRY(hipStreamSynchronize(g_stream));
+    return 0;
+}
+
 static int buf_reserve(int which, size_t bytes, void **out)
 {
     dev_buf *b = &g_buf[which];
@@ -298,7 +344,8 @@ static int stage_out_sync(int which, void *dst, size_t dst_pitch, size_t src_pit
         if (rc) return rc;
         rc = ckq_launch_copy(g_pin[which].dev, dev, round16(span), g_stream);
         if (rc) return fail(rc, "download through the pinned twin");
-        HIP_TRY(hipStreamSynchronize(g_stream));
+        rc = stream_wait();
+        if (rc) return rc;
         for (size_t r = 0; r < rows; ++r) memcpy((uint8_t *)dst + r * dst_pitch, (const uint8_t *)h + r * src_pitch, w);
         return 0;
     }
@@ -660,8 +707,7 @@ static void matmul_locked(int fmt, const void *A, const void *B, const float *bi
         int rc = ckq_launch_gemv(fmt, dC, dB, dA, (const float *)dbias, nrows, K, ntok, ld, row0, row1, NULL, g_stream);
         if (rc) { fail(rc, "ckq_launch_gemv"); break; }
         if (ypin) {
-            hipError_t e = hipStreamSynchronize(g_stream);
-            if (e != hipSuccess) { fail((int)e, "hipStreamSynchronize"); break; }
+            if (stream_wait()) break;
             const size_t w = (size_t)(row1 - row0) * sizeof(float);
             for (int t = 0; t < ntok; ++t) memcpy(C + (size_t)t * ldc + row0, (const uint8_t *)ypin + (size_t)t * w, w);
         } else if (!c_on_dev) {
@@ -1282,28 +1328,6 @@ static int issue_producer(const ckq_matmul_op *o, void *stream)
     }
 }
 
-/* 0 = never, 1 = where it was measured to pay (below), 2 = wherever a fused form exists */
-static int g_fuse_producers = 1;
-void ckq_set_fused_producers(int mode) { __atomic_store_n(&g_fuse_producers, mode < 0 || mode > 2 ? 1 : mode, __ATOMIC_RELAXED); }
-/* Weight bytes of the matmuls up to which a fused launch beats two launches.
- * Measured at one token (us; producer + matmul as two launches -> fused):
- * fp32 -> Q8_K or SiLU*up -> Q8_K in front of Q4_K 1024x4096 11.0 -> 8.7,
- * 4096x4096 8.1 -> 6.8; 11008x4096 8.2 -> 10.2 and Q6_K 4096x11008 11.8 -> 13.6
- * lose: the handover (the producers' write-back, the counter, the first
- * poll) is four round trips through memory, which cost what a launch
- * boundary costs once the matmul is long enough to hide the next dispatch.
- * RMSNorm in front loses at every size (4096x4096 8.8 -> 11.2): as a
- * four-wave producer block its serial chains are slower than in the
- * sixteen-wave kernel. */
-enum { FUSE_MAX_WEIGHT_BYTES = 12 << 20 };
-
-int ckq_fused_producer_timeouts(void *stream)
-{
-    unsigned n = 0;
-    const int rc = ckq_launch_pro_timeouts(stream, &n);
-    return rc ? (rc > 0 ? -rc : rc) : (int)n;
-}
-
 /* Number of consecutive matmul entries from ops[i] on that can share a launch (1..4). */
 static int group_length(const ckq_matmul_op *ops, int i, int nops)
 {
@@ -1311,60 +1335,16 @@ static int group_length(const ckq_matmul_op *ops, int i, int nops)
     const ckq_matmul_op *o = &ops[i];
     int n = 1;
     const int groupable = o->A_q8 && o->B && o->C && o->M >= 1 && o->M <= 8 && o->N > 0 && o->K > 0 &&
-                          o->ldc >= o->N && !is_f32act(o->fmt) && o->K % fmt_block_elems(o->fmt) == 0;
+                          o->ldc >= o->N && !is_f32act(o->fmt) && !(o->fmt & CKQ_ACT_F32) && o->K % fmt_block_elems(o->fmt) == 0;
     while (groupable && n < GROUP_MAX && i + n < nops) {
         if (ops[i + n].fmt >= CKQ_STEP_QUANTIZE_Q8_K && ops[i + n].fmt <= CKQ_STEP_SWIGLU_Q8_K) break;
+        if (ops[i + n].fmt & CKQ_ACT_F32) break;
         int ok = 1;
         for (int j = 0; j < n && ok; ++j) ok = ops_independent(&ops[i + j], &ops[i + n]);
         if (!ok) break;
         ++n;
     }
     return n;
-}
-
-/* Producer entry p followed by the n matmul entries m[0..n): one fused launch
- * when every one of them reads the producer's output and nothing else of the
- * producer's memory is written by them.  Returns CKQ_EUNFUSED when the steps
- * have to go out one by one. */
-static int issue_fused(const ckq_matmul_op *p, const ckq_matmul_op *m, int n, void *stream)
-{
-    const int mode = __atomic_load_n(&g_fuse_producers, __ATOMIC_RELAXED);
-    if (!mode) return CKQ_EUNFUSED;
-    const int kind = p->fmt == CKQ_STEP_QUANTIZE_Q8_K ? 1 : p->fmt == CKQ_STEP_RMSNORM_Q8_K ? 2
-                   : p->fmt == CKQ_STEP_SWIGLU_Q8_K ? 3 : 0;
-    if (!kind || !p->A_q8 || !p->C || p->M <= 0 || p->K <= 0) return CKQ_EUNFUSED;
-    if (kind != 1 && !p->B) return CKQ_EUNFUSED;
-    const long pld = p->ldc ? p->ldc : p->K;
-    if (pld < p->K) return CKQ_EUNFUSED;
-    const size_t in_bytes = ((size_t)(p->M - 1) * (size_t)pld + (size_t)p->K) * sizeof(float);
-    float *y[4];
-    const void *W[4], *X[4];
-    const float *b[4];
-    int rows[4];
-    long ld[4];
-    if (mode == 1) {
-        size_t wbytes = 0;
-        for (int j = 0; j < n; ++j) wbytes += (size_t)m[j].N * weight_row_bytes(m[j].fmt, m[j].K);
-        if (kind == 2 || wbytes > FUSE_MAX_WEIGHT_BYTES) return CKQ_EUNFUSED;
-    }
-    for (int j = 0; j < n; ++j) {
-        const ckq_matmul_op *q = &m[j];
-        if (q->fmt != m[0].fmt || q->M != p->M || q->K != p->K || q->A_q8 != (const void *)p->C) return CKQ_EUNFUSED;
-        if (!q->B || !q->C || q->N <= 0 || q->ldc < q->N) return CKQ_EUNFUSED;
-        /* the matmuls run while the producer reads its input: they must not write it */
-        const size_t qc = ((size_t)(q->M - 1) * (size_t)q->ldc + (size_t)q->N) * sizeof(float);
-        if (ranges_overlap(q->C, qc, p->A_q8, in_bytes)) return CKQ_EUNFUSED;
-        if (kind != 1 && ranges_overlap(q->C, qc, p->B, kind == 2 ? (size_t)p->K * sizeof(float) : in_bytes)) return CKQ_EUNFUSED;
-        /* the matmul blocks read their weights (and nothing else of the producer's concern) before the
-         * producer has finished: no cache line of its output may be shared with them */
-        const uintptr_t o0 = (uintptr_t)p->C & ~(uintptr_t)127;
-        const size_t ob = (size_t)p->M * act_row_bytes(q->fmt, q->K);
-        const size_t olen = (((uintptr_t)p->C + ob + 127) & ~(uintptr_t)127) - o0;
-        if (ranges_overlap((const void *)o0, olen, q->B, (size_t)q->N * weight_row_bytes(q->fmt, q->K))) return CKQ_EUNFUSED;
-        y[j] = q->C; W[j] = q->B; X[j] = q->A_q8; b[j] = q->bias; rows[j] = q->N; ld[j] = q->ldc;
-    }
-    return ckq_launch_gemv_pro(m[0].fmt, n, y, W, X, b, rows, ld, m[0].K, m[0].M, kind, (const float *)p->A_q8,
-                               (const float *)p->B, p->C, p->M, p->K, pld, p->eps, stream);
 }
 
 int ckq_matmul_sequence_dev(const ckq_matmul_op *ops, int nops, int repeat, void *stream)
@@ -1375,16 +1355,14 @@ int ckq_matmul_sequence_dev(const ckq_matmul_op *ops, int nops, int repeat, void
         for (int i = 0; i < nops;) {
             const ckq_matmul_op *o = &ops[i];
             if (o->fmt >= CKQ_STEP_QUANTIZE_Q8_K && o->fmt <= CKQ_STEP_SWIGLU_Q8_K) {
-                /* a producer and the matmuls right behind it that read its output: one launch,
-                 * the weights stream while the producer runs */
-                if (i + 1 < nops && !(ops[i + 1].fmt >= CKQ_STEP_QUANTIZE_Q8_K && ops[i + 1].fmt <= CKQ_STEP_SWIGLU_Q8_K) &&
-                    ops[i + 1].M <= 8) {
-                    const int n = group_length(ops, i + 1, nops);
-                    const int rc = issue_fused(o, &ops[i + 1], n, stream);
-                    if (rc == 0) { i += 1 + n; continue; }
-                    if (rc != CKQ_EUNFUSED) return rc;
-                }
                 const int rc = issue_producer(o, stream);
+                if (rc) return rc;
+                ++i;
+                continue;
+            }
+            if (o->fmt & CKQ_ACT_F32) {              /* fp32 activations: the dequant-dot kernels, one launch per entry */
+                const int rc = ckq_gemm_nt_f32act_dev(o->fmt & ~CKQ_ACT_F32, (const float *)o->A_q8, o->B, o->bias, o->C, o->M,
+                                                      o->N, o->K, o->ldc, stream);
                 if (rc) return rc;
                 ++i;
                 continue;

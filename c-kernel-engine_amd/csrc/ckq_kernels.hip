@@ -95,8 +95,7 @@ static std::recursive_mutex g_split_mu;
 std::recursive_mutex &gemm_split_mutex() { return g_split_mu; }
 
 /* Grow-only device scratch per (device, stream, kind); see ckq_gemm_common.hpp.
- * kind 0: partial tiles of a K split; kind 1: weights rewritten for another kernel;
- * kind 2: the completion counter of fused producer launches (pro_counter below).
+ * kind 0: partial tiles of a K split; kind 1: weights rewritten for another kernel.
  * When all slots are taken the least recently used one is recycled: the device is
  * synchronised (its stream may no longer exist), its buffer freed.  A destroyed
  * stream whose handle value is given out again finds the old stream's slot: harmless,
@@ -328,102 +327,6 @@ extern "C" int ckq_launch_gemv_group(int fmt, int n, float *const *y, const void
     return launch_gemv_args(fmt, a, grp, K, stream);
 }
 
-/* The completion counter of fused producer launches on `s`: two dwords of
- * device memory per (device, stream), zeroed when created, and the value
- * flag[0] will have once everything enqueued so far has run.  The caller holds
- * g_split_mu from here until its launch is enqueued and then adds the
- * launch's producer blocks to *epoch. */
-static int pro_counter(hipStream_t s, unsigned **flag, unsigned **epoch)
-{
-    WsSlot *sl = nullptr;
-    bool fresh = false;
-    int rc = workspace_slot(2, s, 64, &sl, &fresh);
-    if (rc) return rc;
-    if (fresh) {
-        hipError_t e = hipMemsetAsync(sl->p, 0, 64, s);
-        if (e != hipSuccess) return (int)e;
-        sl->epoch = 0;
-    }
-    *flag = (unsigned *)sl->p;
-    *epoch = &sl->epoch;
-    return 0;
-}
-
-static std::atomic<int> g_pro_spin_limit{1 << 20};     /* polls of ~0.5 us each before a matmul block gives up waiting */
-extern "C" void ckq_launch_set_pro_spin_limit(int polls) { g_pro_spin_limit.store(polls > 0 ? polls : 1 << 20); }
-
-/* Expired waits recorded by fused launches on `stream` so far (synchronises the stream). */
-extern "C" int ckq_launch_pro_timeouts(void *stream, unsigned *count)
-{
-    std::lock_guard<std::recursive_mutex> lock(g_split_mu);
-    unsigned *flag, *epoch;
-    int rc = pro_counter((hipStream_t)stream, &flag, &epoch);
-    if (rc) return rc;
-    hipError_t e = hipMemcpyAsync(count, flag + 1, sizeof(unsigned), hipMemcpyDeviceToHost, (hipStream_t)stream);
-    if (e == hipSuccess) e = hipStreamSynchronize((hipStream_t)stream);
-    return (int)e;
-}
-
-/* A producer (CKQ_PRO_*: fp32 rows -> Q8_K blocks at `dst`) and the n (1..4)
- * matmuls that read `dst` as ONE launch: producer blocks in front, the matmul
- * blocks start streaming their weights at once and wait for the producer's
- * count before they touch the activations.  Up to eight tokens, Q4_K / Q5_K /
- * Q6_K weights.  Returns CKQ_EUNFUSED, with nothing enqueued, when this
- * combination has no fused form (the caller then issues the steps one by one):
- * other formats, a token tile or a row too large for LDS, a stream that is
- * being captured (the counter's expected value is baked into the launch, so a
- * replay would not wait). */
-extern "C" int ckq_launch_gemv_pro(int fmt, int n, float *const *y, const void *const *W, const void *const *X,
-                                   const float *const *bias, const int *rows, const long *ldys, int K, int ntok,
-                                   int kind, const float *src, const float *src2, void *dst, int pro_rows, int pro_k,
-                                   long pro_ld, float eps, void *stream)
-{
-    if (n < 1 || n > CKQ_GROUP_MAX || !y || !W || !X || !rows || !ldys || K <= 0 || ntok < 1) return CKQ_EINVAL;
-    if (!src || !dst || pro_rows <= 0 || pro_k <= 0 || pro_ld < pro_k) return CKQ_EINVAL;
-    if (fmt != CKQ_FMT_Q4_K && fmt != CKQ_FMT_Q5_K && fmt != CKQ_FMT_Q6_K) return CKQ_EUNFUSED;
-    if (ntok > CKQ_STREAM_TOKENS || K % 256 || pro_k % 256) return CKQ_EUNFUSED;
-    if (kind != CKQ_PRO_QUANT_Q8K && kind != CKQ_PRO_RMSNORM_Q8K && kind != CKQ_PRO_SWIGLU_Q8K) return CKQ_EINVAL;
-    if (kind != CKQ_PRO_QUANT_Q8K && !src2) return CKQ_EINVAL;
-    if (pro_ld % 4 || ((uintptr_t)src | (uintptr_t)src2) % 16) return CKQ_EUNFUSED;
-    if (!group_tile_fits_lds(fmt, K, ntok)) return CKQ_EUNFUSED;
-    if (kind == CKQ_PRO_RMSNORM_Q8K && (size_t)pro_k * 4 + 32 > 65536) return CKQ_EUNFUSED;
-    int nrows = 0;
-    for (int i = 0; i < n; ++i) {
-        if (rows[i] <= 0 || !W[i] || !X[i] || !y[i] || ldys[i] < rows[i] || ldys[i] > 0x7fffffff) return CKQ_EINVAL;
-        if (rows[i] > nrows) nrows = rows[i];
-    }
-    hipStream_t s = (hipStream_t)stream;
-    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(s, &cap) != hipSuccess) { (void)hipGetLastError(); return CKQ_EUNFUSED; }
-    if (cap != hipStreamCaptureStatusNone) return CKQ_EUNFUSED;
-
-    std::lock_guard<std::recursive_mutex> lock(g_split_mu);
-    unsigned *flag, *epoch;
-    int rc = pro_counter(s, &flag, &epoch);
-    if (rc) return rc;
-    GemvPro pro = {};
-    pro.src = src; pro.src2 = src2; pro.dst = (uint8_t *)dst; pro.flag = flag; pro.target = *epoch;
-    pro.spin_limit = g_pro_spin_limit.load(std::memory_order_relaxed);
-    { static const int nap = getenv("CKQ_PRO_NAP") ? atoi(getenv("CKQ_PRO_NAP")) : 1; pro.nap = nap > 0 ? nap : 1; }
-    pro.kind = kind; pro.rows = pro_rows; pro.k = pro_k; pro.ld = pro_ld; pro.eps = eps;
-    int pro_blocks = 0;
-    GemvArgs a = {};
-    GemvGroup grp = k_no_group;
-    a.y = y[0]; a.W = (const uint8_t *)W[0]; a.X = (const uint8_t *)X[0]; a.bias = bias ? bias[0] : nullptr; a.sub = nullptr;
-    a.nrows = nrows; a.ntok = ntok; a.row0 = 0; a.row1 = rows[0]; a.ldy = ldys[0];
-    a.pro = &pro; a.pro_blocks = &pro_blocks;
-    for (int i = 1; i < n; ++i) {
-        grp.y[i - 1] = y[i]; grp.W[i - 1] = (const uint8_t *)W[i]; grp.X[i - 1] = (const uint8_t *)X[i];
-        grp.bias[i - 1] = bias ? bias[i] : nullptr;
-        grp.nrows[i - 1] = rows[i];
-        grp.ldy[i - 1] = (int)ldys[i];
-    }
-    grp.n = n;
-    rc = launch_gemv_args(fmt, a, grp, K, stream);
-    if (rc == 0) *epoch += (unsigned)pro_blocks;
-    return rc;
-}
-
 static int launch_gemv_args(int fmt_flags, GemvArgs &a, const GemvGroup &grp, int K, void *stream, const GemmOpts &opts)
 {
     int fmt = fmt_flags;
@@ -434,9 +337,7 @@ static int launch_gemv_args(int fmt_flags, GemvArgs &a, const GemvGroup &grp, in
     const long ldy = a.ldy;
     hipStream_t s = (hipStream_t)stream;
     const bool dump = a.sub != nullptr;
-    if (a.pro && (dump || ntok > CKQ_STREAM_TOKENS || (fmt != CKQ_FMT_Q4_K && fmt != CKQ_FMT_Q5_K && fmt != CKQ_FMT_Q6_K)))
-        return CKQ_EINVAL;
-    const bool whole = !a.pro && !dump && grp.n == 1 && row0 == 0 && row1 == nrows;   /* what a matrix-core GEMM can take */
+    const bool whole = !dump && grp.n == 1 && row0 == 0 && row1 == nrows;   /* what a matrix-core GEMM can take */
     switch (fmt) {
     case CKQ_FMT_Q4_K:
         if (K % 256) return CKQ_ESHAPE;

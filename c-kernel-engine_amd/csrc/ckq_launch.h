@@ -19,7 +19,6 @@ extern "C" {
 #define CKQ_ESHAPE  (-2)  /* K not a multiple of the block size */
 #define CKQ_EFORMAT (-3)  /* unknown format tag */
 #define CKQ_ESCRATCH (-4) /* the call needs more scratch than the entry point that allocates nothing holds */
-#define CKQ_EUNFUSED (-5) /* internal: this producer + matmul combination has no fused launch; nothing was enqueued */
 
 /* Weight-format tags as in ckq_blocks.h, plus the fp32-activation variants
  * (X is then ntok rows of K floats). */
@@ -90,18 +89,7 @@ int ckq_launch_dequant_rows(int fmt, const void *table, const int32_t *ids, int 
  * device (once per device; also done by the first call on a device). */
 #define CKQ_NOALLOC_SCRATCH_BYTES ((size_t)4 << 20)
 int ckq_launch_noalloc_setup(void);
-/* A producer step (kind 1 = fp32 -> Q8_K, 2 = RMSNorm -> Q8_K with gamma at src2, 3 = SiLU(src) * src2 -> Q8_K;
- * pro_rows rows of pro_k floats, pro_ld apart, blocks to dst) and the n (1..4) matmuls that read dst, as one
- * launch: the matmul blocks stream their weights while the producer blocks run.  CKQ_EUNFUSED = no fused form
- * for this combination, nothing enqueued. */
-int ckq_launch_gemv_pro(int fmt, int n, float *const *y, const void *const *W, const void *const *X,
-                        const float *const *bias, const int *rows, const long *ldys, int K, int ntok,
-                        int kind, const float *src, const float *src2, void *dst, int pro_rows, int pro_k,
-                        long pro_ld, float eps, void *stream);
-/* Bound of a matmul block's wait for the producers (polls; <= 0 restores the default) and the number of
- * waits that expired on `stream` so far (synchronises the stream). */
-void ckq_launch_set_pro_spin_limit(int polls);
-int ckq_launch_pro_timeouts(void *stream, unsigned *count);
+
 /* Frees the K-split / rewrite scratch held for `stream` on the current device. */
 int ckq_launch_release_stream(void *stream);
 

@@ -1,37 +1,10 @@
 /*
  * ckq_producers.hpp - the activation producers (fp32 -> Q8_K, SiLU(gate)*up ->
- * Q8_K, RMSNorm -> Q8_K) as device functions, shared by their stand-alone
- * kernels and by the producer blocks at the front of a fused matmul launch, so
- * that both write the same bits; and the completion counter through which the
- * matmul blocks of such a launch learn that their activations exist.
- *
- * A fused launch (gemv_pro_kernel): the first `nblocks` blocks of grid x run
- * the producer, every other block is a matmul block that waits, resident and
- * with nothing in flight, until the producers have counted up to `target`,
- * and then runs as it would in a launch of its own.  What the fusion saves is
- * the boundary between two dependent launches (the producer's end-of-kernel
- * cache write-back, the next dispatch, its ramp): the matmul's waves are
- * already on the chip when the activations appear.  Block 0 is dispatched
- * first and never waits for anything, so the wait always ends; it is bounded
- * all the same (spin_limit polls), and an expired wait is recorded in flag[1].
+ * Q8_K, RMSNorm -> Q8_K) as device functions: the arithmetic of the stand-alone
+ * producer kernels of ckq_kernels.hip, kept apart from their launch shapes.
  */
 #pragma once
 #include "ckq_device.hpp"
-
-enum { CKQ_PRO_QUANT_Q8K = 1, CKQ_PRO_RMSNORM_Q8K = 2, CKQ_PRO_SWIGLU_Q8K = 3 };
-
-struct GemvPro {
-    const float *src;      /* fp32 rows (the gate rows of SwiGLU) */
-    const float *src2;     /* gamma (RMSNorm) / up rows (SwiGLU) / unused */
-    uint8_t     *dst;      /* rows x (k/256) Q8_K blocks */
-    unsigned    *flag;     /* flag[0]: producer blocks completed since the counter was created; flag[1]: expired waits */
-    unsigned     target;   /* flag[0] once every producer block of this launch has finished */
-    int          spin_limit;
-    int          nap;      /* naps of ~0.25 us between two polls of a waiting block */
-    int          kind, nblocks, rows, k;
-    long         ld;       /* floats between rows of src (and src2 for SwiGLU) */
-    float        eps;
-};
 
 /* ---- SiLU(gate) * up as the reference's tile loop evaluates it -------------
  * (fused/prefill_fused_gemm.c:904-906, 1034-1040): g / (1 + expf(-g)), then
@@ -158,62 +131,4 @@ __device__ __forceinline__ void rms_row(const float *__restrict__ x, const float
     for (int b = wave + NW * GREG; b < nb; b += NW)
         rms_quant_block(reinterpret_cast<const float4 *>(xs + 256 * b)[lane],
                         reinterpret_cast<const float4 *>(gamma + 256 * b)[lane], rstd, lane, y + (size_t)b * 292);
-}
-
-/* ---- producer blocks and the completion counter of a fused launch --------- */
-
-/* Producer block `pb` of a fused launch (a block of WPB waves). */
-template <int WPB>
-__device__ __forceinline__ void pro_block(const GemvPro &pro, int pb, uint8_t *smem)
-{
-    const int lane = threadIdx.x & 63, wave = wave_in_block();
-    const int bpr = pro.k / 256;
-    if (pro.kind == CKQ_PRO_RMSNORM_Q8K) {
-        if (pb < pro.rows)
-            rms_row<WPB, 8 / WPB>(pro.src + (size_t)pb * pro.ld, pro.src2, pro.dst + (size_t)pb * bpr * 292, pro.k, pro.eps,
-                                   reinterpret_cast<float *>(smem));
-    } else {
-        const long blk = (long)pb * WPB + wave, total = (long)pro.rows * bpr;
-        if (blk < total) {
-            if (pro.kind == CKQ_PRO_SWIGLU_Q8K) pro_quantize_block<true>(pro.src, pro.src2, pro.dst, blk, bpr, pro.ld, lane);
-            else pro_quantize_block<false>(pro.src, nullptr, pro.dst, blk, bpr, pro.ld, lane);
-        }
-    }
-    /* every wave makes its stores visible to the device, then one thread counts the block */
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-    __syncthreads();
-    if (threadIdx.x == 0) __hip_atomic_fetch_add(pro.flag, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-/* Number of producer blocks of WPB waves each. */
-static inline int pro_block_count(int kind, int rows, int k, int wpb)
-{
-    if (kind == CKQ_PRO_RMSNORM_Q8K) return rows;
-    const long total = (long)rows * (k / 256);
-    return (int)((total + wpb - 1) / wpb);
-}
-
-/* A matmul block of a fused launch: wait (bounded) until the producers of this
- * launch have all counted.  The activations are read only after this, with
- * ordinary loads and WITHOUT a cache invalidate: the producers have written
- * them back to memory (their release), and no cache on the reader's side can
- * hold an older copy of those lines - the launch began with the queue's
- * acquire, no matmul block touches the activations before its wait has ended,
- * and the host refuses to fuse when their cache lines are shared with anything
- * the matmul blocks read earlier (the weights).  An invalidate per block would
- * be correct too, but one per block of a launch of thousands costs ten times
- * the launch (measured: 36-91 us against 8-12). */
-__device__ __forceinline__ void pro_wait(const GemvPro &pro)
-{
-    if (threadIdx.x == 0) {
-        int n = 0;
-        while ((int)(__hip_atomic_load(pro.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - pro.target) < 0) {
-            if (++n > pro.spin_limit) {
-                __hip_atomic_fetch_add(pro.flag + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                break;
-            }
-            for (int k = 0; k < pro.nap; ++k) __builtin_amdgcn_s_sleep(8);     /* ~0.25 us per nap */
-        }
-    }
-    __syncthreads();
 }

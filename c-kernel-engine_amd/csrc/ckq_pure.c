@@ -7,6 +7,8 @@
 
 uint64_t ckq_fingerprint(const void *p, size_t bytes)
 {
+    /* FNV-1a-style mixing over 64 samples of 64 bytes spread across the range, eight bytes at a
+     * time (a byte-wise hash of the same 4 KB costs 3.5 us of every host-pointer call) */
     const uint8_t *b = (const uint8_t *)p;
     uint64_t h = 0xcbf29ce484222325ull ^ bytes;
     const size_t chunk = 64, n = 64;
@@ -14,8 +16,14 @@ uint64_t ckq_fingerprint(const void *p, size_t bytes)
     for (size_t i = 0; i < n; ++i) {
         size_t off = i * step;
         if (off >= bytes) break;
-        size_t len = bytes - off < chunk ? bytes - off : chunk;
-        for (size_t j = 0; j < len; ++j) h = (h ^ b[off + j]) * 0x100000001b3ull;
+        size_t len = bytes - off < chunk ? bytes - off : chunk, j = 0;
+        for (; j + 8 <= len; j += 8) {
+            uint64_t w;
+            memcpy(&w, b + off + j, 8);
+            h = (h ^ w) * 0x100000001b3ull;
+            h ^= h >> 29;
+        }
+        for (; j < len; ++j) h = (h ^ b[off + j]) * 0x100000001b3ull;
     }
     return h;
 }

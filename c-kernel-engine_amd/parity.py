@@ -143,9 +143,13 @@ def dev_quantize(x_t, fmt="q8_k", rows=1):
     return out
 
 
+ACT_F32 = 0x200
+
+
 def fmt_tag(name):
-    """Weight-format tag of a format name."""
-    return FMT[name]
+    """Weight-format tag of a format name; "<fmt>+f32" adds CKQ_ACT_F32 (a sequence entry
+    with fp32 activations, no quantization)."""
+    return FMT[name[:-4]] | ACT_F32 if name.endswith("+f32") else FMT[name]
 
 
 def dev_gemm_nt(fmt, A_t, B_t, bias_t, M, N, K, out=None):

@@ -295,25 +295,11 @@ int ckq_gemm_nt_f32act_dev(int fmt, const float *A, const void *B, const float *
  *                           apart (0 = K), gamma at B, epsilon in eps (rmsnorm_q8_k_fused)
  *   CKQ_STEP_SWIGLU_Q8_K    C = Q8_K(SiLU(gate) * up): gate at A_q8, up at B, M rows of K floats, rows
  *                           ldc floats apart (0 = K) (ckq_swiglu_q8_k_dev)
- * N and bias are unused by producer entries; C is the block buffer.
- * A Q8_K producer entry followed directly by matmul entries (one, or a group
- * as above; Q4_K / Q5_K / Q6_K weights, at most eight tokens) that all read
- * its output can go out as ONE launch with them: the producer runs in the
- * first blocks of the grid, the matmul blocks are resident behind them and
- * wait on a device counter before they start, which saves the boundary
- * between two dependent launches.  Every buffer gets the bits of the unfused
- * steps.  ckq_set_fused_producers: 1 (default) fuses where that was measured
- * to pay - the plain and the SiLU*up quantizer in front of at most 12 MB of
- * weights (1.2 to 2.3 us per pair; larger matmuls and RMSNorm lose) -, 2
- * wherever a fused form exists, 0 never.  Not taken while the stream is being
- * captured (the counter's expected value is baked into the launch), when the
- * matmuls write the producer's input, or when the producer's output shares a
- * cache line with their weights.  The counter is two dwords of
- * device memory per stream, created on the first such launch (released by
- * ckq_release_stream); a matmul block's wait is bounded, and waits that
- * expired - none unless a producer block died - are counted:
- * ckq_fused_producer_timeouts returns their number for `stream` so far
- * (synchronises the stream; negative = error). */
+ * N and bias are unused by producer entries; C is the block buffer. */
+/* Added to a matmul entry's weight tag (CKQ_FMT_Q4_K, _Q6_K or _Q8_0): the
+ * activations at A_q8 are M rows of K floats and the entry computes what
+ * ckq_gemm_nt_f32act_dev computes (no activation quantization). */
+#define CKQ_ACT_F32 0x200
 #define CKQ_STEP_QUANTIZE_Q8_K 32
 #define CKQ_STEP_QUANTIZE_Q8_0 33
 #define CKQ_STEP_RMSNORM_Q8_K  34
@@ -331,8 +317,6 @@ typedef struct {
     float        eps;    /* CKQ_STEP_RMSNORM_Q8_K only */
 } ckq_matmul_op;
 int ckq_matmul_sequence_dev(const ckq_matmul_op *ops, int nops, int repeat, void *stream);
-void ckq_set_fused_producers(int mode);
-int  ckq_fused_producer_timeouts(void *stream);
 
 /* Raw integer sub-block dots of W (M rows) against one activation row, as the
  * GEMV kernel computes them: out[row*(K/sub) + i], sub = 32 (Q4_K, Q5_K, Q8_0)

@@ -995,6 +995,8 @@ typedef struct {
     const void *W, *x;
     int M, K, ith, nth, iters;
     time_gate *gate;
+    size_t w_stride;           /* round i reads the weight copy at W + (i % w_copies) * w_stride */
+    int    w_copies;
 } time_arg;
 
 static void *time_main(void *p)
@@ -1007,7 +1009,7 @@ static void *time_main(void *p)
     if (go < 0) return NULL;
     for (int i = 0; i < a->iters; ++i) {
         pthread_barrier_wait(&a->gate->bar);
-        a->fn(a->y, a->W, a->x, a->M, a->K, a->ith, a->nth);
+        a->fn(a->y, (const uint8_t *)a->W + (size_t)(i % a->w_copies) * a->w_stride, a->x, a->M, a->K, a->ith, a->nth);
         pthread_barrier_wait(&a->gate->bar);
     }
     return NULL;
@@ -1016,7 +1018,16 @@ static void *time_main(void *p)
 int orc_time_split_gemv(orc_split_gemv_fn fn, float *y, const void *W, const void *x_q8, int M, int K, int nth, int iters,
                         double *seconds)
 {
-    if (!fn || !y || !W || !x_q8 || !seconds || M <= 0 || K <= 0 || nth < 1 || nth > 256 || iters < 1) return -1;
+    return orc_time_split_gemv_rotating(fn, y, W, 0, 1, x_q8, M, K, nth, iters, seconds);
+}
+
+/* The same with `w_copies` copies of the weights, `w_stride` bytes apart: round i
+ * reads copy i % w_copies, so that with enough copies the weights come from DRAM
+ * and not from the last-level cache. */
+int orc_time_split_gemv_rotating(orc_split_gemv_fn fn, float *y, const void *W, size_t w_stride, int w_copies,
+                                 const void *x_q8, int M, int K, int nth, int iters, double *seconds)
+{
+    if (!fn || !y || !W || !x_q8 || !seconds || M <= 0 || K <= 0 || nth < 1 || nth > 256 || iters < 1 || w_copies < 1) return -1;
     time_gate gate;
     if (pthread_barrier_init(&gate.bar, NULL, (unsigned)nth)) return -1;
     pthread_mutex_init(&gate.mu, NULL);
@@ -1026,7 +1037,7 @@ int orc_time_split_gemv(orc_split_gemv_fn fn, float *y, const void *W, const voi
     time_arg  arg[256];
     int made = 1;
     for (; made < nth; ++made) {
-        arg[made] = (time_arg){fn, y, W, x_q8, M, K, made, nth, iters, &gate};
+        arg[made] = (time_arg){fn, y, W, x_q8, M, K, made, nth, iters, &gate, w_stride, w_copies};
         if (pthread_create(&tid[made], NULL, time_main, &arg[made])) break;
     }
     const int ok = made == nth;      /* a thread short: the barrier would never open, so nobody enters it */
@@ -1038,7 +1049,7 @@ int orc_time_split_gemv(orc_split_gemv_fn fn, float *y, const void *W, const voi
         struct timespec t0, t1;
         pthread_barrier_wait(&gate.bar);
         clock_gettime(CLOCK_MONOTONIC, &t0);
-        fn(y, W, x_q8, M, K, 0, nth);
+        fn(y, (const uint8_t *)W + (size_t)(i % w_copies) * w_stride, x_q8, M, K, 0, nth);
         pthread_barrier_wait(&gate.bar);
         clock_gettime(CLOCK_MONOTONIC, &t1);
         seconds[i] = (double)(t1.tv_sec - t0.tv_sec) + 1e-9 * (double)(t1.tv_nsec - t0.tv_nsec);

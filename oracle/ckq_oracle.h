@@ -61,6 +61,9 @@ void orc_gemv_q4_k_q8_k(float *y, const void *W, const void *x_q8, int M, int K)
 typedef void (*orc_split_gemv_fn)(float *y, const void *W, const void *x_q8, int M, int K, int ith, int nth);
 int orc_time_split_gemv(orc_split_gemv_fn fn, float *y, const void *W, const void *x_q8, int M, int K, int nth, int iters,
                         double *seconds);
+/* ... over w_copies copies of the weights, w_stride bytes apart, one per round in turn (DRAM-resident weights). */
+int orc_time_split_gemv_rotating(orc_split_gemv_fn fn, float *y, const void *W, size_t w_stride, int w_copies,
+                                 const void *x_q8, int M, int K, int nth, int iters, double *seconds);
 void orc_gemv_q4_k_q8_k_parallel(float *y, const void *W, const void *x_q8, int M, int K, int ith, int nth); /* :212-243 */
 void orc_gemv_q5_k_q8_k(float *y, const void *W, const void *x_q8, int M, int K);      /* gemm_kernels_q5_k.c:130-208,305-329 */
 void orc_gemv_q5_k(float *y, const void *W, const float *x, int M, int K);             /* gemm_kernels_q5_k.c:369-391 (K%256==0 branch) */

@@ -383,159 +383,64 @@ def test_sequence_with_producer_steps():
     assert T.norm_err(one["y"].cpu().numpy(), T.oracle_gemv("q6_k", Wd, one["hq"].cpu().numpy(), D, F)) <= TOL
 
 
-# ---- producers fused with the matmuls that read them ------------------------------------------------------
+# ---- producer steps in a sequence, one activation buffer reused ------------------------------------------
 
-def _fused_vs_separate(steps_of, names):
-    """Runs the step list once as ONE sequence call (producers fuse with the matmuls behind them)
-    and once with fusion switched off; every buffer must hold the same bits; no wait expired."""
-    import torch
-    L = ckq.lib()
-    one, sep = steps_of(), steps_of()
-    L.ckq_set_fused_producers(2)                 # every combination that has a fused form, not only those that pay
-    try:
-        P.dev_matmul_sequence(one[0], repeat=2)
-        L.ckq_set_fused_producers(0)
-        P.dev_matmul_sequence(sep[0], repeat=2)
-    finally:
-        L.ckq_set_fused_producers(1)
-    torch.cuda.synchronize()
-    for name in names:
-        assert torch.equal(one[1][name], sep[1][name]), name
-    assert L.ckq_fused_producer_timeouts(P._stream()) == 0
-    return one[1]
-
-
-@pytest.mark.parametrize("fmt", ["q4_k", "q5_k", "q6_k"])
-def test_fused_producer_launch_matches_separate_steps(fmt):
-    """A Q8_K producer (plain quantizer, RMSNorm, SiLU(gate)*up) and the matmul
-    behind it as one launch - the matmul blocks stream their weights while the
-    producer blocks at the front of the grid run, then wait for their count -
-    has the bits of the two steps issued one after the other, for every token
-    tile and lane mapping, with zero blocks, ties for the largest magnitude and a
-    partial last tile; the producers are bit-exact with the oracle."""
+def test_sequence_steps_reuse_one_activation_buffer():
+    """Consecutive (quantizer, matmul) pairs of one sequence call write DIFFERENT
+    activations into the same Q8_K buffer (as every layer of a model does), for
+    the three producers and one to eight tokens: each matmul sees its own
+    producer's blocks; the producers are bit-exact with the oracle."""
     import torch
     f32 = lambda n: torch.zeros(n, dtype=torch.float32, device="cuda")
-    u8 = lambda n: torch.zeros(n, dtype=torch.uint8, device="cuda")
-    for (N, K), Ms in (((70, 256), (1, 3)), ((300, 1024), (1, 2)), ((129, 2048), (1, 5)), ((512, 4096), (1, 2, 4, 8)),
-                       ((96, 11008), (1, 2, 3)), ((9000, 512), (1,)), ((2100, 4096), (1,)), ((40, 14336), (1, 2))):
-        W = P.to_device(T.synth_weights(fmt, N, K, seed=N + K))
-        gam = T.normal(K, 1.0, 0.2, seed=K)
-        gam_t = P.to_device(gam)
-        for M in Ms:
-            x = T.normal(M * K, 0.0, 1.0, seed=3 * N + M)
-            u = T.normal(M * K, 0.0, 1.0, seed=5 * N + M)
-            x[:256] = 0.0                                  # an all-zero block
-            if K >= 512:
-                x[256:512] = np.where(np.arange(256) % 2 == 0, 0.75, -0.75)   # every element ties for the maximum
-            x_t, u_t = P.to_device(x), P.to_device(u)
-            for kind in ("quantize_q8_k", "rmsnorm_q8_k", "swiglu_q8_k"):
-                say(f"fused producer {kind} + {fmt} {N}x{K} M={M}")
-
-                def steps_of():
-                    b = dict(xq=u8(M * T.row_bytes("q8_k", K)), y=f32(M * N))
-                    pro = {"quantize_q8_k": ("quantize_q8_k", x_t, None, b["xq"], M, K),
-                           "rmsnorm_q8_k": ("rmsnorm_q8_k", x_t, gam_t, b["xq"], M, K, K, 1e-5),
-                           "swiglu_q8_k": ("swiglu_q8_k", x_t, u_t, b["xq"], M, K, K)}[kind]
-                    return [pro, (fmt, b["xq"], W, None, b["y"], M, N, K)], b
-
-                got = _fused_vs_separate(steps_of, ("xq", "y"))
-                xq = got["xq"].cpu().numpy()
-                if kind == "quantize_q8_k":
-                    assert np.array_equal(xq, T.oracle_quantize(x, "q8_k", rows=M))
-                elif kind == "rmsnorm_q8_k":
-                    want = np.zeros_like(xq)
-                    T.oracle().orc_rmsnorm_q8_k_fused(T.ptr(x), T.ptr(gam), T.ptr(want), M, K, K, ctypes.c_float(1e-5))
-                    assert np.array_equal(xq, want)
-                assert T.norm_err(got["y"].cpu().numpy(), T.oracle_gemm_nt(fmt, xq, T.synth_weights(fmt, N, K, seed=N + K),
-                                                                           None, M, N, K)) <= TOL
-
-
-def test_fused_producer_with_grouped_matmuls():
-    """RMSNorm -> Q8_K in front of Q/K/V and of gate/up (grouped launches of
-    unequal row counts), at one and at three tokens and at a 7B layer's widths:
-    the bits of the separate steps."""
-    import torch
-    f32 = lambda n: torch.zeros(n, dtype=torch.float32, device="cuda")
-    u8 = lambda n: torch.zeros(n, dtype=torch.uint8, device="cuda")
-    for D, rows, Ms in ((1024, (1024, 256, 256), (1, 3)), (4096, (11008, 11008), (1, 8)), (4096, (4096, 1024, 1024), (1, 2))):
-        Ws = [P.to_device(T.synth_weights("q4_k", n, D, seed=194 + i)) for i, n in enumerate(rows)]
-        gam_t = P.to_device(T.normal(D, 1.0, 0.2, seed=D))
-        for M in Ms:
-            x_t = P.to_device(T.normal(M * D, 0.0, 1.0, 191 + M))
-            say(f"fused RMSNorm + grouped matmuls D={D} rows={rows} M={M}")
-
-            def steps_of():
-                b = dict(xq=u8(M * T.row_bytes("q8_k", D)))
-                for i, n in enumerate(rows):
-                    b["y%d" % i] = f32(M * n)
-                return ([("rmsnorm_q8_k", x_t, gam_t, b["xq"], M, D, D, 1e-5)] +
-                        [("q4_k", b["xq"], Ws[i], None, b["y%d" % i], M, n, D) for i, n in enumerate(rows)]), b
-
-            _fused_vs_separate(steps_of, ["xq"] + ["y%d" % i for i in range(len(rows))])
-
-
-def test_fused_launches_reuse_one_activation_buffer():
-    """Consecutive fused launches write DIFFERENT activations into the same Q8_K
-    buffer (as every layer of a model does): each matmul must see its own
-    producer's blocks, never a cached copy of the previous launch's."""
-    import torch
-    f32 = lambda n: torch.zeros(n, dtype=torch.float32, device="cuda")
-    N, K, R = 11008, 4096, 6
+    N, K, R = 3000, 4096, 4
     W = P.to_device(T.synth_weights("q4_k", N, K, seed=17))
-    for M in (1, 4):
-        xs = [P.to_device(T.normal(M * K, 0.0, 1.0 + r, seed=300 + r)) for r in range(R)]
+    gam = T.normal(K, 1.0, 0.2, seed=18)
+    gam_t = P.to_device(gam)
+    for M in (1, 4, 8):
+        xs = [T.normal(M * K, 0.0, 1.0 + r, seed=300 + r) for r in range(R)]
+        xs_t = [P.to_device(x) for x in xs]
         xq = torch.zeros(M * T.row_bytes("q8_k", K), dtype=torch.uint8, device="cuda")
         ys = [f32(M * N) for _ in range(R)]
+        kinds = ["quantize_q8_k", "rmsnorm_q8_k", "swiglu_q8_k", "quantize_q8_k"]
         steps = []
         for r in range(R):
-            steps += [("quantize_q8_k", xs[r], None, xq, M, K), ("q4_k", xq, W, None, ys[r], M, N, K)]
-        say(f"fused launches sharing one activation buffer M={M}")
-        ckq.lib().ckq_set_fused_producers(2)
-        try:
-            P.dev_matmul_sequence(steps, repeat=3)
-        finally:
-            ckq.lib().ckq_set_fused_producers(1)
+            pro = {"quantize_q8_k": ("quantize_q8_k", xs_t[r], None, xq, M, K),
+                   "rmsnorm_q8_k": ("rmsnorm_q8_k", xs_t[r], gam_t, xq, M, K, K, 1e-5),
+                   "swiglu_q8_k": ("swiglu_q8_k", xs_t[r], xs_t[(r + 1) % R], xq, M, K, K)}[kinds[r]]
+            steps += [pro, ("q4_k", xq, W, None, ys[r], M, N, K)]
+        say(f"producer steps sharing one activation buffer M={M}")
+        P.dev_matmul_sequence(steps, repeat=2)
         torch.cuda.synchronize()
         for r in range(R):
-            want = P.dev_gemm_nt("q4_k", P.dev_quantize(xs[r], "q8_k", rows=M), W, None, M, N, K).view(-1)
-            assert torch.equal(ys[r], want), r
-    assert ckq.lib().ckq_fused_producer_timeouts(P._stream()) == 0
+            if kinds[r] == "quantize_q8_k":
+                want_q = T.oracle_quantize(xs[r], "q8_k", rows=M)
+            elif kinds[r] == "rmsnorm_q8_k":
+                want_q = np.zeros(M * T.row_bytes("q8_k", K), np.uint8)
+                T.oracle().orc_rmsnorm_q8_k_fused(T.ptr(xs[r]), T.ptr(gam), T.ptr(want_q), M, K, K, ctypes.c_float(1e-5))
+            else:
+                want_q = P.dev_swiglu_q8_k(xs_t[r], xs_t[(r + 1) % R], M, K, K).cpu().numpy()
+            want = P.dev_gemm_nt("q4_k", P.to_device(want_q), W, None, M, N, K).view(-1)
+            assert torch.equal(ys[r], want), (M, r)
 
 
-def test_fused_producer_is_not_taken_when_it_cannot_be():
-    """Steps with no fused form go out one by one with the same results: a Q8_0
-    consumer, a matmul that does not read the producer's output, more than eight
-    tokens, a matmul that overwrites the producer's input."""
+def test_sequence_with_fp32_activation_entries():
+    """A sequence entry tagged CKQ_ACT_F32 computes what ckq_gemm_nt_f32act_dev
+    computes, between ordinary entries."""
     import torch
-    f32 = lambda n: torch.zeros(n, dtype=torch.float32, device="cuda")
-    u8 = lambda n: torch.zeros(n, dtype=torch.uint8, device="cuda")
-    N, K = 320, 1024
-    W4 = P.to_device(T.synth_weights("q4_k", N, K, seed=7))
-    W8 = P.to_device(T.synth_weights("q8_0", N, K, seed=8))
-    for M in (1, 12):
-        x = T.normal(M * K, 0.0, 1.0, seed=70 + M)
-        x_t = P.to_device(x)
-        xq, x0, other = u8(M * T.row_bytes("q8_k", K)), u8(M * T.row_bytes("q8_0", K)), P.dev_quantize(x_t, "q8_k", rows=M)
-        y4, y8, yo = f32(M * N), f32(M * N), f32(M * N)
-        say(f"unfusable sequences M={M}")
-        P.dev_matmul_sequence([("quantize_q8_k", x_t, None, xq, M, K), ("q4_k", other, W4, None, yo, M, N, K),
-                               ("q4_k", xq, W4, None, y4, M, N, K),
-                               ("quantize_q8_0", x_t, None, x0, M, K), ("q8_0", x0, W8, None, y8, M, N, K)])
+    N, K, M = 300, 1024, 2
+    x = T.normal(M * K, 0.0, 1.0, seed=81)
+    x_t = P.to_device(x)
+    for fmt in ("q4_k", "q6_k", "q8_0"):
+        W = P.to_device(T.synth_weights(fmt, N, K, seed=82))
+        xq = P.dev_quantize(x_t, T.act_fmt(fmt), rows=M)
+        y0 = torch.zeros(M * N, dtype=torch.float32, device="cuda")
+        y1, y2 = torch.zeros_like(y0), torch.zeros_like(y0)
+        say("sequence with fp32-activation entry", fmt)
+        P.dev_matmul_sequence([(fmt, xq, W, None, y0, M, N, K), (fmt + "+f32", x_t, W, None, y1, M, N, K),
+                               (fmt, xq, W, None, y2, M, N, K)])
         torch.cuda.synchronize()
-        assert torch.equal(y4, yo)
-        assert np.array_equal(xq.cpu().numpy(), T.oracle_quantize(x, "q8_k", rows=M))
-        assert torch.equal(y8, P.dev_gemm_nt("q8_0", x0, W8, None, M, N, K).view(-1))
-    # the matmul writes the producer's own input: the steps must run in order
-    M, K2 = 1, 1024
-    buf = P.to_device(T.normal(K2, 0.0, 1.0, seed=75))
-    ref = buf.clone()
-    xq, xq2 = u8(T.row_bytes("q8_k", K2)), u8(T.row_bytes("q8_k", K2))
-    Wsq = P.to_device(T.synth_weights("q4_k", K2, K2, seed=9))
-    P.dev_matmul_sequence([("quantize_q8_k", buf, None, xq, M, K2), ("q4_k", xq, Wsq, None, buf, M, K2, K2)])
-    want = P.dev_gemm_nt("q4_k", P.dev_quantize(ref, "q8_k", rows=1), Wsq, None, 1, K2, K2).view(-1)
-    torch.cuda.synchronize()
-    assert torch.equal(buf, want)
-    assert ckq.lib().ckq_fused_producer_timeouts(P._stream()) == 0
+        assert torch.equal(y1, P.dev_gemm_nt_f32act(fmt, x_t, W, None, M, N, K).view(-1))
+        assert torch.equal(y0, y2) and torch.equal(y0, P.dev_gemm_nt(fmt, xq, W, None, M, N, K).view(-1))
 
 
 # ---- host-pointer paths with the weight cache off, long contexts ---------------------------------------
