@@ -23,6 +23,7 @@ import json
 import os
 import re
 import statistics
+import subprocess
 import sys
 import time
 
@@ -216,6 +217,21 @@ def drop_in_latency(H, W, xq, rows, K):
                     lambda: pool.gemv_q4_k_q8_k_parallel_dispatch(p(y), p(W), p(xq), rows, K), 100)
         L.ckq_set_parallel_whole(-1)          # back to the library's default
         pool.ck_threadpool_global_destroy()
+    # cold start in a fresh process: loading the shared object (dlopen), ckq_init() (HIP start-up, stream, the
+    # scratch symbol, which loads the code object) and the first kernel
+    code = ("import ctypes, time, numpy as np\n"
+            "t0 = time.perf_counter(); L = ctypes.CDLL(%r); t1 = time.perf_counter()\n"
+            "rc = L.ckq_init(); t2 = time.perf_counter()\n"
+            "x = np.ones(256, np.float32); y = np.zeros(292, np.uint8)\n"
+            "L.quantize_row_q8_k(x.ctypes.data_as(ctypes.c_void_p), y.ctypes.data_as(ctypes.c_void_p), 256); t3 = time.perf_counter()\n"
+            "print(rc, (t1 - t0) * 1e3, (t2 - t1) * 1e3, (t3 - t2) * 1e3)\n" % H.ckq.lib_path())
+    try:
+        r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120)
+        rc, load_ms, init_ms, first_ms = r.stdout.split()[-4:]
+        out["cold_start_ms"] = {"dlopen": round(float(load_ms), 1), "ckq_init": round(float(init_ms), 1),
+                                "first_call": round(float(first_ms), 1), "library_bytes": os.path.getsize(H.ckq.lib_path())}
+    except Exception as e:                              # the timing is informative only
+        out["cold_start_ms"] = {"error": str(e)[:200]}
     return out
 
 

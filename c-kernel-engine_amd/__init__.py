@@ -15,6 +15,8 @@ from .api import (  # noqa: F401
     CkqError,
     build,
     declared_symbols,
+    dump_lib,
+    dump_lib_path,
     lib,
     lib_path,
     row_bytes,

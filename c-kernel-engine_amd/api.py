@@ -27,7 +27,13 @@ def lib_path():
     return os.path.join(CSRC, "libckernel_quant_hip.so")
 
 
-def build(targets=("synth", "hip")):
+def dump_lib_path():
+    """The test build of the same sources: every kernel also exists in a form that stores the
+    integers behind its outputs (the exactness tests' entry points run only there)."""
+    return os.path.join(CSRC, "libckernel_quant_hip_dump.so")
+
+
+def build(targets=("synth", "hip", "dump")):
     """Compile the host helper and the gfx950 library in-tree (hipcc
     cross-compiles without a GPU)."""
     subprocess.run(["make", "-C", CSRC, "-B"] + list(targets), check=True)
@@ -184,6 +190,26 @@ def lib():
             fn.argtypes = args
         _lib = L
     return _lib
+
+
+_dump = None
+
+
+def dump_lib():
+    """The library with the integer-dump instantiations (test infrastructure; the product
+    library answers the dump entry points with CKQ_ENODUMP)."""
+    global _dump
+    if _dump is None:
+        path = dump_lib_path()
+        if not os.path.exists(path):
+            raise CkqError("%s is missing: build it with `make -C %s dump`" % (path, CSRC))
+        L = ctypes.CDLL(path)
+        for name, (res, args) in _SIGS.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _dump = L
+    return _dump
 
 
 def synth_lib():

@@ -388,8 +388,12 @@ int launch_gemm_q4k_mfma(const void *A, const void *B, const float *bias, float 
     const int tiles = g.ntt * g.nnt, sp = gemm_choose_splits(tiles, g.nb);
     const bool two_groups = tiles * sp <= 256 && (g.nb + sp - 1) / sp >= 8;
     if (sums) {
+#if CKQ_WITH_DUMP
         if (two_groups) return gemm_launch_split(gemm_q4k_mfma_kernel<CKQ_GEMM_WPE, 2, true>, g, (unsigned)(g.ntt * nnt8), g.nb, s, 512);
         return gemm_launch_split(gemm_q4k_mfma_kernel<CKQ_GEMM_WPE, 1, true>, g, (unsigned)(g.ntt * nnt8), g.nb, s, 256);
+#else
+        return CKQ_ENODUMP;
+#endif
     }
     if (two_groups) return gemm_launch_split(gemm_q4k_mfma_kernel<CKQ_GEMM_WPE, 2>, g, (unsigned)(g.ntt * nnt8), g.nb, s, 512);
     return gemm_launch_split(gemm_q4k_mfma_kernel<CKQ_GEMM_WPE, 1>, g, (unsigned)(g.ntt * nnt8), g.nb, s, 256);

@@ -325,6 +325,10 @@ int launch_gemm_q5k_mfma(const void *A, const void *B, const float *bias, float 
     g.ntt = (M + GEMM5_BM - 1) / GEMM5_BM;
     g.nnt = (N + GEMM5_BN - 1) / GEMM5_BN;
     const int nnt8 = (g.nnt + 7) / 8 * 8;
+#if CKQ_WITH_DUMP
     if (sums) return gemm_launch_split(gemm_q5k_mfma_kernel<true>, g, (unsigned)(g.ntt * nnt8), g.nb, s);
+#else
+    if (sums) return CKQ_ENODUMP;
+#endif
     return gemm_launch_split(gemm_q5k_mfma_kernel<false>, g, (unsigned)(g.ntt * nnt8), g.nb, s);
 }

@@ -346,10 +346,18 @@ int launch_gemm_q6k_mfma(const void *A, const void *B, const float *bias, float 
     const int ntt4 = (M + 127) / 128;
     if (ntt4 * g.nnt > 128) {
         g.ntt = ntt4;
+#if CKQ_WITH_DUMP
         if (sums) return gemm_launch_split(gemm_q6k_mfma_kernel<4, true>, g, (unsigned)(g.ntt * nnt8), g.nb, s);
+#else
+        if (sums) return CKQ_ENODUMP;
+#endif
         return gemm_launch_split(gemm_q6k_mfma_kernel<4>, g, (unsigned)(g.ntt * nnt8), g.nb, s);
     }
     g.ntt = (M + 63) / 64;
+#if CKQ_WITH_DUMP
     if (sums) return gemm_launch_split(gemm_q6k_mfma_kernel<2, true>, g, (unsigned)(g.ntt * nnt8), g.nb, s);
+#else
+    if (sums) return CKQ_ENODUMP;
+#endif
     return gemm_launch_split(gemm_q6k_mfma_kernel<2>, g, (unsigned)(g.ntt * nnt8), g.nb, s);
 }

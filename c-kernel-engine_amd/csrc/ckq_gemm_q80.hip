@@ -266,6 +266,10 @@ int launch_gemm_q80_mfma(const void *A, const void *B, const float *bias, float 
     g.ntt = (M + GEMM8_BM - 1) / GEMM8_BM;
     g.nnt = (N + GEMM8_BN - 1) / GEMM8_BN;
     const int nnt8 = (g.nnt + 7) / 8 * 8;
+#if CKQ_WITH_DUMP
     if (sums) return gemm_launch_split(gemm_q80_mfma_kernel<true>, g, (unsigned)(g.ntt * nnt8), (g.nb + GEMM8_KB - 1) / GEMM8_KB, s);
+#else
+    if (sums) return CKQ_ENODUMP;
+#endif
     return gemm_launch_split(gemm_q80_mfma_kernel<false>, g, (unsigned)(g.ntt * nnt8), (g.nb + GEMM8_KB - 1) / GEMM8_KB, s);
 }

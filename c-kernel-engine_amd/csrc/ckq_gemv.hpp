@@ -279,11 +279,15 @@ static int launch_tile(const GemvArgs &a, const GemvGroup &grp, hipStream_t s)
 {
     const bool fits = F::xs_lds_bytes((size_t)MT * (size_t)a.xrow) <= 65536;
     if (a.sub) {
+#if CKQ_WITH_DUMP
         if constexpr (F::TOKEN_TILES) {
             if (fits) return launch_one<F, LPR, PPL, MT, RPI, true, WPB, true>(a, grp, s);
             if (MT == 1 && grp.n == 1) return launch_one<F, LPR, PPL, 1, 1, true, 4, false>(a, grp, s);
         }
         return CKQ_EINVAL;
+#else
+        return CKQ_ENODUMP;      /* the dump builds live in libckernel_quant_hip_dump.so */
+#endif
     }
     if (fits) return launch_one<F, LPR, PPL, MT, RPI, false, WPB, true>(a, grp, s);
     return launch_one<F, LPR, PPL, MT, RPI, false, WPB, false>(a, grp, s);

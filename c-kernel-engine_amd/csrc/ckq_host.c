@@ -102,6 +102,7 @@ const char *ckq_error_string(int code)
     case CKQ_EINVAL: return "invalid argument (NULL pointer or non-positive dimension)";
     case CKQ_ESHAPE: return "K is not a multiple of the quantization block size";
     case CKQ_EFORMAT: return "unknown weight format";
+    case CKQ_ENODUMP: return "the integer dumps of the exactness tests are built into libckernel_quant_hip_dump.so, not into this library";
     case CKQ_ESCRATCH: return "the call needs more scratch than ckq_gemm_nt_noalloc_dev holds (4 MiB); use ckq_gemm_nt_dev or fewer tokens per call";
     default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
     }

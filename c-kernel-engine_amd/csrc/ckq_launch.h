@@ -19,6 +19,12 @@ extern "C" {
 #define CKQ_ESHAPE  (-2)  /* K not a multiple of the block size */
 #define CKQ_EFORMAT (-3)  /* unknown format tag */
 #define CKQ_ESCRATCH (-4) /* the call needs more scratch than the entry point that allocates nothing holds */
+#define CKQ_ENODUMP (-6)  /* the integer dumps are compiled into libckernel_quant_hip_dump.so only */
+/* 1 in the test library (same sources, same templates, plus the DUMP instantiations that also
+ * store the integers behind every output); 0 in the product library, which stays smaller for it. */
+#ifndef CKQ_WITH_DUMP
+#define CKQ_WITH_DUMP 0
+#endif
 
 /* Weight-format tags as in ckq_blocks.h, plus the fp32-activation variants
  * (X is then ntok rows of K floats). */

@@ -9,7 +9,7 @@ import ctypes
 
 import numpy as np
 
-from .api import BLOCK_ELEMS, FMT, STEP, MatmulOp, check, lib, row_bytes
+from .api import BLOCK_ELEMS, FMT, STEP, MatmulOp, check, dump_lib, lib, row_bytes
 
 _vp = ctypes.c_void_p
 
@@ -204,7 +204,7 @@ def dev_subblock_dots(fmt, W_t, x_t, M, K):
     import torch
     per = (K // 16) if fmt == "q6_k" else (K // 32)
     out = torch.zeros(M * per, dtype=torch.int32, device=W_t.device)
-    check(lib().ckq_subblock_dots_dev(FMT[fmt], _dp(out), _dp(W_t), _dp(x_t), M, K, _stream()),
+    check(dump_lib().ckq_subblock_dots_dev(FMT[fmt], _dp(out), _dp(W_t), _dp(x_t), M, K, _stream()),
           "ckq_subblock_dots_dev")
     return out.view(M, per)
 
@@ -215,7 +215,7 @@ def dev_subblock_dots_tokens(fmt, W_t, X_t, M, K, ntok):
     import torch
     per = (K // 16) if fmt == "q6_k" else (K // 32)
     out = torch.zeros(ntok * M * per, dtype=torch.int32, device=W_t.device)
-    check(lib().ckq_subblock_dots_tokens_dev(FMT[fmt], _dp(out), _dp(W_t), _dp(X_t), M, K, ntok, _stream()),
+    check(dump_lib().ckq_subblock_dots_tokens_dev(FMT[fmt], _dp(out), _dp(W_t), _dp(X_t), M, K, ntok, _stream()),
           "ckq_subblock_dots_tokens_dev")
     return out.view(ntok, M, per)
 
@@ -229,7 +229,7 @@ def dev_subblock_dots_group(fmt, W_ts, X_ts, rows, K, ntok):
     Wp = (_vp * n)(*[w.data_ptr() for w in W_ts])
     Xp = (_vp * n)(*[x.data_ptr() for x in X_ts])
     rp = (ctypes.c_int * n)(*rows)
-    check(lib().ckq_subblock_dots_group_dev(FMT[fmt], n, _dp(out), ctypes.cast(Wp, _vp), ctypes.cast(Xp, _vp),
+    check(dump_lib().ckq_subblock_dots_group_dev(FMT[fmt], n, _dp(out), ctypes.cast(Wp, _vp), ctypes.cast(Xp, _vp),
                                             ctypes.cast(rp, _vp), K, ntok, _stream()), "ckq_subblock_dots_group_dev")
     return out.view(n, ntok, mx, per)
 
@@ -240,7 +240,7 @@ def dev_gemm_block_sums(fmt, A_t, B_t, bias_t, M, N, K):
     nblk, per = (K // 32, 1) if fmt == "q8_0" else (K // 256, 1 if fmt == "q6_k" else 2)
     c = torch.empty(M * N, dtype=torch.float32, device=B_t.device)
     sums = torch.zeros(M * N * nblk * per, dtype=torch.int32, device=B_t.device)
-    check(lib().ckq_gemm_block_sums_dev(FMT[fmt], _dp(A_t), _dp(B_t), _dp(bias_t), _dp(c), _dp(sums), M, N, K, _stream()),
+    check(dump_lib().ckq_gemm_block_sums_dev(FMT[fmt], _dp(A_t), _dp(B_t), _dp(bias_t), _dp(c), _dp(sums), M, N, K, _stream()),
           "ckq_gemm_block_sums_dev")
     return c.view(M, N), sums.view(M, N, nblk, per)
 

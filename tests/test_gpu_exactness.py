@@ -96,6 +96,25 @@ def test_grouped_launch_subblock_dots_bit_exact(fmt, rows, K, tokens):
         assert not got[g][:, rows[g]:].any()
 
 
+def test_product_library_has_no_dump_kernels():
+    """The integer dumps are test infrastructure: the shipped library answers
+    their entry points with CKQ_ENODUMP (-6) and enqueues nothing; the test
+    build of the same sources (libckernel_quant_hip_dump.so) runs them."""
+    import torch
+    L = ckq.lib()
+    W = P.to_device(T.synth_weights("q4_k", 64, 256, seed=1))
+    x = P.to_device(T.oracle_quantize(T.normal(256, 0.0, 1.0, 2), "q8_k"))
+    out = torch.full((64 * 8,), 77, dtype=torch.int32, device="cuda")
+    assert L.ckq_subblock_dots_dev(P.FMT["q4_k"], P._dp(out), P._dp(W), P._dp(x), 64, 256, P._stream()) == -6
+    c = torch.zeros(64, dtype=torch.float32, device="cuda")
+    assert L.ckq_gemm_block_sums_dev(P.FMT["q4_k"], P._dp(x), P._dp(W), None, P._dp(c), P._dp(out), 1, 64, 256, P._stream()) == -6
+    torch.cuda.synchronize()
+    assert (out == 77).all()
+    assert b"dump" in L.ckq_error_string(-6)
+    assert np.array_equal(P.dev_subblock_dots("q4_k", W, x, 64, 256).cpu().numpy(),
+                          T.oracle_subdots("q4_k", T.synth_weights("q4_k", 64, 256, seed=1), x.cpu().numpy(), 64, 256))
+
+
 # ---- matrix-core GEMMs: integer block sums ----------------------------------------------------------
 
 def np_block_sums(fmt, W, A, M, N, K):
