@@ -321,7 +321,60 @@ PROFILE_WORKLOADS = {
     "gemv_q6_k_4096x11008": ("q6_k", 4096, 11008, 1),
     "gemm_q6_k_M512_4096x11008": ("q6_k", 4096, 11008, 512),
     "gemv_q4_k_4096x4096": ("q4_k", 4096, 4096, 1),
+    "layer_7b_decode_chain_M1": None,        # eight launches per layer: four producers, four (grouped) matmuls
 }
+
+
+def build_7b_layer_steps(H):
+    """Four rotated 7B decoder layers (502 MB of weights): the projection set as matmul
+    entries (`layers`) and the real chain with its activation producers (`chains`)."""
+    torch, P, T = H.torch, H.P, H.T
+    # a 7B decoder layer's projection set at M=1: Q,K,V,O (4096x4096 Q4_K), gate, up
+    # (11008x4096 Q4_K), down (4096x11008 Q6_K), one C call per layer, weights of
+    # successive steps distinct (4 rotated layers = 502 MB).  The sequence call issues
+    # independent same-shape entries as one launch; to keep the dependencies of a real
+    # layer, O reads its activations from V's output buffer, gate/up from O's and down
+    # from up's (the bytes are not meaningful activations; the timing does not care),
+    # so the launches are Q+K+V | O | gate+up | down.
+    x4k = P.dev_quantize(P.to_device(T.normal(4096, seed=31)), "q8_k")
+    layers, keep, lbytes = [], [], 0
+    for li in range(4):
+        ops = []
+        for j, (fmt, r, k) in enumerate([("q4_k", 4096, 4096)] * 4 + [("q4_k", 11008, 4096)] * 2 + [("q6_k", 4096, 11008)]):
+            Wj = torch.from_numpy(T.synth_weights(fmt, r, k, seed=1000 + j)).cuda()
+            if li:
+                Wj = torch.roll(Wj.view(r, -1), shifts=li * 13 + j, dims=0).contiguous().reshape(-1)
+            o = torch.zeros(r, dtype=torch.float32, device="cuda")
+            keep += [Wj, o]
+            src = x4k if j < 3 else ops[2][4] if j == 3 else ops[3][4] if j < 6 else ops[5][4]
+            ops.append((fmt, src, Wj, None, o, 1, r, k))
+            if li == 0:
+                lbytes += gemv_bytes(fmt, r, k)
+        layers.append(ops)
+    # the same layer as the REAL chain, activation quantizers included, one C call per layer:
+    # RMSNorm->Q8_K | Q+K+V | Q8_K(attention output; V's output stands in) | O | RMSNorm->Q8_K |
+    # gate+up | SiLU(gate)*up->Q8_K | down: four matmul launches and four producer launches
+    f32z = lambda n: torch.zeros(n, dtype=torch.float32, device="cuda")
+    u8z = lambda n: torch.zeros(n, dtype=torch.uint8, device="cuda")
+    xres = P.to_device(T.normal(4096, 0.0, 1.0, seed=32))
+    gam = P.to_device(T.normal(4096, 1.0, 0.2, seed=33))
+    chains = []
+    for ops in layers:
+        (q_, k_, v_, o_, g_, u_, d_) = ops
+        xq_, aq_, fq_ = u8z(4672), u8z(4672), u8z(4672)
+        hq_ = u8z(43 * 292)
+        keep += [xq_, aq_, fq_, hq_]
+        chains.append([
+            ("rmsnorm_q8_k", xres, gam, xq_, 1, 4096, 4096, 1e-5),
+            ("q4_k", xq_, q_[2], None, q_[4], 1, 4096, 4096), ("q4_k", xq_, k_[2], None, k_[4], 1, 4096, 4096),
+            ("q4_k", xq_, v_[2], None, v_[4], 1, 4096, 4096),
+            ("quantize_q8_k", v_[4], None, aq_, 1, 4096),
+            ("q4_k", aq_, o_[2], None, o_[4], 1, 4096, 4096),
+            ("rmsnorm_q8_k", o_[4], gam, fq_, 1, 4096, 4096, 1e-5),
+            ("q4_k", fq_, g_[2], None, g_[4], 1, 11008, 4096), ("q4_k", fq_, u_[2], None, u_[4], 1, 11008, 4096),
+            ("swiglu_q8_k", g_[4], u_[4], hq_, 1, 11008, 11008),
+            ("q6_k", hq_, d_[2], None, d_[4], 1, 4096, 11008)])
+    return layers, chains, keep, lbytes
 
 
 def copy_calibration(H):
@@ -338,6 +391,11 @@ def copy_calibration(H):
 
 
 def run_only(H, name, steps, warmup, calibrate):
+    if name == "layer_7b_decode_chain_M1":
+        _, chains, keep, _ = build_7b_layer_steps(H)
+        sc = H.time_sequence(chains, max(4, steps), 3)
+        print(json.dumps({"only": name, "layers_per_repetition": max(4, steps), "repetitions": 4, "median_us_per_layer": round(sc * 1e6, 3)}))
+        return
     fmt, rows, K, M = PROFILE_WORKLOADS[name]
     P, T = H.P, H.T
     _, copies = H.weight_copies(fmt, rows, K, seed=rows + K, min_total=(3 * MALL_BYTES // 2) if M == 1 else 1)
@@ -528,55 +586,11 @@ def main():
                 prod["%s_T%d_us" % (name, tk)] = round(e0.elapsed_time(e1) * 10.0, 2)
         extras["producer_d4096"] = prod
 
-        # a 7B decoder layer's projection set at M=1: Q,K,V,O (4096x4096 Q4_K), gate, up
-        # (11008x4096 Q4_K), down (4096x11008 Q6_K), one C call per layer, weights of
-        # successive steps distinct (4 rotated layers = 502 MB).  The sequence call issues
-        # independent same-shape entries as one launch; to keep the dependencies of a real
-        # layer, O reads its activations from V's output buffer, gate/up from O's and down
-        # from up's (the bytes are not meaningful activations; the timing does not care),
-        # so the launches are Q+K+V | O | gate+up | down.
-        x4k = P.dev_quantize(P.to_device(T.normal(4096, seed=31)), "q8_k")
-        layers, keep, lbytes = [], [], 0
-        for li in range(4):
-            ops = []
-            for j, (fmt, r, k) in enumerate([("q4_k", 4096, 4096)] * 4 + [("q4_k", 11008, 4096)] * 2 + [("q6_k", 4096, 11008)]):
-                Wj = torch.from_numpy(T.synth_weights(fmt, r, k, seed=1000 + j)).cuda()
-                if li:
-                    Wj = torch.roll(Wj.view(r, -1), shifts=li * 13 + j, dims=0).contiguous().reshape(-1)
-                o = torch.zeros(r, dtype=torch.float32, device="cuda")
-                keep += [Wj, o]
-                src = x4k if j < 3 else ops[2][4] if j == 3 else ops[3][4] if j < 6 else ops[5][4]
-                ops.append((fmt, src, Wj, None, o, 1, r, k))
-                if li == 0:
-                    lbytes += gemv_bytes(fmt, r, k)
-            layers.append(ops)
+        layers, chains, keep, lbytes = build_7b_layer_steps(H)
         s = H.time_sequence(layers, 64, 5)
         extras["layer_7b_projection_set_M1"] = {"us": round(s * 1e6, 2), "gbs": round(lbytes / s / 1e9, 1), "bytes": lbytes,
                                                 "frac_hbm": round(lbytes / s / 1e9 / HBM_PEAK_GBS, 4), "launches": 4,
                                                 "note": "Q+K+V and gate+up each as one grouped launch"}
-        # the same layer as the REAL chain, activation quantizers included, one C call per layer:
-        # RMSNorm->Q8_K | Q+K+V | Q8_K(attention output; V's output stands in) | O | RMSNorm->Q8_K |
-        # gate+up | SiLU(gate)*up->Q8_K | down: four matmul launches and four producer launches
-        f32z = lambda n: torch.zeros(n, dtype=torch.float32, device="cuda")
-        u8z = lambda n: torch.zeros(n, dtype=torch.uint8, device="cuda")
-        xres = P.to_device(T.normal(4096, 0.0, 1.0, seed=32))
-        gam = P.to_device(T.normal(4096, 1.0, 0.2, seed=33))
-        chains = []
-        for ops in layers:
-            (q_, k_, v_, o_, g_, u_, d_) = ops
-            xq_, aq_, fq_ = u8z(4672), u8z(4672), u8z(4672)
-            hq_ = u8z(43 * 292)
-            keep += [xq_, aq_, fq_, hq_]
-            chains.append([
-                ("rmsnorm_q8_k", xres, gam, xq_, 1, 4096, 4096, 1e-5),
-                ("q4_k", xq_, q_[2], None, q_[4], 1, 4096, 4096), ("q4_k", xq_, k_[2], None, k_[4], 1, 4096, 4096),
-                ("q4_k", xq_, v_[2], None, v_[4], 1, 4096, 4096),
-                ("quantize_q8_k", v_[4], None, aq_, 1, 4096),
-                ("q4_k", aq_, o_[2], None, o_[4], 1, 4096, 4096),
-                ("rmsnorm_q8_k", o_[4], gam, fq_, 1, 4096, 4096, 1e-5),
-                ("q4_k", fq_, g_[2], None, g_[4], 1, 11008, 4096), ("q4_k", fq_, u_[2], None, u_[4], 1, 11008, 4096),
-                ("swiglu_q8_k", g_[4], u_[4], hq_, 1, 11008, 11008),
-                ("q6_k", hq_, d_[2], None, d_[4], 1, 4096, 11008)])
         sc = H.time_sequence(chains, 64, 5)
         extras["layer_7b_decode_chain_M1"] = {"us": round(sc * 1e6, 2), "matmul_only_us": round(s * 1e6, 2),
                                               "producers_us": round((sc - s) * 1e6, 2), "launches": 8,
