@@ -133,7 +133,7 @@ class Harness:
             run(warmup)
         return summarize(self.timed_reps(run, launches, reps))
 
-    def time_read_floor(self, copies, nbytes, launches=LAUNCHES_PER_REP, reps=5):
+    def time_read_floor(self, copies, nbytes, launches=LAUNCHES_PER_REP, reps=5, tuned_search=True):
         """Seconds per launch of kernels that only pull `nbytes` out of the same
         rotated weight buffers: the one-load-per-lane read, and the fastest of a
         small search over the tuned streaming read (grid = what the chip holds,
@@ -150,6 +150,8 @@ class Harness:
                 L.ckq_read_dev(ptrs[i % n], nbytes, sp, stream)
 
         res = {"plain": summarize(self.timed_reps(plain, launches, reps))[0]}
+        if not tuned_search:
+            return res
         cus = torch.cuda.get_device_properties(0).multi_processor_count
         best = None
         for bpc in (2, 4, 8):
@@ -555,7 +557,9 @@ def main():
             xq = P.dev_quantize(P.to_device(T.normal(k, seed=k)), T.act_fmt(fmt))
             s, _, _ = H.time_gemv(fmt, r, k, 1, cps, xq, 128, 5)
             b = gemv_bytes(fmt, r, k)
-            extras[name] = {"gbs": round(b / s / 1e9, 1), "us": round(s * 1e6, 2), "frac_hbm": round(b / s / 1e9 / HBM_PEAK_GBS, 4)}
+            rd = H.time_read_floor(cps, r * T.row_bytes(fmt, k), 128, 5, tuned_search=False)["plain"]
+            extras[name] = {"gbs": round(b / s / 1e9, 1), "us": round(s * 1e6, 2), "frac_hbm": round(b / s / 1e9 / HBM_PEAK_GBS, 4),
+                            "read_same_bytes_us": round(rd * 1e6, 2), "gemv_over_read": round(s / rd, 3)}
             del cps
             torch.cuda.empty_cache()
         # fp32-activation entry point (gemv_q4_k: weights dequantized on the fly, nothing quantized)
