@@ -153,6 +153,36 @@ __device__ __forceinline__ u32 pk_mad_u16(u32 a, u32 b, u32 c)
     return __builtin_bit_cast(u32, (ckq_v2u16)(x * y + z));
 }
 
+/* acc += u * (lane 16*(l/16) + R of x): the multiply-add takes its first factor
+ * from lane R of the caller's 16-lane row (DPP row_newbcast), so sixteen values
+ * held one per lane serve sixteen instructions without being spread out first.
+ * x must come from memory (LDS), not from a VALU instruction right before. */
+__device__ __forceinline__ float fmac_row_lane(float acc, float x, float u, int r)
+{
+#define CKQ_BC(R) case R: asm("v_fmac_f32_dpp %0, %1, %2 row_newbcast:" #R " row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(x), "v"(u)); break;
+    switch (r) {
+        CKQ_BC(0) CKQ_BC(1) CKQ_BC(2) CKQ_BC(3) CKQ_BC(4) CKQ_BC(5) CKQ_BC(6) CKQ_BC(7)
+        CKQ_BC(8) CKQ_BC(9) CKQ_BC(10) CKQ_BC(11) CKQ_BC(12) CKQ_BC(13) CKQ_BC(14) CKQ_BC(15)
+    }
+#undef CKQ_BC
+    return acc;
+}
+
+/* A value that a VALU instruction computed, made safe as the x of fmac_row_lane: a DPP
+ * instruction must not read a register a VALU instruction wrote in the two issue slots before it. */
+__device__ __forceinline__ float dpp_source(float x)
+{
+    asm volatile("s_nop 1" : "+v"(x));
+    return x;
+}
+
+/* Which token of its 32-token group output r = (lane & 15) of a lane is (the 32x32 MFMA result layout:
+ * register r of lane l is row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32). */
+__device__ __forceinline__ int mfma32_row_of_lane(int lane)
+{
+    return 8 * ((lane & 15) >> 2) + 4 * (lane >> 5) + (lane & 3);
+}
+
 /* The four kernels, one translation unit each: C[m*ldc + n] = dot(B row n, A row m) (+ bias[n]).
  * See GemmOpts for the options. */
 int launch_gemm_q4k_mfma(const void *A, const void *B, const float *bias, float *C, int M, int N, int K, long ldc, const GemmOpts &opts, hipStream_t s);

@@ -125,26 +125,25 @@ __device__ __forceinline__ void gemm_block_pipe(const GemmStage &st, u32 wofs, c
 
     ckq_v8bf bm;
     ckq_v4i ab[2];
-    float4 dx[4];
+    float dxl = 0.0f;     /* block scale of the token of output (lane & 15) of this lane's 16-lane row */
     ckq_v16f i2;
     auto combine = [&](int ts, int r) {
-        const float4 d4 = dx[r >> 2];
-        const float dxr = (r & 3) == 0 ? d4.x : (r & 3) == 1 ? d4.y : (r & 3) == 2 ? d4.z : d4.w;
         const int i1 = (aH[ts][r] << 3) + aL[ts][r];
         const float f = (float)i1;
         const float u = dw * f - dmin * i2[r];
-        acc[ts][r] += u * dxr;
+        acc[ts][r] = fmac_row_lane(acc[ts][r], dxl, u, r);
         if constexpr (DUMP) {
             const int tok = 32 * ts + 8 * (r >> 2) + (r & 3);
             dl.put(tok, 0, i1);
             dl.put(tok, 1, (int)i2[r]);
         }
     };
+    /* lane i of every 16-lane row fetches the scale of the token of its output r = i (through the
+     * integer type: an LDS read of a float after a global->LDS load makes the compiler wait for that
+     * load); the multiply-add of output r then takes lane r of the row as its factor */
+    const int dx_tok = mfma32_row_of_lane(col + 32 * half);
     auto load_dx = [&](int ts) {
-#pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4)   /* through the integer vector type: an LDS read of a float after a
-                                          * global->LDS load makes the compiler wait for that load */
-            dx[r4] = __builtin_bit_cast(float4, lds16(reinterpret_cast<const uint8_t *>(&st.d[32 * ts + 8 * r4 + 4 * half])));
+        dxl = __builtin_bit_cast(float, *reinterpret_cast<const int *>(&st.d[32 * ts + dx_tok]));
     };
     auto min_mfma = [&](int ts) {
         ckq_v16f zero;

@@ -67,13 +67,12 @@ __device__ __forceinline__ void gemm5_block(const Gemm5Stage &st, u32 wrow, cons
 
     /* token scales and stored bsums, read (through the integer vector type)
      * before the first copy is issued */
-    float4 dx[2][4];
+    float dx[2];      /* per token group: the block scale of the token of output (lane & 15) */
     ckq_v4i bs[2][2];
+    const int dx_tok = mfma32_row_of_lane(col + 32 * half);
 #pragma unroll
     for (int ts = 0; ts < 2; ++ts) {
-#pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4)
-            dx[ts][r4] = __builtin_bit_cast(float4, lds16(&st.d[32 * ts + 8 * r4 + 4 * half]));
+        dx[ts] = __builtin_bit_cast(float, *reinterpret_cast<const int *>(&st.d[32 * ts + dx_tok]));
         bs[ts][0] = lds16(&st.b[(col + 32 * ts) * 32]);
         bs[ts][1] = lds16(&st.b[(col + 32 * ts) * 32 + 16]);
     }
@@ -162,12 +161,10 @@ __device__ __forceinline__ void gemm5_block(const Gemm5Stage &st, u32 wrow, cons
     for (int ts = 0; ts < 2; ++ts)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const float4 d4 = dx[ts][r >> 2];
-            const float dxr = (r & 3) == 0 ? d4.x : (r & 3) == 1 ? d4.y : (r & 3) == 2 ? d4.z : d4.w;
             const int i1 = (iH[ts][r] << 8) + iL[ts][r], i2 = (mH[ts][r] << 8) + mL[ts][r];
             const float f1 = (float)i1;
             const float f2 = (float)i2;
-            acc[ts][r] += (dw * dxr) * f1 - (dmin * dxr) * f2;
+            acc[ts][r] = fmac_row_lane(acc[ts][r], dx[ts], dw * f1 - dmin * f2, r);
             if constexpr (DUMP) {
                 const int tok = 32 * ts + 8 * (r >> 2) + (r & 3);
                 dl.put(tok, 0, i1);

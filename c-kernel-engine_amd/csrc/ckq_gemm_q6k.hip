@@ -73,7 +73,7 @@ __device__ __forceinline__ void gemm6_head_read(const Gemm6Stage<TH> &st, u32 wr
 /* Integer sums of one block and the scales they are combined under. */
 template <int TH> struct Gemm6Sums {
     ckq_v16i iL[TH], iH[TH];
-    float4   dx[TH][4];
+    float    dx[TH];     /* per token group: the block scale of the token of output (lane & 15) */
     float    dw;
 };
 
@@ -84,10 +84,8 @@ __device__ __forceinline__ void gemm6_combine(const Gemm6Sums<TH> &p, ckq_v16f (
     for (int ts = 0; ts < TH; ++ts)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const float4 d4 = p.dx[ts][r >> 2];
-            const float dxr = (r & 3) == 0 ? d4.x : (r & 3) == 1 ? d4.y : (r & 3) == 2 ? d4.z : d4.w;
             const int i = (p.iH[ts][r] << 8) + p.iL[ts][r];
-            acc[ts][r] += (p.dw * dxr) * (float)i;
+            acc[ts][r] = fmac_row_lane(acc[ts][r], p.dx[ts], p.dw * (float)i, r);
             if constexpr (DUMP) dl.put(32 * ts + 8 * (r >> 2) + (r & 3), 0, i);
         }
 }
@@ -115,11 +113,10 @@ __device__ __forceinline__ void gemm6_slabs(const Gemm6Stage<TH> &st, const Gemm
     /* token scales: read before the first copy is issued (an LDS read of a
      * float after a global->LDS load would wait for the load), and through the
      * integer vector type like every other read of a stage */
+    const int dx_tok = mfma32_row_of_lane((int)(threadIdx.x & 63));
 #pragma unroll
     for (int ts = 0; ts < TH; ++ts)
-#pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4)
-            out.dx[ts][r4] = __builtin_bit_cast(float4, lds16(reinterpret_cast<const uint8_t *>(&st.d[32 * ts + 8 * r4 + 4 * half])));
+        out.dx[ts] = __builtin_bit_cast(float, *reinterpret_cast<const int *>(&st.d[32 * ts + dx_tok]));
     out.dw = h2f(h.dw16);
 
     u32 scp[2], cp[2];

@@ -12,12 +12,13 @@
  *   are int8 already, so nothing is unpacked.  Every instruction starts from a
  *   zero accumulator and its 16 outputs per lane are scaled and added into the
  *   fp32 accumulators: three VALU operations per output per block (convert,
- *   scale product, fused multiply-add), which is what bounds the kernel; the
+ *   product with the token's scale, fused multiply-add with the row's), which is what bounds the kernel; the
  *   matrix pipe is mostly idle and two blocks share a CU to keep the VALU fed.
  * - The weights are the A operand and the tokens the B operand, so a lane holds
  *   ONE token and 16 weight rows of the 32x32 result: the token's scale is one
- *   4-byte LDS read per instruction, and the 16 row scales (four 16-byte reads
- *   per block) are shared by both token groups.
+ *   4-byte LDS read per instruction; of the 16 row scales a lane fetches only the
+ *   one of output (lane & 15) - one 4-byte read per block - and the multiply-add
+ *   of output r takes lane r of the 16-lane row as its factor (fmac_row_lane).
  * - Operands reach LDS by global->LDS loads: the 32 quants of a block as two
  *   16-byte chunks (block starts are only 2-byte aligned in memory; the loads
  *   accept that), the fp16 scales as 2-byte loads, which land zero-extended in
@@ -42,16 +43,6 @@ struct Gemm8Stage {
     u32      xd[GEMM8_KB * GEMM8_BM];        /* fp16 scales zero-extended, [block][token] */
 };
 
-/* (float)fp16(low half of h) * x, rounded once: v_fma_mix_f32 converts the
- * half operand on the fly (the product of the two block scales, as the
- * reference forms it in fp32). */
-__device__ __forceinline__ float scale_product(int h, float x)
-{
-    float r;
-    asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel_hi:[1,0,0]" : "=v"(r) : "v"(h), "v"(x));
-    return r;
-}
-
 template <bool DUMP>
 __global__ void __launch_bounds__(256, 2) gemm_q80_mfma_kernel(GemmArgs a)
 {
@@ -60,6 +51,7 @@ __global__ void __launch_bounds__(256, 2) gemm_q80_mfma_kernel(GemmArgs a)
 
     const int tid = threadIdx.x, lane = tid & 63, wave = wave_in_block();
     const int col = lane & 31, half = lane >> 5;
+    const int dw_row = mfma32_row_of_lane(lane);      /* row (of the wave's 32) of this lane's output lane & 15 */
 
     /* token tiles fastest inside an XCD, so each XCD's L2 sees a weight tile once */
     const GemmWork work = gemm_work(a, (a.nb + KB - 1) / KB);
@@ -173,12 +165,11 @@ __global__ void __launch_bounds__(256, 2) gemm_q80_mfma_kernel(GemmArgs a)
         /* Operands of block j (read one block ahead of their use, through the
          * integer vector types only): the row's quants, the four 16-byte groups
          * of row scales, and per token group the token's quants and scale. */
-        ckq_v4i wq[2], xq[2][2], dwh[2][4];
-        u32 dxh[2][2];
+        ckq_v4i wq[2], xq[2][2];
+        u32 dwh[2], dxh[2][2];     /* dwh: the scale of the row of output (lane & 15), one per lane */
         auto read_block = [&](int j) {
             wq[j & 1] = lds16(st.wq + bofs[j]);
-#pragma unroll
-            for (int q = 0; q < 4; ++q) dwh[j & 1][q] = lds16(&st.wd[j * BN + 32 * wave + 8 * q + 4 * half]);
+            dwh[j & 1] = st.wd[j * BN + 32 * wave + dw_row];
 #pragma unroll
             for (int ts = 0; ts < 2; ++ts) {
                 xq[j & 1][ts] = lds16(st.xq + aofs[j] + 32 * 128 * ts);
@@ -206,8 +197,9 @@ __global__ void __launch_bounds__(256, 2) gemm_q80_mfma_kernel(GemmArgs a)
             if (2 * k + 1 < NCOPY) copy_one(2 * k + 1);
             if (j < valid) {
                 const float dx = h2f(dxh[j & 1][ts]);
+                const float dwf = dpp_source(h2f(dwh[j & 1]));
 #pragma unroll
-                for (int r = 0; r < 16; ++r) acc[ts][r] += scale_product(dwh[j & 1][r >> 2][r & 3], dx) * (float)d[k & 1][r];
+                for (int r = 0; r < 16; ++r) acc[ts][r] = fmac_row_lane(acc[ts][r], dwf, dx * (float)d[k & 1][r], r);
                 if constexpr (DUMP) {
                     const int t = t0 + col + 32 * ts;
 #pragma unroll
