@@ -357,6 +357,7 @@ PROFILE_WORKLOADS = {
     "gemv_q6_k_32000x4096": ("q6_k", 32000, 4096, 1),
     "gemv_q6_k_4096x11008": ("q6_k", 4096, 11008, 1),
     "gemm_q6_k_M512_4096x11008": ("q6_k", 4096, 11008, 512),
+    "gemm_q4_k_M2048_11008x4096": ("q4_k", 11008, 4096, 2048),
     "gemv_q4_k_4096x4096": ("q4_k", 4096, 4096, 1),
     "layer_7b_decode_chain_M1": None,        # eight launches per layer: four producers, four (grouped) matmuls
 }
@@ -427,7 +428,71 @@ def copy_calibration(H):
     torch.cuda.synchronize()
 
 
-def run_only(H, name, steps, warmup, calibrate):
+def clock_trace(H, name, launches, seconds=1.6):
+    """Per-repetition launch times of one workload from an idle GPU through
+    `seconds` of launches without a gap, with the shader clock rocm-smi reports
+    sampled three times during the second half: how long the clock takes to
+    settle under the kernel and where it settles."""
+    import threading
+    fmt, rows, K, M = PROFILE_WORKLOADS[name]
+    P, T, torch = H.P, H.T, H.torch
+    _, copies = H.weight_copies(fmt, rows, K, seed=rows + K, min_total=(3 * MALL_BYTES // 2) if M == 1 else 1)
+    if M > 1:
+        copies = copies[:2]
+    x = P.dev_quantize(P.to_device(T.normal(M * K, 0.0, 1.0, seed=K + M)), T.act_fmt(fmt), rows=M)
+    out = torch.empty(M * rows, dtype=torch.float32, device="cuda")
+    ops = [(fmt, x, c, None, out, M, rows, K) for c in copies]
+    n = len(copies)
+    launches = max(n, launches // n * n)
+    P.dev_matmul_sequence(ops, repeat=1)
+    torch.cuda.synchronize()
+    time.sleep(0.5)
+
+    sclk = []
+
+    def sample():
+        time.sleep(seconds * 0.5)
+        for _ in range(3):
+            try:
+                o = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=20).stdout
+                sclk.extend(line.split("(")[-1].split(")")[0] for line in o.splitlines() if "sclk" in line)
+            except (OSError, subprocess.SubprocessError) as e:
+                sclk.append("rocm-smi failed: %s" % e)
+            time.sleep(0.1)
+
+    th = threading.Thread(target=sample)
+    th.start()
+    t0 = time.perf_counter()
+    ev = [torch.cuda.Event(enable_timing=True)]
+    ev[0].record()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(8):
+            P.dev_matmul_sequence(ops, repeat=launches // n)
+            e = torch.cuda.Event(enable_timing=True)
+            e.record()
+            ev.append(e)
+        if len(ev) > 17:
+            ev[-17].synchronize()        # keep two batches queued: the GPU never waits for Python
+    th.join()
+    torch.cuda.synchronize()
+    us = [ev[i].elapsed_time(ev[i + 1]) * 1e3 / launches for i in range(len(ev) - 1)]
+    ms_at = [ev[0].elapsed_time(ev[i + 1]) for i in range(len(us))]
+    marks = [0, 1, 2, 3, 5, 8, 12, 17, 25, 35, 50, 70, 100, 140, 200, 300, 500, 800]
+    pts = []
+    for m in marks:                      # the repetition under way m milliseconds after the first launch
+        i = next((k for k, t in enumerate(ms_at) if t >= m), None)
+        if i is not None:
+            pts.append([m, round(us[i], 2)])
+    tail = us[-(len(us) // 3):]
+    print(json.dumps({"only": name, "clock_trace": True, "launches_per_repetition": launches, "repetitions": len(us),
+                      "us_per_launch_at_ms_after_idle": pts,
+                      "settled_median_us": round(statistics.median(tail), 3), "sclk_during_second_half": sclk}))
+
+
+def run_only(H, name, steps, warmup, calibrate, trace=False):
+    if trace and PROFILE_WORKLOADS.get(name):
+        clock_trace(H, name, max(1, steps))
+        return
     if name == "layer_7b_decode_chain_M1":
         _, chains, keep, _ = build_7b_layer_steps(H)
         sc = H.time_sequence(chains, max(4, steps), 3)
@@ -460,6 +525,9 @@ def main():
     ap.add_argument("--only", choices=sorted(PROFILE_WORKLOADS),
                     help="launch just this workload --steps times and exit (for rocprofv3 runs): no parity guard, "
                          "no CPU leg, a short JSON line")
+    ap.add_argument("--clock-trace", action="store_true",
+                    help="with --only: launch times from an idle GPU through 1.6 s of continuous launches, and the shader "
+                         "clock rocm-smi reports meanwhile")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch the plain copy kernel on a 256 MiB buffer (known traffic), for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings")
@@ -470,7 +538,7 @@ def main():
 
     H = Harness()
     if a.only:
-        run_only(H, a.only, a.steps, a.warmup, a.calibrate_copy)
+        run_only(H, a.only, a.steps, a.warmup, a.calibrate_copy, a.clock_trace)
         return
     torch, P, T = H.torch, H.P, H.T
     rows, K, M = 11008, 4096, 1
