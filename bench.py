@@ -148,6 +148,29 @@ class Harness:
         t = [ev[i].elapsed_time(ev[i + 1]) * 1e-3 / launches for i in range(reps)]
         return summarize(t[-(reps // 3):]), summarize(burst)
 
+    def time_sequence_settled(self, ops, settle_s=0.1):
+        """Median seconds per pass over `ops` (one ckq_matmul_sequence_dev call) in the last third of at
+        least `settle_s` seconds of calls without a gap (see time_gemm_settled)."""
+        torch, P = self.torch, self.P
+        P.dev_matmul_sequence(ops)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        P.dev_matmul_sequence(ops, repeat=2)
+        e1.record()
+        torch.cuda.synchronize()
+        est = max(e0.elapsed_time(e1) * 0.5e-3, 1e-6)
+        per = 4
+        reps = max(15, int(settle_s * 1.5 / (est * per)))
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
+        ev[0].record()
+        for i in range(reps):
+            P.dev_matmul_sequence(ops, repeat=per)
+            ev[i + 1].record()
+        torch.cuda.synchronize()
+        t = [ev[i].elapsed_time(ev[i + 1]) * 1e-3 / per for i in range(reps)]
+        return statistics.median(t[-(reps // 3):])
+
     def time_gemv(self, fmt, rows, K, M, copies, xq_d, launches=LAUNCHES_PER_REP, reps=REPS, warmup=0):
         """Seconds per launch (median, min, max over the repetitions) of
         back-to-back launches rotating through the weight copies; one C call
@@ -712,6 +735,40 @@ def main():
                                               "gbs_of_weight_bytes": round(lbytes / sc / 1e9, 1),
                                               "note": "norm->Q8_K, Q+K+V, Q8_K, O, norm->Q8_K, gate+up, SwiGLU->Q8_K, down in one C call"}
         del layers, keep, chains
+        torch.cuda.empty_cache()
+
+        # the same layer's projection set at prefill size (512 tokens, grouped-query attention: K and V
+        # 1024 rows): Q,K,V | O | gate,up | down.  The sequence call issues Q+K+V and gate+up as one
+        # matrix-core launch each; the same entries one launch each are timed beside it.
+        Mp = 512
+        xp = P.dev_quantize(P.to_device(T.normal(Mp * 4096, seed=34)), "q8_k", rows=Mp)
+        hp = P.dev_quantize(P.to_device(T.normal(Mp * 11008, seed=35)), "q8_k", rows=Mp)
+        pops, pkeep, pflop = [], [], 0.0
+        for j, (fmt, r, k) in enumerate([("q4_k", 4096, 4096), ("q4_k", 1024, 4096), ("q4_k", 1024, 4096), ("q4_k", 4096, 4096),
+                                         ("q4_k", 11008, 4096), ("q4_k", 11008, 4096), ("q6_k", 4096, 11008)]):
+            Wj = torch.from_numpy(T.synth_weights(fmt, r, k, seed=1100 + j)).cuda()
+            o = torch.zeros(Mp * r, dtype=torch.float32, device="cuda")
+            pkeep += [Wj, o]
+            pops.append((fmt, hp if k == 11008 else xp, Wj, None, o, Mp, r, k))
+            pflop += 2.0 * Mp * r * k
+        # O must not join the Q/K/V group, nor gate/up the one before: give them their own activations
+        xp2 = xp.clone()
+        pops[3] = pops[3][:1] + (xp2,) + pops[3][2:]
+        xp3 = xp.clone()
+        pops[4] = pops[4][:1] + (xp3,) + pops[4][2:]
+        pops[5] = pops[5][:1] + (xp3,) + pops[5][2:]
+        pre = {}
+        for label, on in (("grouped", 1), ("one_launch_per_matrix", 0)):
+            H.L.ckq_set_prefill_grouping(on)
+            sp_ = H.time_sequence_settled(pops)
+            pre[label + "_us"] = round(sp_ * 1e6, 2)
+        H.L.ckq_set_prefill_grouping(1)
+        pre.update({"tops": round(pflop / (pre["grouped_us"] * 1e-6) / 1e12, 1), "ops": pflop,
+                    "launches_grouped": 4, "launches_ungrouped": "7 (K and V each with a K split and its reduction)",
+                    "note": "Q 4096, K and V 1024, O 4096 (Q4_K, K = 4096), gate and up 11008 (Q4_K), down 4096x11008 (Q6_K); "
+                            "clock settled"})
+        extras["layer_7b_prefill_set_M512"] = pre
+        del pops, pkeep, xp, xp2, xp3, hp
         torch.cuda.empty_cache()
 
         # small-model batched decode (Qwen2-0.5B-like: hidden 896 padded to K=1024, Q5_K

@@ -144,6 +144,7 @@ _SIGS = {
     "ckq_weights_set_limit": (None, [_c.c_size_t]),
     "ckq_release_stream": (_i, [_vp]),
     "ckq_set_parallel_whole": (None, [_i]),
+    "ckq_set_prefill_grouping": (None, [_i]),
     "ckq_set_gemm_policy": (None, [_i]),
     "ckq_last_error": (_i, []),
     "ckq_clear_error": (None, []),

@@ -16,6 +16,17 @@ typedef unsigned short ckq_v2u16 __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) void ckq_lds_void;
 typedef const __attribute__((address_space(1))) void ckq_glb_void;
 
+/* One weight matrix of a grouped launch: several matrices that multiply the same activations (Q/K/V,
+ * gate/up) share a grid; a matrix owns the block ids [id0, id0 + ntt * round_up(nnt, 8)). */
+constexpr int GEMM_GROUP_MAX = 4;
+struct GemmProblem {
+    const uint8_t *B;
+    const float   *bias;
+    float         *C;
+    long           ldc;
+    int            N, nnt, id0;
+};
+
 struct GemmArgs {
     const uint8_t *A;     /* Q8_K activations, M rows of nb blocks */
     const uint8_t *B;     /* Q4_K weights, N rows of nb blocks */
@@ -24,6 +35,9 @@ struct GemmArgs {
     int  M, N, nb;
     long ldc;
     int  ntt, nnt;        /* token tiles, weight-row tiles */
+    /* grouped launch: ngroup > 1 matrices, never split along K; B, bias, C, N, ldc, nnt above are those of grp[0] */
+    int  ngroup;
+    GemmProblem grp[GEMM_GROUP_MAX];
     /* split K: blockIdx.y = s handles K-steps [s * k_per, min(k_steps, (s + 1) * k_per)) and
      * writes its partial tile, without bias, to part + s * M * N (row pitch N) */
     int    splits, k_per;
@@ -72,14 +86,22 @@ struct GemmOpts {
 /* What one block of a GEMM launch does: which tile id, which K-steps, where it
  * writes and whether it adds the bias. */
 struct GemmOut { float *C; long ldc; const float *bias; };
-struct GemmWork { int id, k0, k1; GemmOut out; };
+struct GemmWork { int id, k0, k1; GemmOut out; const uint8_t *B; int N, nnt; };
 __device__ __forceinline__ GemmWork gemm_work(const GemmArgs &a, int k_steps)
 {
     const int id = blockIdx.x;
-    if (a.splits <= 1) return {id, 0, k_steps, {a.C, a.ldc, a.bias}};
+    if (a.ngroup > 1) {
+        /* uniform selects, no indexing: the argument block stays in scalar registers */
+        GemmProblem g = a.grp[0];
+        if (id >= a.grp[1].id0) g = a.grp[1];
+        if (a.ngroup > 2 && id >= a.grp[2].id0) g = a.grp[2];
+        if (a.ngroup > 3 && id >= a.grp[3].id0) g = a.grp[3];
+        return {id - g.id0, 0, k_steps, {g.C, g.ldc, g.bias}, g.B, g.N, g.nnt};
+    }
+    if (a.splits <= 1) return {id, 0, k_steps, {a.C, a.ldc, a.bias}, a.B, a.N, a.nnt};
     const int k0 = (int)blockIdx.y * a.k_per;
     return {id, k0, min(k_steps, k0 + a.k_per),
-            {a.part + (size_t)blockIdx.y * (size_t)a.M * (size_t)a.N, (long)a.N, nullptr}};
+            {a.part + (size_t)blockIdx.y * (size_t)a.M * (size_t)a.N, (long)a.N, nullptr}, a.B, a.N, a.nnt};
 }
 
 /* Split K when the tile grid leaves most of the chip idle: `tiles` blocks of
@@ -183,8 +205,48 @@ __device__ __forceinline__ int mfma32_row_of_lane(int lane)
     return 8 * ((lane & 15) >> 2) + 4 * (lane >> 5) + (lane & 3);
 }
 
+/* Grouped launch: the matrices of `in` against the same M x K activations, as one grid (no K split; the
+ * callers group only what fills the chip without one).  rows_per_tile = weight rows of a block's tile. */
+struct GemmGroupIn {
+    int          n;
+    const void  *B[GEMM_GROUP_MAX];
+    const float *bias[GEMM_GROUP_MAX];
+    float       *C[GEMM_GROUP_MAX];
+    int          N[GEMM_GROUP_MAX];
+    long         ldc[GEMM_GROUP_MAX];
+};
+/* Below this many tiles a single matrix is split along K instead (gemm_choose_splits); a group is not. */
+constexpr int GEMM_GROUP_MIN_TILES = 160;
+static int gemm_group_tiles(const GemmGroupIn &in, int M, int tokens_per_tile, int rows_per_tile = GEMM_TILE_ROWS)
+{
+    int tiles = 0;
+    for (int p = 0; p < in.n; ++p)
+        tiles += ((M + tokens_per_tile - 1) / tokens_per_tile) * ((in.N[p] + rows_per_tile - 1) / rows_per_tile);
+    return tiles;
+}
+template <class Kernel>
+static int gemm_launch_grouped(Kernel kernel, GemmArgs &g, const GemmGroupIn &in, hipStream_t s, unsigned threads = 256)
+{
+    unsigned grid = 0;
+    g.ngroup = in.n;
+    for (int p = 0; p < in.n; ++p) {
+        const int nnt = (in.N[p] + GEMM_TILE_ROWS - 1) / GEMM_TILE_ROWS;
+        g.grp[p] = {(const uint8_t *)in.B[p], in.bias[p], in.C[p], in.ldc[p], in.N[p], nnt, (int)grid};
+        grid += (unsigned)g.ntt * (unsigned)((nnt + 7) / 8 * 8);
+    }
+    g.B = g.grp[0].B; g.bias = g.grp[0].bias; g.C = g.grp[0].C; g.N = g.grp[0].N; g.ldc = g.grp[0].ldc; g.nnt = g.grp[0].nnt;
+    g.splits = 1; g.k_per = 0; g.part = nullptr;
+    hipLaunchKernelGGL(kernel, dim3(grid, 1u), dim3(threads), 0, s, g);
+    return (int)hipGetLastError();
+}
+
 /* The four kernels, one translation unit each: C[m*ldc + n] = dot(B row n, A row m) (+ bias[n]).
- * See GemmOpts for the options. */
+ * See GemmOpts for the options.  The _group forms return CKQ_ENOGROUP when the matrices are better
+ * launched one by one (too few tiles to fill the chip without a K split). */
+int launch_gemm_q4k_mfma_group(const void *A, const GemmGroupIn &in, int M, int K, hipStream_t s);
+int launch_gemm_q5k_mfma_group(const void *A, const GemmGroupIn &in, int M, int K, hipStream_t s);
+int launch_gemm_q6k_mfma_group(const void *A, const GemmGroupIn &in, int M, int K, hipStream_t s);
+int launch_gemm_q80_mfma_group(const void *A, const GemmGroupIn &in, int M, int K, hipStream_t s);
 int launch_gemm_q4k_mfma(const void *A, const void *B, const float *bias, float *C, int M, int N, int K, long ldc, const GemmOpts &opts, hipStream_t s);
 int launch_gemm_q5k_mfma(const void *A, const void *B, const float *bias, float *C, int M, int N, int K, long ldc, const GemmOpts &opts, hipStream_t s);
 int launch_gemm_q6k_mfma(const void *A, const void *B, const float *bias, float *C, int M, int N, int K, long ldc, const GemmOpts &opts, hipStream_t s);

@@ -217,11 +217,11 @@ __global__ void __launch_bounds__(256 * KG, KG == 2 ? 1 : WPE) gemm_q4k_mfma_ker
     const int id = work.id, xcd = id & 7, seq = id >> 3;
     const int tt = seq % a.ntt;
     const int nt = (seq / a.ntt) * 8 + xcd;
-    if (nt >= a.nnt) return;
+    if (nt >= work.nnt) return;
     const int t0 = tt * BM, n0 = nt * GEMM_BN;
     const u32 wstride = (u32)a.nb * 144u, xstride = (u32)a.nb * 292u;
     const int b0 = work.k0, b1 = work.k1, last = b1 - 1;
-    const uint8_t *wbase = a.B + (size_t)n0 * wstride;       /* uniform */
+    const uint8_t *wbase = work.B + (size_t)n0 * wstride;       /* uniform */
     const uint8_t *xbase = a.A + (size_t)t0 * xstride;       /* uniform */
 
     /* Copy roles.  One wave instruction moves 64 x 16 bytes into 1 KiB of
@@ -234,7 +234,7 @@ __global__ void __launch_bounds__(256 * KG, KG == 2 ? 1 : WPE) gemm_q4k_mfma_ker
     u32 wofs_g[NWI], qofs_g[NQI];
 #pragma unroll
     for (int i = 0; i < NWI; ++i) {
-        const int chunk = min(wave + 4 * i, 17) * 64 + lane, row = min(chunk / 9, a.N - 1 - n0), part = chunk % 9;
+        const int chunk = min(wave + 4 * i, 17) * 64 + lane, row = min(chunk / 9, work.N - 1 - n0), part = chunk % 9;
         wofs_g[i] = (u32)row * wstride + 16u * part;
     }
 #pragma unroll
@@ -316,10 +316,10 @@ __global__ void __launch_bounds__(256 * KG, KG == 2 ? 1 : WPE) gemm_q4k_mfma_ker
         GemmDumpLane dl = {};
         if constexpr (DUMP) {
             const int n = n0 + wave * 32 + col, tf = t0 + 4 * half;
-            dl.tok_stride = gemm_opaque((size_t)a.N * a.nb * 2);
-            dl.p = a.dump + ((size_t)tf * a.N + n) * a.nb * 2 + (size_t)b * 2;
+            dl.tok_stride = gemm_opaque((size_t)work.N * a.nb * 2);
+            dl.p = a.dump + ((size_t)tf * work.N + n) * a.nb * 2 + (size_t)b * 2;
             dl.tok_left = a.M - tf;
-            dl.row_ok = n < a.N && b < b1;
+            dl.row_ok = n < work.N && b < b1;
         }
         if (KG == 1 || b < b1) gemm_block_pipe<DUMP>(stage[cur], wofs_l, aofs, col, half, acc, copy_one, dl);
         __builtin_amdgcn_sched_barrier(0);
@@ -352,7 +352,7 @@ __global__ void __launch_bounds__(256 * KG, KG == 2 ? 1 : WPE) gemm_q4k_mfma_ker
 
     const GemmOut o = work.out;
     const int n = n0 + wave * 32 + col;
-    if (n < a.N) {
+    if (n < work.N) {
         const float bias = o.bias ? o.bias[n] : 0.0f;
 #pragma unroll
         for (int ts = 0; ts < 2; ++ts)
@@ -396,4 +396,17 @@ int launch_gemm_q4k_mfma(const void *A, const void *B, const float *bias, float 
     }
     if (two_groups) return gemm_launch_split(gemm_q4k_mfma_kernel<CKQ_GEMM_WPE, 2>, g, (unsigned)(g.ntt * nnt8), g.nb, s, 512);
     return gemm_launch_split(gemm_q4k_mfma_kernel<CKQ_GEMM_WPE, 1>, g, (unsigned)(g.ntt * nnt8), g.nb, s, 256);
+}
+
+int launch_gemm_q4k_mfma_group(const void *A, const GemmGroupIn &in, int M, int K, hipStream_t s)
+{
+    const int tiles = gemm_group_tiles(in, M, GEMM_BM);
+    if (tiles < GEMM_GROUP_MIN_TILES) return CKQ_ENOGROUP;
+    GemmArgs g = {};
+    g.A = (const uint8_t *)A; g.M = M; g.nb = K / 256;
+    if ((long long)g.nb * 292 * GEMM_BN >= (1ll << 31)) return (int)hipErrorInvalidValue;
+    g.ntt = (M + GEMM_BM - 1) / GEMM_BM;
+    /* as for one matrix: two groups of waves per tile while every tile gets a CU of its own */
+    if (tiles <= 256 && g.nb >= 8) return gemm_launch_grouped(gemm_q4k_mfma_kernel<CKQ_GEMM_WPE, 2>, g, in, s, 512);
+    return gemm_launch_grouped(gemm_q4k_mfma_kernel<CKQ_GEMM_WPE, 1>, g, in, s, 256);
 }

@@ -188,11 +188,11 @@ __global__ void __launch_bounds__(256, 1) gemm_q5k_mfma_kernel(GemmArgs a)
     const int id = work.id, xcd = id & 7, seq = id >> 3;
     const int tt = seq % a.ntt;
     const int nt = (seq / a.ntt) * 8 + xcd;
-    if (nt >= a.nnt) return;
+    if (nt >= work.nnt) return;
     const int t0 = tt * BM, n0 = nt * GEMM5_BN;
     const u32 wstride = (u32)a.nb * 176u, xstride = (u32)a.nb * 292u;
     const int b0 = work.k0, b1 = work.k1, last = b1 - 1;
-    const uint8_t *wbase = a.B + (size_t)n0 * wstride;       /* uniform */
+    const uint8_t *wbase = work.B + (size_t)n0 * wstride;       /* uniform */
     const uint8_t *xbase = a.A + (size_t)t0 * xstride;       /* uniform */
 
     /* Copy roles.  Weights: 128 rows x 11 chunks = 22 wave instructions, six
@@ -205,7 +205,7 @@ __global__ void __launch_bounds__(256, 1) gemm_q5k_mfma_kernel(GemmArgs a)
     u32 wofs_g[NWI], qofs_g[NQI], dofs_g, bofs_g;
 #pragma unroll
     for (int i = 0; i < NWI; ++i) {
-        const int chunk = min(wave + 4 * i, 21) * 64 + lane, row = min(chunk / 11, a.N - 1 - n0), part = chunk % 11;
+        const int chunk = min(wave + 4 * i, 21) * 64 + lane, row = min(chunk / 11, work.N - 1 - n0), part = chunk % 11;
         wofs_g[i] = (u32)row * wstride + 16u * part;
     }
 #pragma unroll
@@ -276,10 +276,10 @@ __global__ void __launch_bounds__(256, 1) gemm_q5k_mfma_kernel(GemmArgs a)
         GemmDumpLane dl = {};
         if constexpr (DUMP) {
             const int n = n0 + wave * 32 + col, tf = t0 + 4 * half;
-            dl.tok_stride = gemm_opaque((size_t)a.N * a.nb * 2);
-            dl.p = a.dump + ((size_t)tf * a.N + n) * a.nb * 2 + (size_t)b * 2;
+            dl.tok_stride = gemm_opaque((size_t)work.N * a.nb * 2);
+            dl.p = a.dump + ((size_t)tf * work.N + n) * a.nb * 2 + (size_t)b * 2;
             dl.tok_left = a.M - tf;
-            dl.row_ok = n < a.N;
+            dl.row_ok = n < work.N;
         }
         gemm5_block<NCOPY, DUMP>(stage[cur], wrow, aofs, col, half, acc, copy_one, dl);
         __builtin_amdgcn_sched_barrier(0);
@@ -295,7 +295,7 @@ __global__ void __launch_bounds__(256, 1) gemm_q5k_mfma_kernel(GemmArgs a)
 
     const GemmOut o = work.out;
     const int n = n0 + wave * 32 + col;
-    if (n < a.N) {
+    if (n < work.N) {
         const float bias = o.bias ? o.bias[n] : 0.0f;
 #pragma unroll
         for (int ts = 0; ts < 2; ++ts)
@@ -328,4 +328,14 @@ int launch_gemm_q5k_mfma(const void *A, const void *B, const float *bias, float 
     if (sums) return CKQ_ENODUMP;
 #endif
     return gemm_launch_split(gemm_q5k_mfma_kernel<false>, g, (unsigned)(g.ntt * nnt8), g.nb, s);
+}
+
+int launch_gemm_q5k_mfma_group(const void *A, const GemmGroupIn &in, int M, int K, hipStream_t s)
+{
+    if (gemm_group_tiles(in, M, GEMM5_BM) < GEMM_GROUP_MIN_TILES) return CKQ_ENOGROUP;
+    GemmArgs g = {};
+    g.A = (const uint8_t *)A; g.M = M; g.nb = K / 256;
+    if ((long long)g.nb * 292 * 128 >= (1ll << 31)) return (int)hipErrorInvalidValue;
+    g.ntt = (M + GEMM5_BM - 1) / GEMM5_BM;
+    return gemm_launch_grouped(gemm_q5k_mfma_kernel<false>, g, in, s);
 }

@@ -186,11 +186,11 @@ __global__ void __launch_bounds__(256, 1) gemm_q6k_mfma_kernel(GemmArgs a)
     const int id = work.id, xcd = id & 7, seq = id >> 3;
     const int tt = seq % a.ntt;
     const int nt = (seq / a.ntt) * 8 + xcd;
-    if (nt >= a.nnt) return;
+    if (nt >= work.nnt) return;
     const int t0 = tt * BM, n0 = nt * GEMM6_BN;
     const u32 wstride = (u32)a.nb * 210u, xstride = (u32)a.nb * 292u;
     const int b0 = work.k0, b1 = work.k1, last = b1 - 1;
-    const uint8_t *wbase = a.B + (size_t)n0 * wstride;       /* uniform */
+    const uint8_t *wbase = work.B + (size_t)n0 * wstride;       /* uniform */
     const uint8_t *xbase = a.A + (size_t)t0 * xstride;       /* uniform */
 
     /* Copy roles.  One wave instruction moves 64 x 16 bytes into 1 KiB of LDS
@@ -201,7 +201,7 @@ __global__ void __launch_bounds__(256, 1) gemm_q6k_mfma_kernel(GemmArgs a)
     u32 wofs_g[NWI], qofs_g[NQI], dofs_g[NDI];
 #pragma unroll
     for (int i = 0; i < NWI; ++i) {
-        const int chunk = (wave + 4 * i) * 64 + lane, row = min(chunk / 14, a.N - 1 - n0), part = chunk % 14;
+        const int chunk = (wave + 4 * i) * 64 + lane, row = min(chunk / 14, work.N - 1 - n0), part = chunk % 14;
         wofs_g[i] = (u32)row * wstride + (part < 13 ? 16u * part : 194u);
     }
 #pragma unroll
@@ -276,10 +276,10 @@ __global__ void __launch_bounds__(256, 1) gemm_q6k_mfma_kernel(GemmArgs a)
         GemmDumpLane dl = {};
         if constexpr (DUMP) {
             const int n = n0 + wave * 32 + col, tf = t0 + 4 * half;
-            dl.tok_stride = gemm_opaque((size_t)a.N * a.nb);
-            dl.p = a.dump + ((size_t)tf * a.N + n) * a.nb + (size_t)b;
+            dl.tok_stride = gemm_opaque((size_t)work.N * a.nb);
+            dl.p = a.dump + ((size_t)tf * work.N + n) * a.nb + (size_t)b;
             dl.tok_left = a.M - tf;
-            dl.row_ok = n < a.N;
+            dl.row_ok = n < work.N;
         }
         gemm6_slabs<TH, NCOPY>(stage[cur], head, aofs, half, sums, copy_one);
         __builtin_amdgcn_sched_barrier(0);
@@ -313,7 +313,7 @@ __global__ void __launch_bounds__(256, 1) gemm_q6k_mfma_kernel(GemmArgs a)
 
     const GemmOut o = work.out;
     const int n = n0 + wave * 32 + col;
-    if (n < a.N) {
+    if (n < work.N) {
         const float bias = o.bias ? o.bias[n] : 0.0f;
 #pragma unroll
         for (int ts = 0; ts < TH; ++ts)
@@ -357,4 +357,19 @@ int launch_gemm_q6k_mfma(const void *A, const void *B, const float *bias, float 
     if (sums) return CKQ_ENODUMP;
 #endif
     return gemm_launch_split(gemm_q6k_mfma_kernel<2>, g, (unsigned)(g.ntt * nnt8), g.nb, s);
+}
+
+int launch_gemm_q6k_mfma_group(const void *A, const GemmGroupIn &in, int M, int K, hipStream_t s)
+{
+    GemmArgs g = {};
+    g.A = (const uint8_t *)A; g.M = M; g.nb = K / 256;
+    if ((long long)g.nb * 292 * 128 >= (1ll << 31)) return (int)hipErrorInvalidValue;
+    /* tiles of 128 tokens where they fill the chip, else 64 */
+    if (gemm_group_tiles(in, M, 128) >= GEMM_GROUP_MIN_TILES) {
+        g.ntt = (M + 127) / 128;
+        return gemm_launch_grouped(gemm_q6k_mfma_kernel<4>, g, in, s);
+    }
+    if (gemm_group_tiles(in, M, 64) < GEMM_GROUP_MIN_TILES) return CKQ_ENOGROUP;
+    g.ntt = (M + 63) / 64;
+    return gemm_launch_grouped(gemm_q6k_mfma_kernel<2>, g, in, s);
 }

@@ -58,12 +58,12 @@ __global__ void __launch_bounds__(256, 2) gemm_q80_mfma_kernel(GemmArgs a)
     const int id = work.id, xcd = id & 7, seq = id >> 3;
     const int tt = seq % a.ntt;
     const int nt = (seq / a.ntt) * 8 + xcd;
-    if (nt >= a.nnt) return;
+    if (nt >= work.nnt) return;
     const int t0 = tt * BM, n0 = nt * BN;
     const int nblk = a.nb;                                  /* 32-blocks per row */
     const u32 stride = (u32)nblk * 34u;                     /* bytes per weight row and per activation row */
     const int it0 = work.k0, niter = work.k1;               /* this block runs iterations [it0, niter) */
-    const uint8_t *wbase = a.B + (size_t)n0 * stride;       /* uniform */
+    const uint8_t *wbase = work.B + (size_t)n0 * stride;       /* uniform */
     const uint8_t *xbase = a.A + (size_t)t0 * stride;       /* uniform */
 
     /* Copy roles per iteration: weight quants 128 rows x 8 chunks = 16 wave
@@ -80,7 +80,7 @@ __global__ void __launch_bounds__(256, 2) gemm_q80_mfma_kernel(GemmArgs a)
     for (int i = 0; i < NWQ; ++i) {
         const int chunk = (wave + 4 * i) * 64 + lane, row = chunk >> 3, c = (chunk & 7) ^ (row & 7);
         wq_blk[i] = (u32)(c >> 1);
-        wq_g[i] = (u32)min(row, a.N - 1 - n0) * stride + 2u + 16u * (u32)(c & 1);
+        wq_g[i] = (u32)min(row, work.N - 1 - n0) * stride + 2u + 16u * (u32)(c & 1);
     }
 #pragma unroll
     for (int i = 0; i < NXQ; ++i) {
@@ -92,7 +92,7 @@ __global__ void __launch_bounds__(256, 2) gemm_q80_mfma_kernel(GemmArgs a)
     for (int i = 0; i < NWD; ++i) {
         const int e = (wave + 4 * i) * 64 + lane;            /* [block][row] entry */
         wd_blk[i] = (u32)(e >> 7);
-        wd_g[i] = (u32)min(e & 127, a.N - 1 - n0) * stride;
+        wd_g[i] = (u32)min(e & 127, work.N - 1 - n0) * stride;
     }
     {
         const int e = wave * 64 + lane;                      /* [block][token] entry */
@@ -205,7 +205,7 @@ __global__ void __launch_bounds__(256, 2) gemm_q80_mfma_kernel(GemmArgs a)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
                         const int n = n0 + 32 * wave + 8 * (r >> 2) + 4 * half + (r & 3);
-                        if (t < a.M && n < a.N) a.dump[((size_t)t * a.N + n) * nblk + (size_t)(it * KB + j)] = d[k & 1][r];
+                        if (t < a.M && n < work.N) a.dump[((size_t)t * work.N + n) * nblk + (size_t)(it * KB + j)] = d[k & 1][r];
                     }
                 }
             }
@@ -222,7 +222,7 @@ __global__ void __launch_bounds__(256, 2) gemm_q80_mfma_kernel(GemmArgs a)
 
     /* lane: token t0 + col + 32 ts, rows n0 + 32 wave + 8 q + 4 half + (0..3) */
     const GemmOut o = work.out;
-    const bool vec_ok = (o.ldc % 4 == 0) && (((uintptr_t)o.C) % 16 == 0) && (n0 + BN <= a.N);
+    const bool vec_ok = (o.ldc % 4 == 0) && (((uintptr_t)o.C) % 16 == 0) && (n0 + BN <= work.N);
 #pragma unroll
     for (int ts = 0; ts < 2; ++ts) {
         const int t = t0 + col + 32 * ts;
@@ -232,12 +232,12 @@ __global__ void __launch_bounds__(256, 2) gemm_q80_mfma_kernel(GemmArgs a)
             const int n = n0 + 32 * wave + 8 * q + 4 * half;
             float v[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) v[i] = acc[ts][4 * q + i] + ((o.bias && n + i < a.N) ? o.bias[n + i] : 0.0f);
+            for (int i = 0; i < 4; ++i) v[i] = acc[ts][4 * q + i] + ((o.bias && n + i < work.N) ? o.bias[n + i] : 0.0f);
             float *dst = o.C + (size_t)t * o.ldc + n;
             if (vec_ok) *reinterpret_cast<float4 *>(dst) = make_float4(v[0], v[1], v[2], v[3]);
             else {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) if (n + i < a.N) dst[i] = v[i];
+                for (int i = 0; i < 4; ++i) if (n + i < work.N) dst[i] = v[i];
             }
         }
     }
@@ -264,4 +264,14 @@ int launch_gemm_q80_mfma(const void *A, const void *B, const float *bias, float 
     if (sums) return CKQ_ENODUMP;
 #endif
     return gemm_launch_split(gemm_q80_mfma_kernel<false>, g, (unsigned)(g.ntt * nnt8), (g.nb + GEMM8_KB - 1) / GEMM8_KB, s);
+}
+
+int launch_gemm_q80_mfma_group(const void *A, const GemmGroupIn &in, int M, int K, hipStream_t s)
+{
+    if (gemm_group_tiles(in, M, GEMM8_BM) < GEMM_GROUP_MIN_TILES) return CKQ_ENOGROUP;
+    GemmArgs g = {};
+    g.A = (const uint8_t *)A; g.M = M; g.nb = K / 32;
+    if ((long long)g.nb * 34 * GEMM8_BN >= (1ll << 31)) return (int)hipErrorInvalidValue;
+    g.ntt = (M + GEMM8_BM - 1) / GEMM8_BM;
+    return gemm_launch_grouped(gemm_q80_mfma_kernel<false>, g, in, s);
 }

@@ -633,6 +633,12 @@ void ckq_weights_set_cache(int enabled)
 
 void ckq_set_gemm_policy(int policy) { ckq_launch_set_gemm_policy(policy); }
 
+static int g_prefill_grouping = 1;
+void ckq_set_prefill_grouping(int enabled)
+{
+    __atomic_store_n(&g_prefill_grouping, enabled != 0, __ATOMIC_RELAXED);
+}
+
 void ckq_set_parallel_whole(int enabled)
 {
     pthread_mutex_lock(&g_mu);
@@ -1335,11 +1341,13 @@ static int group_length(const ckq_matmul_op *ops, int i, int nops)
     enum { GROUP_MAX = 4 };
     const ckq_matmul_op *o = &ops[i];
     int n = 1;
-    const int groupable = o->A_q8 && o->B && o->C && o->M >= 1 && o->M <= 8 && o->N > 0 && o->K > 0 &&
+    const int groupable = o->A_q8 && o->B && o->C && o->M >= 1 && o->N > 0 && o->K > 0 &&
                           o->ldc >= o->N && !is_f32act(o->fmt) && !(o->fmt & CKQ_ACT_F32) && o->K % fmt_block_elems(o->fmt) == 0;
     while (groupable && n < GROUP_MAX && i + n < nops) {
         if (ops[i + n].fmt >= CKQ_STEP_QUANTIZE_Q8_K && ops[i + n].fmt <= CKQ_STEP_SWIGLU_Q8_K) break;
         if (ops[i + n].fmt & CKQ_ACT_F32) break;
+        /* beyond eight tokens the matrices share a matrix-core launch, which takes one activation matrix */
+        if (o->M > 8 && (ops[i + n].A_q8 != o->A_q8 || !__atomic_load_n(&g_prefill_grouping, __ATOMIC_RELAXED))) break;
         int ok = 1;
         for (int j = 0; j < n && ok; ++j) ok = ops_independent(&ops[i + j], &ops[i + n]);
         if (!ok) break;
@@ -1382,7 +1390,14 @@ int ckq_matmul_sequence_dev(const ckq_matmul_op *ops, int nops, int repeat, void
                     y[j] = ops[i + j].C; W[j] = ops[i + j].B; X[j] = ops[i + j].A_q8; b[j] = ops[i + j].bias;
                     rows[j] = ops[i + j].N; ld[j] = ops[i + j].ldc;
                 }
-                rc = ckq_launch_gemv_group(o->fmt, n, y, W, X, b, rows, ld, o->K, o->M, NULL, stream);
+                rc = o->M > 8 ? ckq_launch_gemm_group(o->fmt, n, y, W, o->A_q8, b, rows, ld, o->K, o->M, stream)
+                              : ckq_launch_gemv_group(o->fmt, n, y, W, X, b, rows, ld, o->K, o->M, NULL, stream);
+                if (rc == CKQ_ENOGROUP) {            /* better one by one (too few tiles, or sizes the streaming kernel serves) */
+                    rc = 0;
+                    for (int j = 0; j < n && !rc; ++j)
+                        rc = ckq_gemm_nt_dev(ops[i + j].fmt, ops[i + j].A_q8, ops[i + j].B, ops[i + j].bias, ops[i + j].C,
+                                             ops[i + j].M, ops[i + j].N, ops[i + j].K, ops[i + j].ldc, stream);
+                }
             } else {
                 rc = ckq_gemm_nt_dev(o->fmt, o->A_q8, o->B, o->bias, o->C, o->M, o->N, o->K, o->ldc, stream);
             }

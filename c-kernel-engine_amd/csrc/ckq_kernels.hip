@@ -399,6 +399,50 @@ static int launch_gemv_args(int fmt_flags, GemvArgs &a, const GemvGroup &grp, in
     }
 }
 
+/* Several weight matrices of one format against the same quantized activations (Q/K/V, gate/up at
+ * prefill sizes) as ONE matrix-core launch: the tiles of all matrices share a grid, so the narrow ones
+ * (K and V under grouped-query attention) fill the chip together with the wide one instead of each
+ * taking a K-split launch of its own, and one launch boundary replaces n.  Every tile is computed
+ * exactly as the single-matrix launch without a K split computes it.  CKQ_ENOGROUP: not taken (the
+ * streaming kernel would serve these sizes, or the tiles of all matrices together still leave most of
+ * the chip idle); the caller then issues the matrices one by one. */
+extern "C" int ckq_launch_gemm_group(int fmt, int n, float *const *C, const void *const *B, const void *A,
+                                     const float *const *bias, const int *N, const long *ldc, int K, int M, void *stream)
+{
+    if (n < 2 || n > GEMM_GROUP_MAX || M <= CKQ_STREAM_TOKENS || !A || K <= 0) return CKQ_ENOGROUP;
+    GemmGroupIn in = {};
+    in.n = n;
+    size_t rows = 0;
+    bool aligned = true;
+    for (int p = 0; p < n; ++p) {
+        if (!C[p] || !B[p] || N[p] <= 0 || ldc[p] < N[p]) return CKQ_EINVAL;
+        in.B[p] = B[p]; in.bias[p] = bias ? bias[p] : nullptr; in.C[p] = C[p]; in.N[p] = N[p]; in.ldc[p] = ldc[p];
+        rows += (size_t)N[p];
+        aligned = aligned && ((uintptr_t)B[p] % 4 == 0);
+    }
+    hipStream_t s = (hipStream_t)stream;
+    switch (fmt) {
+    case CKQ_FMT_Q4_K:
+        if (K % 256) return CKQ_ESHAPE;
+        if (!gemm_on_matrix_cores(M, rows * (K / 256) * 144, 20)) return CKQ_ENOGROUP;
+        return launch_gemm_q4k_mfma_group(A, in, M, K, s);
+    case CKQ_FMT_Q5_K:
+        if (K % 256) return CKQ_ESHAPE;
+        if (!gemm_on_matrix_cores(M, rows * (K / 256) * 176, 40)) return CKQ_ENOGROUP;
+        return launch_gemm_q5k_mfma_group(A, in, M, K, s);
+    case CKQ_FMT_Q6_K:
+        if (K % 256) return CKQ_ESHAPE;
+        if (!gemm_on_matrix_cores(M, rows * (K / 256) * 210, 20)) return CKQ_ENOGROUP;
+        return launch_gemm_q6k_mfma_group(A, in, M, K, s);
+    case CKQ_FMT_Q8_0:
+        if (K % 32) return CKQ_ESHAPE;
+        if (!gemm_q80_on_matrix_cores(M, rows * (K / 32) * 34, K % 64 == 0 && aligned)) return CKQ_ENOGROUP;
+        return launch_gemm_q80_mfma_group(A, in, M, K, s);
+    default:
+        return CKQ_ENOGROUP;
+    }
+}
+
 /* ---- the entry point that allocates nothing ---------------------------------
  * Scratch for the partial tiles of a K-split GEMM, held in the code object:
  * every device the library runs on holds its own copy, at its own address,

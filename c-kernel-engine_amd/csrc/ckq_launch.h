@@ -19,6 +19,7 @@ extern "C" {
 #define CKQ_ESHAPE  (-2)  /* K not a multiple of the block size */
 #define CKQ_EFORMAT (-3)  /* unknown format tag */
 #define CKQ_ESCRATCH (-4) /* the call needs more scratch than the entry point that allocates nothing holds */
+#define CKQ_ENOGROUP (-7) /* internal: a grouped GEMM launch was declined; the caller launches the matrices one by one */
 #define CKQ_ENODUMP (-6)  /* the integer dumps are compiled into libckernel_quant_hip_dump.so only */
 /* 1 in the test library (same sources, same templates, plus the DUMP instantiations that also
  * store the integers behind every output); 0 in the product library, which stays smaller for it. */
@@ -56,6 +57,11 @@ int ckq_launch_gemv(int fmt, float *y, const void *W, const void *X, const float
 int ckq_launch_gemv_group(int fmt, int n, float *const *y, const void *const *W, const void *const *X,
                           const float *const *bias, const int *rows, const long *ldys, int K, int ntok,
                           int32_t *subdots, void *stream);
+
+/* n (2..4) weight matrices of one format against the same M x K quantized activations as one
+ * matrix-core launch; CKQ_ENOGROUP when the matrices should be launched one by one instead. */
+int ckq_launch_gemm_group(int fmt, int n, float *const *C, const void *const *B, const void *A,
+                          const float *const *bias, const int *N, const long *ldc, int K, int M, void *stream);
 
 /* The matrix-core GEMM of `fmt` for any token count, its integer block sums
  * stored next to the result: sums[((t * N + n) * nblk + b) * per + i]; nblk =

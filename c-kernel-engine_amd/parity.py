@@ -246,7 +246,7 @@ def dev_gemm_block_sums(fmt, A_t, B_t, bias_t, M, N, K):
 
 
 def dev_matmul_sequence(ops, repeat=1):
-    """ops: list of matmul entries (fmt, A_t, B_t, bias_t, C_t, M, N, K) and producer
+    """ops: list of matmul entries (fmt, A_t, B_t, bias_t, C_t, M, N, K[, ldc]) and producer
     entries (step, A_t, B_t or None, C_t, M, K[, ld[, eps]]) with step one of
     "quantize_q8_k", "quantize_q8_0", "rmsnorm_q8_k", "swiglu_q8_k"; enqueued
     back-to-back `repeat` times by one C call (no Python between launches)."""
@@ -259,7 +259,8 @@ def dev_matmul_sequence(ops, repeat=1):
             arr[i] = MatmulOp(STEP[step], M, 0, K, ld, A_t.data_ptr(), B_t.data_ptr() if B_t is not None else None,
                               None, C_t.data_ptr(), eps)
         else:
-            fmt, A_t, B_t, bias_t, C_t, M, N, K = op
-            arr[i] = MatmulOp(fmt_tag(fmt), M, N, K, N, A_t.data_ptr(), B_t.data_ptr(),
+            fmt, A_t, B_t, bias_t, C_t, M, N, K = op[:8]
+            ldc = op[8] if len(op) > 8 else N
+            arr[i] = MatmulOp(fmt_tag(fmt), M, N, K, ldc, A_t.data_ptr(), B_t.data_ptr(),
                               bias_t.data_ptr() if bias_t is not None else None, C_t.data_ptr(), 0.0)
     check(lib().ckq_matmul_sequence_dev(ctypes.cast(arr, _vp), len(ops), repeat, _stream()), "ckq_matmul_sequence_dev")

@@ -283,10 +283,16 @@ int ckq_gemm_nt_f32act_dev(int fmt, const float *A, const void *B, const float *
  * per-token chain of a decoder layer (norm -> Q8_K -> Q/K/V ... -> down) is one
  * such list.  A matmul entry (fmt = a ckq_format weight tag) computes
  * C[m*ldc + n] as ckq_gemm_nt_dev does, with the same bits.  Up to four
- * consecutive matmul entries of one format, input width and token count (at
- * most eight tokens; their row counts may differ), none of which writes memory
- * another reads or writes (Q/K/V, gate/up of a decode step), are issued as ONE
- * launch.  A producer entry (fmt = one of CKQ_STEP_*) runs the activation
+ * consecutive matmul entries of one format, input width and token count (their
+ * row counts may differ), none of which writes memory another reads or writes
+ * (Q/K/V, gate/up), are issued as ONE launch: up to eight tokens by the
+ * weight-streaming kernel; beyond that, when the entries also read the same
+ * activations and their tiles together fill the chip, by the matrix-core GEMM
+ * (a prefill's K and V projections then share the grid of Q instead of taking a
+ * K-split launch each; every tile is computed as the unsplit single launch
+ * computes it, so an entry whose single launch would be split along K gets the
+ * unsplit summation order).  ckq_set_prefill_grouping(0) issues entries of more
+ * than eight tokens one by one.  A producer entry (fmt = one of CKQ_STEP_*) runs the activation
  * quantizer that feeds the matmuls after it, so that a whole chain is one C
  * call:
  *   CKQ_STEP_QUANTIZE_Q8_K  C = Q8_K blocks of the M rows of K floats at A_q8 (contiguous rows)
@@ -398,6 +404,10 @@ void ckq_weights_set_limit(size_t bytes);
  * the current device: the partial tiles of K-split GEMMs and rewritten Q5_0
  * weights.  Call it before destroying a stream that ran ckq_*_dev calls. */
 int  ckq_release_stream(void *stream);
+/* 1 (the default): ckq_matmul_sequence_dev issues independent consecutive entries of
+ * more than eight tokens that share their activations as one matrix-core launch;
+ * 0: one launch per entry.  No counterpart in the reference. */
+void ckq_set_prefill_grouping(int enabled);
 /* Thread-split entry points (*_parallel, *_parallel_simd): 0 (the default;
  * CKQ_PARALLEL_MODE=rows) = every call computes exactly the row range of its
  * ith, as the reference does (gemm_kernels_q4k_q8k.c:212-231), so a caller

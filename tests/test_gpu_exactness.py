@@ -462,6 +462,68 @@ def test_sequence_with_fp32_activation_entries():
         assert torch.equal(y0, y2) and torch.equal(y0, P.dev_gemm_nt(fmt, xq, W, None, M, N, K).view(-1))
 
 
+# ---- grouped matrix-core launches (Q/K/V, gate/up at prefill sizes) ------------------------------------
+
+@pytest.mark.parametrize("fmt,K", [("q4_k", 1024), ("q5_k", 1024), ("q6_k", 1024), ("q8_0", 512)])
+def test_grouped_prefill_launch_equals_single_launches(fmt, K):
+    """Three matrices of different, ragged heights against the same 500 tokens as
+    consecutive sequence entries go out as ONE matrix-core launch (168 tiles); every
+    output has the bits of the single-matrix launch (K is short enough that no
+    single launch is split along K), with and without bias, in a padded C."""
+    import torch
+    L = ckq.lib()
+    M, Ns = 500, [1536, 640, 392]
+    x = P.to_device(T.normal(M * K, 0.0, 1.0, seed=301))
+    xq = P.dev_quantize(x, T.act_fmt(fmt), rows=M)
+    Ws = [P.to_device(T.synth_weights(fmt, n, K, seed=302 + i)) for i, n in enumerate(Ns)]
+    bs = [None, P.to_device(T.normal(Ns[1], 0.0, 1.0, seed=310)), None]
+    L.ckq_set_gemm_policy(1)
+    try:
+        ldc = [n + 8 for n in Ns]
+        ys = [torch.full((M * l,), 7.0, dtype=torch.float32, device="cuda") for l in ldc]
+        say("grouped prefill launch", fmt, M, Ns, K)
+        P.dev_matmul_sequence([(fmt, xq, W, b, y, M, n, K, l) for W, b, y, n, l in zip(Ws, bs, ys, Ns, ldc)])
+        torch.cuda.synchronize()
+        for W, b, y, n, l in zip(Ws, bs, ys, Ns, ldc):
+            want = P.dev_gemm_nt(fmt, xq, W, b, M, n, K).view(M, n)
+            got = y.view(M, l)
+            assert torch.equal(got[:, :n], want), (fmt, n)
+            assert bool((got[:, n:] == 7.0).all()), "the padding of C stays untouched"
+        ref = T.oracle_gemm_nt(fmt, xq.cpu().numpy(), Ws[2].cpu().numpy(), None, M, Ns[2], K)
+        assert T.norm_err(ys[2].view(M, ldc[2])[:, :Ns[2]].cpu().numpy().reshape(-1), ref.reshape(-1)) <= TOL
+    finally:
+        L.ckq_set_gemm_policy(0)
+
+
+def test_grouped_prefill_launch_two_wave_groups_and_fallback():
+    """Q4_K, K = 2048: 168 tiles with eight K-steps take the two-wave-group form of the
+    kernel (each single launch would be split along K instead, so the comparison is
+    against the streaming kernel, token by token, at its tolerance); the same three
+    matrices against 100 tokens are too few tiles for a group and are issued one by
+    one, with the bits of the single calls."""
+    import torch
+    L = ckq.lib()
+    K, Ns = 2048, [1536, 640, 392]
+    Ws = [P.to_device(T.synth_weights("q4_k", n, K, seed=322 + i)) for i, n in enumerate(Ns)]
+    for M in (500, 100):
+        xq = P.dev_quantize(P.to_device(T.normal(M * K, 0.0, 1.0, seed=321)), "q8_k", rows=M)
+        ys = [torch.zeros(M * n, dtype=torch.float32, device="cuda") for n in Ns]
+        L.ckq_set_gemm_policy(1)
+        try:
+            say("grouped prefill launch, K=2048", M)
+            P.dev_matmul_sequence([("q4_k", xq, W, None, y, M, n, K) for W, y, n in zip(Ws, ys, Ns)])
+            torch.cuda.synchronize()
+            singles = [P.dev_gemm_nt("q4_k", xq, W, None, M, n, K).view(-1) for W, n in zip(Ws, Ns)]
+            L.ckq_set_gemm_policy(2)
+            streamed = [P.dev_gemm_nt("q4_k", xq, W, None, M, n, K).view(-1) for W, n in zip(Ws, Ns)]
+        finally:
+            L.ckq_set_gemm_policy(0)
+        for y, one, st in zip(ys, singles, streamed):
+            if M == 100:
+                assert torch.equal(y, one)
+            assert T.norm_err(y.cpu().numpy(), st.cpu().numpy()) <= 2e-6
+
+
 # ---- host-pointer paths with the weight cache off, long contexts ---------------------------------------
 
 def test_host_paths_with_weight_cache_off():
