@@ -507,9 +507,38 @@ def clock_trace(H, name, launches, seconds=1.6):
         if i is not None:
             pts.append([m, round(us[i], 2)])
     tail = us[-(len(us) // 3):]
+    probes = {}
+    if M > 8:
+        # what the first launches cost after other work or a short pause instead of a long idle: 12 repetitions of
+        # 10 launches right after (a) 150 ms of single-token launches of the same matrix, (b-d) 100 ms of this
+        # workload followed by a host sleep of 3 / 30 / 300 ms
+        x1 = P.dev_quantize(P.to_device(T.normal(K, 0.0, 1.0, seed=K)), T.act_fmt(fmt))
+        o1 = torch.empty(rows, dtype=torch.float32, device="cuda")
+        gemv = [(fmt, x1, c, None, o1, 1, rows, K) for c in copies]
+        est = max(statistics.median(tail), 1.0) * 1e-6
+
+        def first_reps():
+            e = [torch.cuda.Event(enable_timing=True) for _ in range(13)]
+            e[0].record()
+            for i in range(12):
+                P.dev_matmul_sequence(ops, repeat=max(1, 10 // n))
+                e[i + 1].record()
+            torch.cuda.synchronize()
+            per = max(1, 10 // n) * n
+            return [round(e[i].elapsed_time(e[i + 1]) * 1e3 / per, 1) for i in range(12)]
+
+        time.sleep(0.5)
+        P.dev_matmul_sequence(gemv, repeat=max(1, int(0.15 / 8e-6) // n))
+        probes["after_150ms_of_single_token_launches"] = first_reps()
+        for pause in (0.003, 0.03, 0.3):
+            P.dev_matmul_sequence(ops, repeat=max(1, int(0.1 / est) // n))
+            torch.cuda.synchronize()
+            time.sleep(pause)
+            probes["after_100ms_of_this_workload_then_%gms_idle" % (pause * 1e3)] = first_reps()
     print(json.dumps({"only": name, "clock_trace": True, "launches_per_repetition": launches, "repetitions": len(us),
                       "us_per_launch_at_ms_after_idle": pts,
-                      "settled_median_us": round(statistics.median(tail), 3), "sclk_during_second_half": sclk}))
+                      "settled_median_us": round(statistics.median(tail), 3), "sclk_during_second_half": sclk,
+                      "first_120_launches_us": probes}))
 
 
 def run_only(H, name, steps, warmup, calibrate, trace=False):
