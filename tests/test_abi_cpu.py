@@ -206,3 +206,32 @@ def test_no_device_fails_loudly():
     assert r.returncode != 0
     assert "survived" not in r.stdout
     assert "no CPU fallback" in r.stderr
+
+
+def test_dpp_hazard_checker(tmp_path):
+    """csrc/check_dpp.py, the build's check of the GEMMs' hand-written DPP
+    instructions: a VALU write of the broadcast register one instruction before
+    is a hazard, the same write behind an s_nop 1 or by an LDS read is not, and
+    a VALU write of EXEC needs five wait states."""
+    import importlib.util
+    path = os.path.join(os.path.dirname(ckq.lib_path()), "check_dpp.py")
+    spec = importlib.util.spec_from_file_location("check_dpp", path)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    dpp = "\tv_fmac_f32_dpp v10, v5, v7 row_newbcast:3 row_mask:0xf bank_mask:0xf\n"
+    cases = {
+        "valu_adjacent": ("\tv_cvt_f32_f16_e32 v5, v9\n" + dpp, 1),
+        "valu_two_back": ("\tv_cvt_f32_f16_e32 v5, v9\n\tv_mov_b32_e32 v1, v2\n" + dpp, 1),
+        "valu_three_back": ("\tv_cvt_f32_f16_e32 v5, v9\n\tv_mov_b32_e32 v1, v2\n\tv_mov_b32_e32 v3, v2\n" + dpp, 0),
+        "valu_then_nop": ("\tv_cvt_f32_f16_e32 v5, v9\n\ts_nop 1\n" + dpp, 0),
+        "lds_read": ("\tds_read_b32 v5, v9\n\ts_waitcnt lgkmcnt(0)\n" + dpp, 0),
+        "wide_write": ("\tv_pk_mul_lo_u16 v[4:5], v1, v2\n" + dpp, 1),
+        "other_register": ("\tv_mov_b32_e32 v6, v9\n" + dpp, 0),
+        "valu_exec": ("\tv_cmpx_lt_i32_e32 v1, v2\n\tv_mov_b32_e32 v1, v2\n\tv_mov_b32_e32 v3, v2\n" + dpp, 1),
+        "salu_exec": ("\ts_or_b64 exec, exec, s[6:7]\n" + dpp, 0),
+    }
+    for name, (text, want) in cases.items():
+        f = tmp_path / (name + ".s")
+        f.write_text(text)
+        count, bad = mod.check(str(f))
+        assert count == 1 and bad == want, (name, count, bad)
