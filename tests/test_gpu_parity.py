@@ -1156,3 +1156,36 @@ def test_matmul_sequence_keeps_order_where_entries_depend():
     assert np.array_equal(a1, a2) and np.array_equal(b1, b2)
     ref = P.dev_gemm_nt(fmt, x, W2, None, M, N, K).cpu().numpy().reshape(-1).view(np.uint32)
     assert np.array_equal(b1, ref)
+
+
+def test_host_inputs_stored_straight_into_device_memory_are_never_stale():
+    """Host-pointer calls copy small inputs with CPU stores into a device buffer the
+    next kernel reads (no upload launch).  3000 calls in a row, each with a
+    different activation vector of a different length and, every other call, a
+    bias: every result has the bits the device-pointer path gives for the same
+    inputs, so no call has read an earlier call's bytes."""
+    import torch
+    rng = np.random.default_rng(4711)
+    N = 384
+    Ks = [256, 512, 1024, 2048]
+    Wh = {K: T.synth_weights("q4_k", N, K, seed=900 + K) for K in Ks}
+    Wd = {K: P.to_device(Wh[K]) for K in Ks}
+    pool = {K: [T.oracle_quantize(T.normal(K, 0.0, 1.0 + 0.1 * i, seed=1000 * K + i), "q8_k") for i in range(24)] for K in Ks}
+    biases = [T.normal(N, 0.0, 1.0, seed=77 + i) for i in range(4)]
+    want = {}
+    for K in Ks:
+        for i, xq in enumerate(pool[K]):
+            for bi in (-1, 0, 1, 2, 3):
+                b = None if bi < 0 else P.to_device(biases[bi])
+                want[(K, i, bi)] = P.dev_gemm_nt("q4_k", P.to_device(xq), Wd[K], b, 1, N, K).cpu().numpy().reshape(-1)
+    torch.cuda.synchronize()
+    say("3000 host-pointer calls with changing inputs")
+    bad = 0
+    for it in range(3000):
+        K = Ks[int(rng.integers(len(Ks)))]
+        i = int(rng.integers(24))
+        bi = int(rng.integers(4)) if it & 1 else -1
+        xq = pool[K][i].copy()                      # a fresh host address most of the time
+        got = P.gemm_nt("q4_k", xq, Wh[K], None if bi < 0 else biases[bi], 1, N, K).reshape(-1)
+        bad += int(not np.array_equal(got, want[(K, i, bi)]))
+    assert bad == 0, "%d of 3000 calls read stale inputs" % bad
