@@ -24,7 +24,9 @@ def row_bytes(fmt, k):
 
 
 def lib_path():
-    return os.path.join(CSRC, "libckernel_quant_hip.so")
+    """The product library; CKQ_LIBRARY names another build of it to load instead (the UBSan
+    build of the host layer, `make -C csrc ubsan`)."""
+    return os.environ.get("CKQ_LIBRARY") or os.path.join(CSRC, "libckernel_quant_hip.so")
 
 
 def dump_lib_path():
