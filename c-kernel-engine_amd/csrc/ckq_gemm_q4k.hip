@@ -97,7 +97,11 @@ __device__ __forceinline__ void gemm_block_pipe(const GemmStage &st, u32 wofs, c
     const u32 h0 = (u32)hv[0], h1 = (u32)hv[1], h2 = (u32)hv[2], h3 = (u32)hv[3];
     const u32 sc03 = h1 & 0x3f3f3f3fu;
     const u32 sc47 = (h3 & 0x0f0f0f0fu) | (((h1 >> 6) & 0x03030303u) << 4);
-    const float dw = h2f(h0 & 0xffff), dmin = h2f(h0 >> 16);
+    float dw = h2f(h0 & 0xffff);
+    const float dmin = h2f(h0 >> 16);
+    /* dw as a float of its own: folded into the combine as an fp16 operand (v_fma_mix) its result would need
+     * a wait state in front of every lane-broadcast multiply-add that consumes it */
+    asm volatile("" : "+v"(dw));
 
     /* the two 3-bit halves of the eight scales, four per word; byte k of a word
      * becomes the u16 pair {k-th, k-th} a plane is multiplied by with one v_perm_b32
@@ -159,6 +163,7 @@ __device__ __forceinline__ void gemm_block_pipe(const GemmStage &st, u32 wofs, c
         if (s + 2 < 16) av[(s + 2) % 3] = a_read(s + 2);
         /* the first step of each token half starts from a literal zero accumulator */
         aH[ts] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[s % 3], bH[j], (s == 0 || s == 4) ? zero16 : aH[ts], 0, 0, 0);
+        CKQ_PIN();     /* the MFMA first: VALU work that reads the previous MFMAs' results would otherwise wait in front of it */
         /* VALU work placed under this step's two MFMAs */
         if (s < 3) decode(s + 1);                    /* pass 1: planes 1..3 */
         else if (s >= 4 && s < 8) decode(s);         /* pass 2: planes 4..7 */
