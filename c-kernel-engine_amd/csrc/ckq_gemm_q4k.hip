@@ -37,26 +37,9 @@
  * 32w..32w+31.  Grid: token tiles fastest inside an XCD so the eight XCD L2s
  * each see a weight tile once.
  */
-#include "ckq_gemm_common.hpp"
+#include "ckq_gemm_q4k.hpp"
+#include <atomic>
 #include <type_traits>
-
-#ifndef CKQ_GEMM_WPE
-#define CKQ_GEMM_WPE 2          /* waves per SIMD the register budget is sized for */
-#endif
-
-/* packed u8x4 times a small scalar, byte-wise (every product < 256) */
-__device__ __forceinline__ int mul_bytes(u32 v, u32 s16x2)
-{
-    const ckq_v2u16 a = __builtin_bit_cast(ckq_v2u16, v), b = __builtin_bit_cast(ckq_v2u16, s16x2);
-    return __builtin_bit_cast(int, (ckq_v2u16)(a * b));
-}
-
-/* two floats whose low 16 bits are zero (integers of at most 8 significant
- * bits) -> their bf16 forms in one dword, lo in the low half: one v_perm_b32 */
-__device__ __forceinline__ u32 bf16_pair(float lo, float hi)
-{
-    return __builtin_amdgcn_perm(__builtin_bit_cast(u32, hi), __builtin_bit_cast(u32, lo), 0x07060302u);
-}
 
 constexpr int GEMM_BM = 64;     /* tokens per tile */
 constexpr int GEMM_BN = GEMM_TILE_ROWS;    /* weight rows per tile */
@@ -369,6 +352,23 @@ __global__ void __launch_bounds__(256 * KG, KG == 2 ? 1 : WPE) gemm_q4k_mfma_ker
     }
 }
 
+/* Which token tile a launch takes.  A 96-token tile (ckq_gemm_q4k_t96.hip) costs 1.37 times a 64-token one for 1.5
+ * times the tokens, in blocks that run that much longer and leave a 32- or 64-token remainder tile that costs 0.6 / 0.8 of
+ * a whole one: it pays when the grid is one round of whole tiles (two blocks per CU) or at least a round and a half deep,
+ * and loses when a few long blocks are left over for a second round (512 tokens x 11008 rows: 516 blocks on 512 slots,
+ * 67 us against 62).  `tiles64`: tiles of the 64-token kernel, `blocks96`: blocks of the 96-token one. */
+static std::atomic<int> g_q4k_tile{0};
+extern "C" void ckq_launch_set_q4k_tile(int tokens) { g_q4k_tile.store(tokens == 64 || tokens == 96 ? tokens : 0); }
+static bool q4k_take_t96(int M, int tiles64, int blocks96)
+{
+    const int forced = g_q4k_tile.load(std::memory_order_relaxed);
+    if (forced) return forced == 96;
+    constexpr int SLOTS = 512;                /* 256 CUs, two blocks each */
+    if (M < 576 || tiles64 <= 256) return false;
+    if (blocks96 <= SLOTS) return M % 96 == 0;
+    return 2 * blocks96 >= 3 * SLOTS;
+}
+
 int launch_gemm_q4k_mfma(const void *A, const void *B, const float *bias, float *C,
                          int M, int N, int K, long ldc, const GemmOpts &opts, hipStream_t s)
 {
@@ -391,6 +391,7 @@ int launch_gemm_q4k_mfma(const void *A, const void *B, const float *bias, float 
      * (11008x4096: 78 us against 88). */
     const int tiles = g.ntt * g.nnt, sp = gemm_choose_splits(tiles, g.nb);
     const bool two_groups = tiles * sp <= 256 && (g.nb + sp - 1) / sp >= 8;
+    if (q4k_take_t96(M, tiles, gemm_q4k_t96_token_tiles(M) * g.nnt)) return launch_gemm_q4k_t96(g, s);
     if (sums) {
 #if CKQ_WITH_DUMP
         if (two_groups) return gemm_launch_split(gemm_q4k_mfma_kernel<CKQ_GEMM_WPE, 2, true>, g, (unsigned)(g.ntt * nnt8), g.nb, s, 512);
@@ -410,6 +411,7 @@ int launch_gemm_q4k_mfma_group(const void *A, const GemmGroupIn &in, int M, int 
     GemmArgs g = {};
     g.A = (const uint8_t *)A; g.M = M; g.nb = K / 256;
     if ((long long)g.nb * 292 * GEMM_BN >= (1ll << 31)) return (int)hipErrorInvalidValue;
+    if (q4k_take_t96(M, tiles, gemm_group_tiles(in, M, 96))) return launch_gemm_q4k_t96_group(g, in, s);
     g.ntt = (M + GEMM_BM - 1) / GEMM_BM;
     /* as for one matrix: two groups of waves per tile while every tile gets a CU of its own */
     if (tiles <= 256 && g.nb >= 8) return gemm_launch_grouped(gemm_q4k_mfma_kernel<CKQ_GEMM_WPE, 2>, g, in, s, 512);

@@ -690,6 +690,7 @@ void ckq_weights_set_cache(int enabled)
 }
 
 void ckq_set_gemm_policy(int policy) { ckq_launch_set_gemm_policy(policy); }
+void ckq_set_q4k_prefill_tile(int tokens) { ckq_launch_set_q4k_tile(tokens); }
 
 static int g_prefill_grouping = 1;
 void ckq_set_prefill_grouping(int enabled)

@@ -73,6 +73,8 @@ int ckq_launch_gemm_block_sums(int fmt, const void *A, const void *B, const floa
 /* Kernel choice for more than eight tokens: 0 = by token count and weight size
  * (default), 1 = always the matrix-core GEMM, 2 = always the streaming kernel. */
 void ckq_launch_set_gemm_policy(int policy);
+/* Token tile of the Q4_K x Q8_K matrix-core GEMM: 0 = by shape (default), 64 or 96 = always that kernel. */
+void ckq_launch_set_q4k_tile(int tokens);
 
 /* fp32 [rows x k] -> Q8_K / Q8_0 blocks, row-major. */
 int ckq_launch_quantize_q8_k(const float *x, void *y, int rows, int k, void *stream);

@@ -624,3 +624,84 @@ def test_f32act_gemv_with_more_tokens_than_grid_y():
     want = T.oracle_gemm_nt_f32act(fmt, A, W, None, M, N, K)
     assert T.norm_err(got, want) <= TOL
     assert T.norm_err(got[65530:65540], want[65530:65540]) <= TOL
+
+
+# ---- Q4_K x Q8_K on 96-token tiles -------------------------------------------------------------------
+
+Q4K_T96_SHAPES = [
+    # (M, N, K): one, two and three token groups in the last tile, ragged rows, one to six K-blocks (odd and even)
+    (96, 128, 512), (97, 130, 1024), (150, 300, 256), (33, 256, 768), (64, 200, 1536), (200, 128, 512), (500, 260, 1280),
+]
+
+
+def test_q4k_96_token_tiles_integer_block_sums_bit_exact():
+    """The 96-token kernel forced for every shape: I1 / I2 per (token, row, block) against brute
+    force - the carried group of each block included, whose sums are stored one block late - and the
+    fp32 result of the dump build, of the production build and of the 64-token kernel agree bit for bit
+    (neither splits K nor puts two wave groups on a tile at these sizes)."""
+    L, D = ckq.lib(), ckq.dump_lib()       # each library has its own switch
+    try:
+        D.ckq_set_q4k_prefill_tile(96)
+        for M, N, K in Q4K_T96_SHAPES:
+            W, A = rand_case("q4_k", N, K, 5 * M + N + K, tokens=M)
+            say("q4_k 96-token tiles", M, N, K)
+            Ad, Wd = P.to_device(A), P.to_device(W)
+            b = P.to_device(T.normal(N, 0.0, 1.0, seed=N))
+            L.ckq_set_q4k_prefill_tile(96)
+            c, sums = P.dev_gemm_block_sums("q4_k", Ad, Wd, b, M, N, K)
+            assert np.array_equal(sums.cpu().numpy().astype(np.int64), np_block_sums("q4_k", W, A, M, N, K)), (M, N, K)
+            L.ckq_set_gemm_policy(1)
+            prod96 = P.dev_gemm_nt("q4_k", Ad, Wd, b, M, N, K).cpu().numpy()
+            L.ckq_set_q4k_prefill_tile(64)
+            prod64 = P.dev_gemm_nt("q4_k", Ad, Wd, b, M, N, K).cpu().numpy()
+            L.ckq_set_gemm_policy(0)
+            assert np.array_equal(c.cpu().numpy(), prod96), (M, N, K)
+            assert np.array_equal(prod96, prod64), (M, N, K)
+            assert T.norm_err(prod96, T.oracle_gemm_nt("q4_k", A, W, b.cpu().numpy(), M, N, K)) <= TOL
+    finally:
+        L.ckq_set_gemm_policy(0)
+        L.ckq_set_q4k_prefill_tile(0)
+        D.ckq_set_q4k_prefill_tile(0)
+
+
+def test_q4k_96_token_tiles_chosen_by_shape_and_grouped():
+    """768 tokens x 8192 rows is one round of whole 96-token tiles: the default choice takes that kernel
+    (same bits as the 64-token kernel forced, which does not split K here either).  Three ragged matrices
+    against 500 tokens as ONE grouped launch of 96-token tiles: the bits of the single launches, the
+    padding of C untouched."""
+    import torch
+    L = ckq.lib()
+    try:
+        M, N, K = 768, 8192, 512
+        xq = P.dev_quantize(P.to_device(T.normal(M * K, 0.0, 1.0, seed=401)), "q8_k", rows=M)
+        W = P.to_device(T.synth_weights("q4_k", N, K, seed=402))
+        say("q4_k tile by shape", M, N, K)
+        L.ckq_set_gemm_policy(1)
+        auto = P.dev_gemm_nt("q4_k", xq, W, None, M, N, K).clone()
+        L.ckq_set_q4k_prefill_tile(64)
+        t64 = P.dev_gemm_nt("q4_k", xq, W, None, M, N, K).clone()
+        L.ckq_set_q4k_prefill_tile(96)
+        t96 = P.dev_gemm_nt("q4_k", xq, W, None, M, N, K).clone()
+        assert torch.equal(auto, t64) and torch.equal(auto, t96)
+        rows = [0, 95, 96, 767]
+        ref = T.oracle_gemm_nt("q4_k", xq.view(M, -1)[rows].cpu().numpy().reshape(-1), W.cpu().numpy(), None, len(rows), N, K)
+        assert T.norm_err(auto.view(M, N)[rows].cpu().numpy().reshape(-1), ref.reshape(-1)) <= TOL
+
+        M, K, Ns = 500, 1024, [1536, 640, 392]
+        xq = P.dev_quantize(P.to_device(T.normal(M * K, 0.0, 1.0, seed=411)), "q8_k", rows=M)
+        Ws = [P.to_device(T.synth_weights("q4_k", n, K, seed=412 + i)) for i, n in enumerate(Ns)]
+        bs = [None, P.to_device(T.normal(Ns[1], 0.0, 1.0, seed=420)), None]
+        ldc = [n + 8 for n in Ns]
+        ys = [torch.full((M * l,), 7.0, dtype=torch.float32, device="cuda") for l in ldc]
+        say("q4_k grouped launch of 96-token tiles", M, Ns, K)
+        P.dev_matmul_sequence([("q4_k", xq, W, b, y, M, n, K, l) for W, b, y, n, l in zip(Ws, bs, ys, Ns, ldc)])
+        torch.cuda.synchronize()
+        L.ckq_set_q4k_prefill_tile(64)
+        for W, b, y, n, l in zip(Ws, bs, ys, Ns, ldc):
+            want = P.dev_gemm_nt("q4_k", xq, W, b, M, n, K).view(M, n)
+            got = y.view(M, l)
+            assert torch.equal(got[:, :n], want), n
+            assert bool((got[:, n:] == 7.0).all()), "the padding of C stays untouched"
+    finally:
+        L.ckq_set_gemm_policy(0)
+        L.ckq_set_q4k_prefill_tile(0)
