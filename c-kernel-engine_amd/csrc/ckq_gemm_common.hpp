@@ -205,6 +205,22 @@ __device__ __forceinline__ int mfma32_row_of_lane(int lane)
     return 8 * ((lane & 15) >> 2) + 4 * (lane >> 5) + (lane & 3);
 }
 
+/* A result leaves the chip once: the K-quant kernels store theirs non-temporally (whole 128-byte runs per wave
+ * instruction; a tile's results are not read again by the launch that writes them, and the next launch runs on other
+ * XCDs' L2s anyway): 1-2 % per launch.  The Q8_0 kernel, whose lanes store 16 bytes each to different rows, is 5-14 %
+ * slower that way and keeps plain stores. */
+#ifndef CKQ_GEMM_NT_STORE
+#define CKQ_GEMM_NT_STORE 1
+#endif
+__device__ __forceinline__ void gemm_store(float *p, float v)
+{
+#if CKQ_GEMM_NT_STORE
+    __builtin_nontemporal_store(v, p);
+#else
+    *p = v;
+#endif
+}
+
 /* Grouped launch: the matrices of `in` against the same M x K activations, as one grid (no K split; the
  * callers group only what fills the chip without one).  rows_per_tile = weight rows of a block's tile. */
 struct GemmGroupIn {

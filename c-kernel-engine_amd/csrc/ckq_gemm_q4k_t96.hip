@@ -361,7 +361,7 @@ __global__ void __launch_bounds__(256, DUMP ? 1 : WPE) gemm_q4k_t96_kernel(GemmA
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int t = t0 + 32 * g + 8 * (r >> 2) + 4 * half + (r & 3);
-                if (t < a.M) o.C[(size_t)t * o.ldc + n] = acc[g][r] + bias;
+                if (t < a.M) gemm_store(&o.C[(size_t)t * o.ldc + n], acc[g][r] + bias);
             }
     }
 }

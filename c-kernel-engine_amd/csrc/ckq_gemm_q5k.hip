@@ -302,7 +302,7 @@ __global__ void __launch_bounds__(256, 1) gemm_q5k_mfma_kernel(GemmArgs a)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int t = t0 + 32 * ts + 8 * (r >> 2) + 4 * half + (r & 3);
-                if (t < a.M) o.C[(size_t)t * o.ldc + n] = acc[ts][r] + bias;
+                if (t < a.M) gemm_store(&o.C[(size_t)t * o.ldc + n], acc[ts][r] + bias);
             }
     }
 }

@@ -176,6 +176,8 @@ static int init_locked(void)
     const char *gp = getenv("CKQ_GEMM_POLICY");
     if (gp && strcmp(gp, "matrix") == 0) ckq_launch_set_gemm_policy(CKQ_GEMM_MATRIX);
     if (gp && strcmp(gp, "stream") == 0) ckq_launch_set_gemm_policy(CKQ_GEMM_STREAM);
+    const char *tile = getenv("CKQ_Q4K_TILE");
+    if (tile) ckq_launch_set_q4k_tile(atoi(tile));
     /* address of the static scratch of the entry point that allocates nothing, for this device */
     {
         const int rc = ckq_launch_noalloc_setup();

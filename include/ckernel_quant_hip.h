@@ -430,8 +430,8 @@ void ckq_set_gemm_policy(int policy);
 /* Token tile of the Q4_K x Q8_K matrix-core GEMM.  Two kernels compute the same sums in the same order: tiles of 128
  * rows x 64 tokens, and tiles of 128 rows x 96 tokens, which need fewer instructions per token in blocks that run
  * longer.  0, the default, picks by shape (96 where the grid is one round of whole tiles or at least a round and a
- * half deep); 64 or 96 force one of them (tests, tuning).  Results are bit-identical wherever neither launch splits K
- * or puts two wave groups on a tile. */
+ * half deep); 64 or 96 force one of them (tests, tuning; CKQ_Q4K_TILE=64|96 sets it from the environment).  Results are
+ * bit-identical wherever neither launch splits K or puts two wave groups on a tile. */
 void ckq_set_q4k_prefill_tile(int tokens);
 /* Last error of the calling process (0 = none), its text, and a reset for
  * callers that run with CKQ_ABORT_ON_ERROR=0 and handle errors themselves. */
