@@ -148,7 +148,7 @@ _SIGS = {
     "ckq_set_parallel_whole": (None, [_i]),
     "ckq_set_prefill_grouping": (None, [_i]),
     "ckq_set_gemm_policy": (None, [_i]),
-    "ckq_set_q4k_prefill_tile": (None, [_i]),
+    "ckq_set_prefill_variant": (None, [_i, _i]),
     "ckq_last_error": (_i, []),
     "ckq_clear_error": (None, []),
     "ckq_error_string": (_c.c_char_p, [_i]),

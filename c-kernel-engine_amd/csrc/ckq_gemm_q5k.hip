@@ -30,6 +30,7 @@
  * Block = 4 waves = 64 tokens x 128 weight rows; wave w owns rows 32w..32w+31.
  */
 #include "ckq_gemm_common.hpp"
+#include <atomic>
 #include <type_traits>
 
 constexpr int GEMM5_BM = 64, GEMM5_BN = 128, GEMM5_ROW = 176;
@@ -43,13 +44,14 @@ struct Gemm5Stage {
 
 /* One 256-block of a tile.  The planes of slab s+1 are expanded between the
  * MFMAs of slab s; copy_one(i) issues one global->LDS copy of a later block. */
-template <int NCOPY, bool DUMP, class CopyFn>
-__device__ __forceinline__ void gemm5_block(const Gemm5Stage &st, u32 wrow, const u32 (&aofs)[8], int col, int half,
-                                            ckq_v16f (&acc)[2], CopyFn copy_one, const GemmDumpLane &dl)
+template <int NCOPY, bool DUMP, class CopyFn, class AfterFn>
+__device__ __forceinline__ void gemm5_block(const uint8_t *w, const uint8_t *q, const uint8_t *bsum, const float *d, u32 wrow,
+                                            const u32 (&aofs)[8], int col, int half, ckq_v16f (&acc)[2], CopyFn copy_one,
+                                            AfterFn after_weights, const GemmDumpLane &dl)
 {
 #define CKQ_PIN() __builtin_amdgcn_sched_barrier(0)
     auto lds16 = [&](const void *p) { return *reinterpret_cast<const ckq_v4i *>(p); };
-    const uint8_t *wr = st.w + wrow;
+    const uint8_t *wr = w + wrow;
 
     /* raw block of this lane's row: header, fifth bits and nibbles its k-half touches */
     const ckq_v4i hv = lds16(wr);
@@ -61,7 +63,7 @@ __device__ __forceinline__ void gemm5_block(const Gemm5Stage &st, u32 wrow, cons
     ckq_v4i av[2][2];
     auto a_read = [&](int s) {
 #pragma unroll
-        for (int ts = 0; ts < 2; ++ts) av[s & 1][ts] = lds16(&st.q[aofs[s] + 32 * 256 * ts]);
+        for (int ts = 0; ts < 2; ++ts) av[s & 1][ts] = lds16(&q[aofs[s] + 32 * 256 * ts]);
     };
     a_read(0);
 
@@ -72,9 +74,9 @@ __device__ __forceinline__ void gemm5_block(const Gemm5Stage &st, u32 wrow, cons
     const int dx_tok = mfma32_row_of_lane(col + 32 * half);
 #pragma unroll
     for (int ts = 0; ts < 2; ++ts) {
-        dx[ts] = __builtin_bit_cast(float, *reinterpret_cast<const int *>(&st.d[32 * ts + dx_tok]));
-        bs[ts][0] = lds16(&st.b[(col + 32 * ts) * 32]);
-        bs[ts][1] = lds16(&st.b[(col + 32 * ts) * 32 + 16]);
+        dx[ts] = __builtin_bit_cast(float, *reinterpret_cast<const int *>(&d[32 * ts + dx_tok]));
+        bs[ts][0] = lds16(&bsum[(col + 32 * ts) * 32]);
+        bs[ts][1] = lds16(&bsum[(col + 32 * ts) * 32 + 16]);
     }
 
     const u32 h0 = (u32)hv[0], h1 = (u32)hv[1], h2 = (u32)hv[2], h3 = (u32)hv[3];
@@ -140,6 +142,11 @@ __device__ __forceinline__ void gemm5_block(const Gemm5Stage &st, u32 wrow, cons
             const int ts = k >> 1;
             if ((k & 1) == 0) iL[ts] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[s & 1][ts], pL[s & 1], s == 0 ? zero16 : iL[ts], 0, 0, 0);
             else              iH[ts] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[s & 1][ts], pH[s & 1], s == 0 ? zero16 : iH[ts], 0, 0, 0);
+            if (s == 0 && k == 0) {
+                CKQ_PIN();
+                after_weights();      /* the paired kernel: the weight image is in registers, it may take the next block */
+                CKQ_PIN();
+            }
             /* VALU work under this MFMA: a dword of the next slab's planes */
             if (s < 7) decode(s + 1, k);
             if (k == 0 && s < 7) a_read(s + 1);       /* operands of the next slab, three MFMAs ahead of their use */
@@ -281,7 +288,7 @@ __global__ void __launch_bounds__(256, 1) gemm_q5k_mfma_kernel(GemmArgs a)
             dl.tok_left = a.M - tf;
             dl.row_ok = n < work.N;
         }
-        gemm5_block<NCOPY, DUMP>(stage[cur], wrow, aofs, col, half, acc, copy_one, dl);
+        gemm5_block<NCOPY, DUMP>(stage[cur].w, stage[cur].q, stage[cur].b, stage[cur].d, wrow, aofs, col, half, acc, copy_one, [] {}, dl);
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_waitcnt(0x0070 | (NCOPY & 15) | ((NCOPY >> 4) << 14));
         __builtin_amdgcn_s_barrier();
@@ -307,6 +314,144 @@ __global__ void __launch_bounds__(256, 1) gemm_q5k_mfma_kernel(GemmArgs a)
     }
 }
 
+/* Two blocks per CU: ONE LDS image of the weights and two of the activations, bsums and scales (59 KB).  A lane takes
+ * its row's whole raw block into registers at the start of a 256-block, so a barrier behind those reads frees the
+ * image for the next block's weights; a second, independent block on the CU runs its MFMAs under this one's plane
+ * expansion and fp32 combine and fills the waits of the shallower pipeline (a fetch has one iteration to land
+ * instead of two).  Every LDS region is an object of its own: the compiler then puts no wait for a copy in front
+ * of the reads of another region.  Same sums in the same order as gemm_q5k_mfma_kernel. */
+template <bool DUMP>
+__global__ void __launch_bounds__(256, 2) gemm_q5k_pair_kernel(GemmArgs a)
+{
+    constexpr int BM = GEMM5_BM;
+    __shared__ __attribute__((aligned(16))) uint8_t wimg[GEMM5_BN * GEMM5_ROW];
+    __shared__ __attribute__((aligned(16))) uint8_t q_even[BM * 256], q_odd[BM * 256];
+    __shared__ __attribute__((aligned(16))) uint8_t b_even[BM * 32], b_odd[BM * 32];
+    __shared__ __attribute__((aligned(16))) float d_even[BM], d_odd[BM];
+    auto qst = [&](auto c) __attribute__((always_inline)) -> uint8_t * { if constexpr (decltype(c)::value == 0) return q_even; else return q_odd; };
+    auto bst = [&](auto c) __attribute__((always_inline)) -> uint8_t * { if constexpr (decltype(c)::value == 0) return b_even; else return b_odd; };
+    auto dst = [&](auto c) __attribute__((always_inline)) -> float * { if constexpr (decltype(c)::value == 0) return d_even; else return d_odd; };
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = wave_in_block();
+    const int col = lane & 31, half = lane >> 5;
+
+    const GemmWork work = gemm_work(a, a.nb);
+    const int id = work.id, xcd = id & 7, seq = id >> 3;
+    const int tt = seq % a.ntt;
+    const int nt = (seq / a.ntt) * 8 + xcd;
+    if (nt >= work.nnt) return;
+    const int t0 = tt * BM, n0 = nt * GEMM5_BN;
+    const u32 wstride = (u32)a.nb * 176u, xstride = (u32)a.nb * 292u;
+    const int b0 = work.k0, b1 = work.k1, last = b1 - 1;
+    const uint8_t *wbase = work.B + (size_t)n0 * wstride;
+    const uint8_t *xbase = a.A + (size_t)t0 * xstride;
+
+    /* copy roles as in gemm_q5k_mfma_kernel */
+    constexpr int NWI = 6, NQI = 4, NCOPY = NWI + NQI + 2;
+    u32 wofs_g[NWI], qofs_g[NQI], dofs_g, bofs_g;
+#pragma unroll
+    for (int i = 0; i < NWI; ++i) {
+        const int chunk = min(wave + 4 * i, 21) * 64 + lane, row = min(chunk / 11, work.N - 1 - n0), part = chunk % 11;
+        wofs_g[i] = (u32)row * wstride + 16u * part;
+    }
+#pragma unroll
+    for (int i = 0; i < NQI; ++i) {
+        const int tl = 4 * (wave + 4 * i) + (lane >> 4), c = (lane & 15) ^ (tl & 15);
+        qofs_g[i] = (u32)min(tl, a.M - 1 - t0) * xstride + 4u + 16u * c;
+    }
+    dofs_g = (u32)min(lane, a.M - 1 - t0) * xstride;
+    {
+        const int e = (wave & 1) * 64 + lane;
+        bofs_g = (u32)min(e >> 1, a.M - 1 - t0) * xstride + 260u + 16u * (u32)(e & 1);
+    }
+    const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc((void *)wbase, 0, 0x7fffffff, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rs_x = __builtin_amdgcn_make_buffer_rsrc((void *)xbase, 0, 0x7fffffff, 0x00020000);
+    int cp_w = 0, cp_x = 0;
+    auto copy_begin = [&](int b) __attribute__((always_inline)) {
+        cp_w = b * 176;
+        cp_x = b * 292;
+    };
+    auto copy_one = [&](int i, auto bufc) __attribute__((always_inline)) {
+        if (i < NWI)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (ckq_lds_void *)(wimg + 1024 * min(wave + 4 * i, 21)), 16, (int)(wofs_g[i]), cp_w, 0, 0);
+        else if (i < NWI + NQI)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, (ckq_lds_void *)(qst(bufc) + 1024 * (wave + 4 * (i - NWI))), 16,
+                                                     (int)qofs_g[i - NWI], cp_x, 0, 0);
+        else if (i == NWI + NQI)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, (ckq_lds_void *)(dst(bufc)), 4, (int)(dofs_g), cp_x, 0, 0);
+        else
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, (ckq_lds_void *)(bst(bufc) + 1024 * (wave & 1)), 16, (int)(bofs_g), cp_x, 0, 0);
+    };
+
+    const u32 wrow = (u32)(32 * wave + col) * (u32)GEMM5_ROW;
+    u32 aofs[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) aofs[s] = (u32)col * 256u + 16u * (u32)((2 * s + half) ^ (col & 15));
+
+    ckq_v16f acc[2];
+#pragma unroll
+    for (int ts = 0; ts < 2; ++ts)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[ts][r] = 0.0f;
+
+    copy_begin(b0);
+#pragma unroll
+    for (int i = 0; i < NCOPY; ++i) copy_one(i, std::integral_constant<int, 0>{});
+    __builtin_amdgcn_s_waitcnt(0x0070);
+    __builtin_amdgcn_s_barrier();
+
+    auto kstep = [&](int b, auto curc) __attribute__((always_inline)) {
+        constexpr int cur = decltype(curc)::value;
+        GemmDumpLane dl = {};
+        if constexpr (DUMP) {
+            const int n = n0 + wave * 32 + col, tf = t0 + 4 * half;
+            dl.tok_stride = gemm_opaque((size_t)work.N * a.nb * 2);
+            dl.p = a.dump + ((size_t)tf * work.N + n) * a.nb * 2 + (size_t)b * 2;
+            dl.tok_left = a.M - tf;
+            dl.row_ok = n < work.N;
+        }
+        auto after_weights = [&]() __attribute__((always_inline)) {
+            __builtin_amdgcn_s_waitcnt(0xc07f);      /* lgkmcnt(0): this wave's reads of the images have returned */
+            __builtin_amdgcn_s_barrier();
+            copy_begin(min(b + 1, last));
+        };
+        auto copy_next = [&](int i) __attribute__((always_inline)) { copy_one(i, std::integral_constant<int, cur ^ 1>{}); };
+        __builtin_amdgcn_sched_barrier(0);
+        gemm5_block<NCOPY, DUMP>(wimg, qst(curc), bst(curc), dst(curc), wrow, aofs, col, half, acc, copy_next, after_weights, dl);
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(0x0070);
+        __builtin_amdgcn_s_barrier();
+    };
+    for (int b = b0; b < b1; b += 2) {
+        kstep(b, std::integral_constant<int, 0>{});
+        if (b + 1 < b1) kstep(b + 1, std::integral_constant<int, 1>{});
+    }
+
+    const GemmOut o = work.out;
+    const int n = n0 + wave * 32 + col;
+    if (n < work.N) {
+        const float bias = o.bias ? o.bias[n] : 0.0f;
+#pragma unroll
+        for (int ts = 0; ts < 2; ++ts)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int t = t0 + 32 * ts + 8 * (r >> 2) + 4 * half + (r & 3);
+                if (t < a.M) gemm_store(&o.C[(size_t)t * o.ldc + n], acc[ts][r] + bias);
+            }
+    }
+}
+
+/* More tiles than CUs: the paired kernel (512 x 11008, K = 4096: 99.2 -> 85.3 us; 2048 tokens: 374 -> 320; 512 x 8192:
+ * 67.9 -> 60.4); up to one tile per CU the three-stage kernel, whose deeper pipeline serves a block that has its CU to
+ * itself (256 tiles: 81.7 against 83.0).  variant: 0 = by tile count, 1 = one block per CU always, 2 = paired always. */
+static std::atomic<int> g_q5k_variant{0};
+extern "C" void ckq_launch_set_q5k_variant(int variant) { g_q5k_variant.store(variant == 1 || variant == 2 ? variant : 0); }
+static bool q5k_take_pair(int tiles)
+{
+    const int forced = g_q5k_variant.load(std::memory_order_relaxed);
+    return forced ? forced == 2 : tiles > 256;
+}
+
 int launch_gemm_q5k_mfma(const void *A, const void *B, const float *bias, float *C,
                          int M, int N, int K, long ldc, const GemmOpts &opts, hipStream_t s)
 {
@@ -322,6 +467,14 @@ int launch_gemm_q5k_mfma(const void *A, const void *B, const float *bias, float 
     g.ntt = (M + GEMM5_BM - 1) / GEMM5_BM;
     g.nnt = (N + GEMM5_BN - 1) / GEMM5_BN;
     const int nnt8 = (g.nnt + 7) / 8 * 8;
+    if (q5k_take_pair(g.ntt * g.nnt)) {
+#if CKQ_WITH_DUMP
+        if (sums) return gemm_launch_split(gemm_q5k_pair_kernel<true>, g, (unsigned)(g.ntt * nnt8), g.nb, s);
+#else
+        if (sums) return CKQ_ENODUMP;
+#endif
+        return gemm_launch_split(gemm_q5k_pair_kernel<false>, g, (unsigned)(g.ntt * nnt8), g.nb, s);
+    }
 #if CKQ_WITH_DUMP
     if (sums) return gemm_launch_split(gemm_q5k_mfma_kernel<true>, g, (unsigned)(g.ntt * nnt8), g.nb, s);
 #else
@@ -337,5 +490,6 @@ int launch_gemm_q5k_mfma_group(const void *A, const GemmGroupIn &in, int M, int 
     g.A = (const uint8_t *)A; g.M = M; g.nb = K / 256;
     if ((long long)g.nb * 292 * 128 >= (1ll << 31)) return (int)hipErrorInvalidValue;
     g.ntt = (M + GEMM5_BM - 1) / GEMM5_BM;
+    if (q5k_take_pair(gemm_group_tiles(in, M, GEMM5_BM))) return gemm_launch_grouped(gemm_q5k_pair_kernel<false>, g, in, s);
     return gemm_launch_grouped(gemm_q5k_mfma_kernel<false>, g, in, s);
 }

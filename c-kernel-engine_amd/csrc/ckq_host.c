@@ -178,6 +178,10 @@ static int init_locked(void)
     if (gp && strcmp(gp, "stream") == 0) ckq_launch_set_gemm_policy(CKQ_GEMM_STREAM);
     const char *tile = getenv("CKQ_Q4K_TILE");
     if (tile) ckq_launch_set_q4k_tile(atoi(tile));
+    const char *q6v = getenv("CKQ_Q6K_VARIANT");
+    if (q6v) ckq_launch_set_q6k_variant(atoi(q6v));
+    const char *q5v = getenv("CKQ_Q5K_VARIANT");
+    if (q5v) ckq_launch_set_q5k_variant(atoi(q5v));
     /* address of the static scratch of the entry point that allocates nothing, for this device */
     {
         const int rc = ckq_launch_noalloc_setup();
@@ -692,7 +696,12 @@ void ckq_weights_set_cache(int enabled)
 }
 
 void ckq_set_gemm_policy(int policy) { ckq_launch_set_gemm_policy(policy); }
-void ckq_set_q4k_prefill_tile(int tokens) { ckq_launch_set_q4k_tile(tokens); }
+void ckq_set_prefill_variant(int fmt, int variant)
+{
+    if (fmt == CKQ_FMT_Q4_K) ckq_launch_set_q4k_tile(variant);
+    else if (fmt == CKQ_FMT_Q6_K) ckq_launch_set_q6k_variant(variant);
+    else if (fmt == CKQ_FMT_Q5_K) ckq_launch_set_q5k_variant(variant);
+}
 
 static int g_prefill_grouping = 1;
 void ckq_set_prefill_grouping(int enabled)

@@ -75,6 +75,10 @@ int ckq_launch_gemm_block_sums(int fmt, const void *A, const void *B, const floa
 void ckq_launch_set_gemm_policy(int policy);
 /* Token tile of the Q4_K x Q8_K matrix-core GEMM: 0 = by shape (default), 64 or 96 = always that kernel. */
 void ckq_launch_set_q4k_tile(int tokens);
+/* Q6_K x Q8_K matrix-core GEMM: 0 = by shape (default), 1 = one block per CU always, 2 = the paired 64-token kernel always. */
+void ckq_launch_set_q6k_variant(int variant);
+/* Q5_K x Q8_K matrix-core GEMM: 0 = by tile count (default), 1 = one block per CU always, 2 = the paired kernel always. */
+void ckq_launch_set_q5k_variant(int variant);
 
 /* fp32 [rows x k] -> Q8_K / Q8_0 blocks, row-major. */
 int ckq_launch_quantize_q8_k(const float *x, void *y, int rows, int k, void *stream);

@@ -427,12 +427,19 @@ void ckq_set_parallel_whole(int enabled);
  * kernels meet the same tolerance; their fp32 summation orders differ. */
 enum { CKQ_GEMM_AUTO = 0, CKQ_GEMM_MATRIX = 1, CKQ_GEMM_STREAM = 2 };
 void ckq_set_gemm_policy(int policy);
-/* Token tile of the Q4_K x Q8_K matrix-core GEMM.  Two kernels compute the same sums in the same order: tiles of 128
- * rows x 64 tokens, and tiles of 128 rows x 96 tokens, which need fewer instructions per token in blocks that run
- * longer.  0, the default, picks by shape (96 where the grid is one round of whole tiles or at least a round and a
- * half deep); 64 or 96 force one of them (tests, tuning; CKQ_Q4K_TILE=64|96 sets it from the environment).  Results are
- * bit-identical wherever neither launch splits K or puts two wave groups on a tile. */
-void ckq_set_q4k_prefill_tile(int tokens);
+/* Variants of the matrix-core GEMMs (tests, tuning; 0, the default, picks by shape).  Every variant of a format computes
+ * the same sums in the same order: results are bit-identical wherever neither launch splits K or puts two wave groups
+ * on a tile.
+ *   CKQ_FMT_Q4_K: 64 or 96 = tiles of 128 rows x 64 tokens, or x 96 tokens - fewer instructions per token in blocks that run
+ *                 longer, taken where the grid is one round of whole tiles or at least a round and a half deep
+ *                 (CKQ_Q4K_TILE=64|96 in the environment);
+ *   CKQ_FMT_Q6_K: 1 = one block per CU (64-token tiles three LDS stages deep, 128-token tiles two), 2 = two blocks per CU
+ *                 on 64-token tiles with one LDS image of the weights, taken where the 128-token grid would waste a
+ *                 quarter or more of its last round (CKQ_Q6K_VARIANT=1|2);
+ *   CKQ_FMT_Q5_K: 1 = one block per CU, three LDS stages deep, 2 = two blocks per CU with one LDS image of the weights,
+ *                 taken for more tiles than CUs (CKQ_Q5K_VARIANT=1|2).
+ * Q8_0 has one variant. */
+void ckq_set_prefill_variant(int fmt, int variant);
 /* Last error of the calling process (0 = none), its text, and a reset for
  * callers that run with CKQ_ABORT_ON_ERROR=0 and handle errors themselves. */
 int         ckq_last_error(void);

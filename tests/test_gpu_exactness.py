@@ -641,18 +641,18 @@ def test_q4k_96_token_tiles_integer_block_sums_bit_exact():
     (neither splits K nor puts two wave groups on a tile at these sizes)."""
     L, D = ckq.lib(), ckq.dump_lib()       # each library has its own switch
     try:
-        D.ckq_set_q4k_prefill_tile(96)
+        D.ckq_set_prefill_variant(P.FMT["q4_k"], 96)
         for M, N, K in Q4K_T96_SHAPES:
             W, A = rand_case("q4_k", N, K, 5 * M + N + K, tokens=M)
             say("q4_k 96-token tiles", M, N, K)
             Ad, Wd = P.to_device(A), P.to_device(W)
             b = P.to_device(T.normal(N, 0.0, 1.0, seed=N))
-            L.ckq_set_q4k_prefill_tile(96)
+            L.ckq_set_prefill_variant(P.FMT["q4_k"], 96)
             c, sums = P.dev_gemm_block_sums("q4_k", Ad, Wd, b, M, N, K)
             assert np.array_equal(sums.cpu().numpy().astype(np.int64), np_block_sums("q4_k", W, A, M, N, K)), (M, N, K)
             L.ckq_set_gemm_policy(1)
             prod96 = P.dev_gemm_nt("q4_k", Ad, Wd, b, M, N, K).cpu().numpy()
-            L.ckq_set_q4k_prefill_tile(64)
+            L.ckq_set_prefill_variant(P.FMT["q4_k"], 64)
             prod64 = P.dev_gemm_nt("q4_k", Ad, Wd, b, M, N, K).cpu().numpy()
             L.ckq_set_gemm_policy(0)
             assert np.array_equal(c.cpu().numpy(), prod96), (M, N, K)
@@ -660,8 +660,8 @@ def test_q4k_96_token_tiles_integer_block_sums_bit_exact():
             assert T.norm_err(prod96, T.oracle_gemm_nt("q4_k", A, W, b.cpu().numpy(), M, N, K)) <= TOL
     finally:
         L.ckq_set_gemm_policy(0)
-        L.ckq_set_q4k_prefill_tile(0)
-        D.ckq_set_q4k_prefill_tile(0)
+        L.ckq_set_prefill_variant(P.FMT["q4_k"], 0)
+        D.ckq_set_prefill_variant(P.FMT["q4_k"], 0)
 
 
 def test_q4k_96_token_tiles_chosen_by_shape_and_grouped():
@@ -678,9 +678,9 @@ def test_q4k_96_token_tiles_chosen_by_shape_and_grouped():
         say("q4_k tile by shape", M, N, K)
         L.ckq_set_gemm_policy(1)
         auto = P.dev_gemm_nt("q4_k", xq, W, None, M, N, K).clone()
-        L.ckq_set_q4k_prefill_tile(64)
+        L.ckq_set_prefill_variant(P.FMT["q4_k"], 64)
         t64 = P.dev_gemm_nt("q4_k", xq, W, None, M, N, K).clone()
-        L.ckq_set_q4k_prefill_tile(96)
+        L.ckq_set_prefill_variant(P.FMT["q4_k"], 96)
         t96 = P.dev_gemm_nt("q4_k", xq, W, None, M, N, K).clone()
         assert torch.equal(auto, t64) and torch.equal(auto, t96)
         rows = [0, 95, 96, 767]
@@ -696,7 +696,7 @@ def test_q4k_96_token_tiles_chosen_by_shape_and_grouped():
         say("q4_k grouped launch of 96-token tiles", M, Ns, K)
         P.dev_matmul_sequence([("q4_k", xq, W, b, y, M, n, K, l) for W, b, y, n, l in zip(Ws, bs, ys, Ns, ldc)])
         torch.cuda.synchronize()
-        L.ckq_set_q4k_prefill_tile(64)
+        L.ckq_set_prefill_variant(P.FMT["q4_k"], 64)
         for W, b, y, n, l in zip(Ws, bs, ys, Ns, ldc):
             want = P.dev_gemm_nt("q4_k", xq, W, b, M, n, K).view(M, n)
             got = y.view(M, l)
@@ -704,4 +704,102 @@ def test_q4k_96_token_tiles_chosen_by_shape_and_grouped():
             assert bool((got[:, n:] == 7.0).all()), "the padding of C stays untouched"
     finally:
         L.ckq_set_gemm_policy(0)
-        L.ckq_set_q4k_prefill_tile(0)
+        L.ckq_set_prefill_variant(P.FMT["q4_k"], 0)
+
+
+# ---- Q6_K x Q8_K, two blocks per CU -------------------------------------------------------------------
+
+def test_q6k_paired_kernel_integer_block_sums_bit_exact_and_chosen_by_shape():
+    """The paired 64-token Q6_K kernel (one LDS image of the weights, two blocks per CU) forced over ragged
+    shapes and one to six K-blocks: the block sums against brute force, the fp32 result equal to the
+    one-block-per-CU kernels' bit for bit.  512 tokens x 11008 rows leave the 128-token grid a third of a
+    second round: the default choice takes the paired kernel there, with the same bits again."""
+    import torch
+    L, D = ckq.lib(), ckq.dump_lib()       # each library has its own switch
+    q6 = P.FMT["q6_k"]
+    try:
+        for M, N, K in [(70, 200, 1024), (130, 384, 768), (33, 128, 256), (500, 260, 1536), (64, 130, 512)]:
+            W, A = rand_case("q6_k", N, K, 7 * M + N + K, tokens=M)
+            say("q6_k paired kernel", M, N, K)
+            Ad, Wd = P.to_device(A), P.to_device(W)
+            b = P.to_device(T.normal(N, 0.0, 1.0, seed=N))
+            D.ckq_set_prefill_variant(q6, 2)
+            c, sums = P.dev_gemm_block_sums("q6_k", Ad, Wd, b, M, N, K)
+            assert np.array_equal(sums.cpu().numpy().astype(np.int64), np_block_sums("q6_k", W, A, M, N, K)), (M, N, K)
+            L.ckq_set_gemm_policy(1)
+            L.ckq_set_prefill_variant(q6, 2)
+            pair = P.dev_gemm_nt("q6_k", Ad, Wd, b, M, N, K).cpu().numpy()
+            L.ckq_set_prefill_variant(q6, 1)
+            lone = P.dev_gemm_nt("q6_k", Ad, Wd, b, M, N, K).cpu().numpy()
+            L.ckq_set_gemm_policy(0)
+            assert np.array_equal(c.cpu().numpy(), pair), (M, N, K)
+            assert np.array_equal(pair, lone), (M, N, K)
+            assert T.norm_err(pair, T.oracle_gemm_nt("q6_k", A, W, b.cpu().numpy(), M, N, K)) <= TOL
+        M, N, K = 512, 11008, 512
+        xq = P.dev_quantize(P.to_device(T.normal(M * K, 0.0, 1.0, seed=501)), "q8_k", rows=M)
+        W = P.to_device(T.synth_weights("q6_k", N, K, seed=502))
+        say("q6_k kernel by shape", M, N, K)
+        L.ckq_set_gemm_policy(1)
+        L.ckq_set_prefill_variant(q6, 0)
+        auto = P.dev_gemm_nt("q6_k", xq, W, None, M, N, K).clone()
+        L.ckq_set_prefill_variant(q6, 1)
+        lone = P.dev_gemm_nt("q6_k", xq, W, None, M, N, K).clone()
+        L.ckq_set_prefill_variant(q6, 2)
+        pair = P.dev_gemm_nt("q6_k", xq, W, None, M, N, K).clone()
+        assert torch.equal(auto, lone) and torch.equal(auto, pair)
+    finally:
+        L.ckq_set_gemm_policy(0)
+        L.ckq_set_prefill_variant(q6, 0)
+        D.ckq_set_prefill_variant(q6, 0)
+
+
+def test_q5k_paired_kernel_integer_block_sums_bit_exact_and_chosen_by_tile_count():
+    """The paired Q5_K kernel (one LDS image of the weights, two blocks per CU) forced over ragged shapes and
+    one to six K-blocks: I1 / I2 against brute force, the fp32 result equal to the three-stage kernel's bit
+    for bit.  640 tokens x 4096 rows are 320 tiles, more than CUs: the default choice takes the paired
+    kernel, with the same bits again; three ragged matrices as one grouped launch of it likewise."""
+    import torch
+    L, D = ckq.lib(), ckq.dump_lib()       # each library has its own switch
+    q5 = P.FMT["q5_k"]
+    try:
+        for M, N, K in [(70, 200, 1024), (130, 384, 768), (33, 128, 256), (500, 260, 1536), (64, 130, 512)]:
+            W, A = rand_case("q5_k", N, K, 9 * M + N + K, tokens=M)
+            say("q5_k paired kernel", M, N, K)
+            Ad, Wd = P.to_device(A), P.to_device(W)
+            b = P.to_device(T.normal(N, 0.0, 1.0, seed=N))
+            D.ckq_set_prefill_variant(q5, 2)
+            c, sums = P.dev_gemm_block_sums("q5_k", Ad, Wd, b, M, N, K)
+            assert np.array_equal(sums.cpu().numpy().astype(np.int64), np_block_sums("q5_k", W, A, M, N, K)), (M, N, K)
+            L.ckq_set_gemm_policy(1)
+            L.ckq_set_prefill_variant(q5, 2)
+            pair = P.dev_gemm_nt("q5_k", Ad, Wd, b, M, N, K).cpu().numpy()
+            L.ckq_set_prefill_variant(q5, 1)
+            lone = P.dev_gemm_nt("q5_k", Ad, Wd, b, M, N, K).cpu().numpy()
+            L.ckq_set_gemm_policy(0)
+            assert np.array_equal(c.cpu().numpy(), pair), (M, N, K)
+            assert np.array_equal(pair, lone), (M, N, K)
+            assert T.norm_err(pair, T.oracle_gemm_nt("q5_k", A, W, b.cpu().numpy(), M, N, K)) <= TOL
+        M, N, K = 640, 4096, 512
+        xq = P.dev_quantize(P.to_device(T.normal(M * K, 0.0, 1.0, seed=601)), "q8_k", rows=M)
+        W = P.to_device(T.synth_weights("q5_k", N, K, seed=602))
+        say("q5_k kernel by tile count", M, N, K)
+        L.ckq_set_gemm_policy(1)
+        L.ckq_set_prefill_variant(q5, 0)
+        auto = P.dev_gemm_nt("q5_k", xq, W, None, M, N, K).clone()
+        L.ckq_set_prefill_variant(q5, 1)
+        lone = P.dev_gemm_nt("q5_k", xq, W, None, M, N, K).clone()
+        assert torch.equal(auto, lone)
+        Ns = [1536, 2048, 904]
+        Ws = [P.to_device(T.synth_weights("q5_k", n, K, seed=612 + i)) for i, n in enumerate(Ns)]
+        ys = [torch.zeros(M * n, dtype=torch.float32, device="cuda") for n in Ns]
+        L.ckq_set_prefill_variant(q5, 0)
+        say("q5_k grouped launch of the paired kernel", M, Ns, K)
+        P.dev_matmul_sequence([("q5_k", xq, Wj, None, y, M, n, K) for Wj, y, n in zip(Ws, ys, Ns)])
+        torch.cuda.synchronize()
+        L.ckq_set_prefill_variant(q5, 1)
+        for Wj, y, n in zip(Ws, ys, Ns):
+            assert torch.equal(y.view(M, n), P.dev_gemm_nt("q5_k", xq, Wj, None, M, n, K).view(M, n)), n
+    finally:
+        L.ckq_set_gemm_policy(0)
+        L.ckq_set_prefill_variant(q5, 0)
+        D.ckq_set_prefill_variant(q5, 0)
