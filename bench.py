@@ -680,6 +680,16 @@ def main():
                                                     "kernel": "two-plane int8 MFMA on sc*(q-32) split by byte, three LDS stages"}
         del cps6, x6
         torch.cuda.empty_cache()
+        # the gate / up shape in the other two K-quant formats (Q5_K_M and Q6_K models): the paired kernels
+        for fq, kern in (("q5_k", "two-plane int8 MFMA on sc*q5 split by byte, min term as two more int8 MFMAs; two blocks per CU"),
+                         ("q6_k", "two-plane int8 MFMA on sc*(q-32) split by byte; two blocks per CU on 64-token tiles")):
+            _, cpsq = H.weight_copies(fq, rows, K, seed=70, min_total=1)
+            (sq, _, _), _ = H.time_gemm_settled(fq, rows, K, Mg, cpsq[:2], xg, GEMM_LAUNCHES_PER_REP)
+            extras["gemm_%s_q8_k_M512_11008x4096" % fq] = {"tops": round(ops / sq / 1e12, 2), "ms": round(sq * 1e3, 4),
+                                                          "frac_int8_peak": round(ops / sq / 1e12 / INT8_PEAK_TOPS, 4),
+                                                          "ops_per_call": ops, "kernel": kern}
+            del cpsq
+        torch.cuda.empty_cache()
         # and for a Q8_0 model's gate/up projection (small model: K = 896) and a 7B-sized one
         for name8, r8, k8 in (("gemm_q8_0_q8_0_M512_9728x896", 9728, 896), ("gemm_q8_0_q8_0_M512_11008x4096", 11008, 4096)):
             _, cps8 = H.weight_copies("q8_0", r8, k8, seed=88, min_total=1)
