@@ -354,9 +354,10 @@ __global__ void __launch_bounds__(256 * KG, KG == 2 ? 1 : WPE) gemm_q4k_mfma_ker
 
 /* Which token tile a launch takes.  A 96-token tile (ckq_gemm_q4k_t96.hip) costs 1.37 times a 64-token one for 1.5
  * times the tokens, in blocks that run that much longer and leave a 32- or 64-token remainder tile that costs 0.6 / 0.8 of
- * a whole one: it pays when the grid is one round of whole tiles (two blocks per CU) or at least a round and a half deep,
- * and loses when a few long blocks are left over for a second round (512 tokens x 11008 rows: 516 blocks on 512 slots,
- * 67 us against 62).  `tiles64`: tiles of the 64-token kernel, `blocks96`: blocks of the 96-token one. */
+ * a whole one: it pays when every block has a CU to itself, when one round of its blocks replaces a round and a bit of
+ * 64-token tiles, or when the grid is at least a round and a half deep; it loses when a few long blocks are left over for
+ * a second round (512 tokens x 11008 rows: 516 blocks on 512 slots, 67 us against 62) and when CUs that hold two of its
+ * blocks compete with 64-token tiles that all fit one round (960 x 4096: 52.6 against 45.4).  `tiles64`: tiles of the 64-token kernel, `blocks96`: blocks of the 96-token one. */
 static std::atomic<int> g_q4k_tile{0};
 extern "C" void ckq_launch_set_q4k_tile(int tokens) { g_q4k_tile.store(tokens == 64 || tokens == 96 ? tokens : 0); }
 static bool q4k_take_t96(int M, int tiles64, int blocks96)
@@ -365,7 +366,8 @@ static bool q4k_take_t96(int M, int tiles64, int blocks96)
     if (forced) return forced == 96;
     constexpr int SLOTS = 512;                /* 256 CUs, two blocks each */
     if (M < 576 || tiles64 <= 256) return false;
-    if (blocks96 <= SLOTS) return M % 96 == 0;
+    if (blocks96 <= SLOTS / 2) return true;                  /* every block has a CU to itself: 36 us against 40 */
+    if (blocks96 <= SLOTS) return tiles64 > SLOTS;           /* one round, against a second round of 64-token tiles */
     return 2 * blocks96 >= 3 * SLOTS;
 }
 

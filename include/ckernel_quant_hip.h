@@ -431,7 +431,7 @@ void ckq_set_gemm_policy(int policy);
  * the same sums in the same order: results are bit-identical wherever neither launch splits K or puts two wave groups
  * on a tile.
  *   CKQ_FMT_Q4_K: 64 or 96 = tiles of 128 rows x 64 tokens, or x 96 tokens - fewer instructions per token in blocks that run
- *                 longer, taken where the grid is one round of whole tiles or at least a round and a half deep
+ *                 longer, taken where they fit one round that 64-token tiles would not, or the grid is a round and a half deep
  *                 (CKQ_Q4K_TILE=64|96 in the environment);
  *   CKQ_FMT_Q6_K: 1 = one block per CU (64-token tiles three LDS stages deep, 128-token tiles two), 2 = two blocks per CU
  *                 on 64-token tiles with one LDS image of the weights, taken where the 128-token grid would waste a
