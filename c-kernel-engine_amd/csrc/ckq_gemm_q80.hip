@@ -22,7 +22,8 @@
  * - Operands reach LDS by global->LDS loads: the 32 quants of a block as two
  *   16-byte chunks (block starts are only 2-byte aligned in memory; the loads
  *   accept that), the fp16 scales as 2-byte loads, which land zero-extended in
- *   one dword per lane: arrays [block][row] and [block][token].  Quant chunks
+ *   one dword per lane: arrays [row][block] and [token][block] (four adjacent lanes fetch the four scales of one
+ *   136-byte run, so an instruction touches 16 runs instead of 64 rows' worth of cache lines).  Quant chunks
  *   of a row are XOR-swizzled by the row number (rows are 128 bytes apart).
  * - K advances 128 (four blocks) per iteration, two LDS stages of 27 KB, two
  *   blocks per CU (one hides the other's fetch).  The block's waves exchange
@@ -39,8 +40,8 @@ constexpr int GEMM8_BM = 64, GEMM8_BN = 128, GEMM8_KB = 4;   /* tokens, rows, 32
 struct Gemm8Stage {
     uint8_t  wq[GEMM8_BN * GEMM8_KB * 32];   /* row r: 8 chunks of 16 B, chunk c in slot c ^ (r & 7) */
     uint8_t  xq[GEMM8_BM * GEMM8_KB * 32];   /* token t likewise */
-    u32      wd[GEMM8_KB * GEMM8_BN];        /* fp16 scales zero-extended, [block][row] */
-    u32      xd[GEMM8_KB * GEMM8_BM];        /* fp16 scales zero-extended, [block][token] */
+    u32      wd[GEMM8_KB * GEMM8_BN];        /* fp16 scales zero-extended, [row][block] */
+    u32      xd[GEMM8_KB * GEMM8_BM];        /* fp16 scales zero-extended, [token][block] */
 };
 
 template <bool DUMP>
@@ -90,14 +91,14 @@ __global__ void __launch_bounds__(256, 2) gemm_q80_mfma_kernel(GemmArgs a)
     }
 #pragma unroll
     for (int i = 0; i < NWD; ++i) {
-        const int e = (wave + 4 * i) * 64 + lane;            /* [block][row] entry */
-        wd_blk[i] = (u32)(e >> 7);
-        wd_g[i] = (u32)min(e & 127, work.N - 1 - n0) * stride;
+        const int e = (wave + 4 * i) * 64 + lane;            /* [row][block] entry: the four scales of a row come from one 136-byte run */
+        wd_blk[i] = (u32)(e & 3);
+        wd_g[i] = (u32)min(e >> 2, work.N - 1 - n0) * stride;
     }
     {
-        const int e = wave * 64 + lane;                      /* [block][token] entry */
-        xd_blk[0] = (u32)(e >> 6);
-        xd_g[0] = (u32)min(e & 63, a.M - 1 - t0) * stride;
+        const int e = wave * 64 + lane;                      /* [token][block] entry */
+        xd_blk[0] = (u32)(e & 3);
+        xd_g[0] = (u32)min(e >> 2, a.M - 1 - t0) * stride;
     }
 
     /* the copies address their source as buffer (uniform base in SGPRs) + per-lane
@@ -169,11 +170,11 @@ __global__ void __launch_bounds__(256, 2) gemm_q80_mfma_kernel(GemmArgs a)
         u32 dwh[2], dxh[2][2];     /* dwh: the scale of the row of output (lane & 15), one per lane */
         auto read_block = [&](int j) {
             wq[j & 1] = lds16(st.wq + bofs[j]);
-            dwh[j & 1] = st.wd[j * BN + 32 * wave + dw_row];
+            dwh[j & 1] = st.wd[(32 * wave + dw_row) * KB + j];
 #pragma unroll
             for (int ts = 0; ts < 2; ++ts) {
                 xq[j & 1][ts] = lds16(st.xq + aofs[j] + 32 * 128 * ts);
-                dxh[j & 1][ts] = st.xd[j * BM + 32 * ts + col];
+                dxh[j & 1][ts] = st.xd[(32 * ts + col) * KB + j];
             }
         };
         read_block(0);
