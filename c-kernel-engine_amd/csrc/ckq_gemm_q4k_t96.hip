@@ -3,14 +3,16 @@
  * tokens: the arithmetic and the operand paths of ckq_gemm_q4k.hip (two int8 planes per weight, the min
  * term as one bf16 MFMA per 32x32 tile and block, everything through LDS by global->LDS loads), with
  * three 32-token groups per wave instead of two.  The two planes of a wave's 32 rows are expanded once
- * per 256-block and serve 48 int8 MFMAs instead of 32, so a block issues 8.1 VALU instructions per MFMA
- * instead of 9.7, and the weights are read from LDS once per 96 tokens instead of once per 64.
+ * per 256-block and serve 48 int8 MFMAs instead of 32, so the loop issues about 8.5 VALU instructions per
+ * MFMA instead of 9.8 (whole launches, by the counters: 10.3 instead of 11.7), and the weights are read
+ * from LDS once per 96 tokens instead of once per 64.
  *
  * What pays for it: the planes of all eight sub-blocks stay in registers across the three groups (64
  * registers), two sets of int32 accumulators are alive at once (a group's fp32 combine runs under the
- * next group's MFMAs), and LDS holds ONE stage of weights - a wave reads its rows' raw blocks at the
- * start of a 256-block, a barrier follows, and the next block's weights are copied in behind it - beside
- * two stages of activations: 74.5 KB, two blocks per CU.
+ * next group's MFMAs, the last group's under the first MFMAs of the next 256-block), and LDS holds ONE
+ * image of the weights - a wave reads its rows' raw blocks at the start of a 256-block, a barrier follows,
+ * and the next block's weights are copied in behind it - beside two images of the activations and the
+ * tokens' scales and bsums as stored: 74.6 KB, two blocks per CU.
  *
  * A token tile that is not full computes only the groups that hold tokens (1, 2 or 3; uniform per
  * block), and such tiles get the last block ids of their XCD, so that what starts late is short.
