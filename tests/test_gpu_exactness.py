@@ -803,3 +803,33 @@ def test_q5k_paired_kernel_integer_block_sums_bit_exact_and_chosen_by_tile_count
         L.ckq_set_gemm_policy(0)
         L.ckq_set_prefill_variant(q5, 0)
         D.ckq_set_prefill_variant(q5, 0)
+
+
+def test_q4k_96_token_tiles_full_size_equal_64_token_tiles():
+    """The prefill shape at 1 000 tokens (ten whole 96-token tiles and one of 40 tokens per 128 rows, 946
+    blocks, sixteen K-blocks): the 96-token kernel, taken by the default choice here, gives the bits of the
+    64-token kernel for every output, and four tokens - first, last of a whole tile, first and last of the
+    remainder tile - agree with the oracle."""
+    import torch
+    L = ckq.lib()
+    q4 = P.FMT["q4_k"]
+    M, N, K = 1000, 11008, 4096
+    try:
+        xq = P.dev_quantize(P.to_device(T.normal(M * K, 0.0, 1.0, seed=701)), "q8_k", rows=M)
+        W = P.to_device(T.synth_weights("q4_k", N, K, seed=702))
+        b = P.to_device(T.normal(N, 0.0, 1.0, seed=703))
+        say("q4_k 96-token tiles, full size", M, N, K)
+        L.ckq_set_gemm_policy(1)
+        L.ckq_set_prefill_variant(q4, 0)
+        auto = P.dev_gemm_nt("q4_k", xq, W, b, M, N, K).clone()
+        L.ckq_set_prefill_variant(q4, 96)
+        t96 = P.dev_gemm_nt("q4_k", xq, W, b, M, N, K).clone()
+        L.ckq_set_prefill_variant(q4, 64)
+        t64 = P.dev_gemm_nt("q4_k", xq, W, b, M, N, K).clone()
+        assert torch.equal(t96, t64) and torch.equal(auto, t96)
+        rows = [0, 95, 960, 999]
+        ref = T.oracle_gemm_nt("q4_k", xq.view(M, -1)[rows].cpu().numpy().reshape(-1), W.cpu().numpy(), b.cpu().numpy(), len(rows), N, K)
+        assert T.norm_err(t96.view(M, N)[rows].cpu().numpy().reshape(-1), ref.reshape(-1)) <= TOL
+    finally:
+        L.ckq_set_gemm_policy(0)
+        L.ckq_set_prefill_variant(q4, 0)
